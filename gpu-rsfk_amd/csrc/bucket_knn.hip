@@ -1,0 +1,188 @@
+// Bucket K-NN: for every leaf bucket, all-pairs squared distances and the
+// per-point top-K update.  One workgroup (4 wavefronts) per bucket.
+//
+// Replaces the reference's bucket kernels (the function they all compute is
+// the same): compute_knn_from_buckets_predist_nolock ("diagonal",
+// src/kernels/compute_knn_from_buckets.cu:998-1378), ..._pertile (:1382-1787)
+// and ..._perblock_coalesced_symmetric_dividek (:547-814).
+//
+// Schedule here:
+//   * the bucket is cut into 64x64 tiles of the pair matrix; only tiles on or
+//     above the diagonal are computed (every pair once, like the reference's
+//     symmetric kernels);
+//   * the rows of the two 64-point groups are gathered from HBM once per tile,
+//     32 dimensions at a time, into LDS with coalesced 128-byte row segments;
+//   * each thread accumulates a 4x4 block of pair distances in registers
+//     (sequential fused multiply-add per dimension, the arithmetic of
+//     euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
+//   * the tile of distances goes to LDS; then one wavefront per point merges
+//     the tile row (and, for off-diagonal tiles, the tile column) into that
+//     point's K-NN row, which lives in registers with K divided over the lanes.
+//     A row is owned by exactly one wavefront at a time, so no locks are needed.
+#include "rsfk_common.hpp"
+#include "knn_list.hpp"
+
+namespace rsfk {
+
+constexpr int kTile = 64;          // points per tile side
+constexpr int kDC = 32;            // dimensions staged per step
+constexpr int kDCP = kDC + 4;      // LDS row pitch in floats: 9 x 16 B, odd => conflict-free b128 reads
+constexpr int kDistPitch = kTile + 1;
+
+struct BucketKnnLds {
+    float a[kTile * kDCP];
+    float b[kTile * kDCP];
+    float dist[kTile * kDistPitch];
+    int ida[kTile];
+    int idb[kTile];
+};
+
+// Stage rows ids[0..rows) x dims [d0, d0+32) into dst (zero filled outside).
+__device__ __forceinline__ void stage_rows(float* __restrict__ dst, const int* __restrict__ ids, int rows,
+                                           const float* __restrict__ points, int D, int d0, bool vec_ok)
+{
+    const int t = threadIdx.x;
+    const int r = t >> 2;            // 0..63
+    const int seg = (t & 3) * 8;     // 0,8,16,24
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    if (r < rows) {
+        const float* src = points + (size_t)ids[r] * (size_t)D + d0 + seg;
+        const int left = D - d0 - seg;
+        if (vec_ok && left >= 8) {
+            const float4 q0 = *reinterpret_cast<const float4*>(src);
+            const float4 q1 = *reinterpret_cast<const float4*>(src + 4);
+            v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w;
+            v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) if (e < left) v[e] = src[e];
+        }
+    }
+    float4* d4 = reinterpret_cast<float4*>(dst + r * kDCP + seg);
+    d4[0] = make_float4(v[0], v[1], v[2], v[3]);
+    d4[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+template <int SL>
+__global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ points, int D, int K,
+                                                     const int* __restrict__ ids, const int* __restrict__ starts,
+                                                     const int* __restrict__ sizes, int stride,
+                                                     int* __restrict__ knn_idx, float* __restrict__ knn_dist)
+{
+    __shared__ BucketKnnLds L;
+    const int bkt = blockIdx.x;
+    const int s = sizes[bkt];
+    if (s < 2) return;
+    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int ty = tid >> 4, tx = tid & 15;
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+    const int nt = (s + kTile - 1) / kTile;
+
+    for (int I = 0; I < nt; ++I) {
+        const int rows = min(kTile, s - I * kTile);
+        for (int J = I; J < nt; ++J) {
+            const int cols = min(kTile, s - J * kTile);
+            const bool diag = (I == J);
+            __syncthreads();   // previous tile's LDS fully consumed
+            if (tid < kTile) {
+                L.ida[tid] = tid < rows ? bid[I * kTile + tid] : -1;
+                L.idb[tid] = tid < cols ? bid[J * kTile + tid] : -1;
+            }
+            const int nrb = (rows + 15) >> 4, ncb = (cols + 15) >> 4;
+            float acc[4][4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+            __syncthreads();
+            for (int d0 = 0; d0 < D; d0 += kDC) {
+                stage_rows(L.a, L.ida, rows, points, D, d0, vec_ok);
+                if (!diag) stage_rows(L.b, L.idb, cols, points, D, d0, vec_ok);
+                __syncthreads();
+                const float* B = diag ? L.a : L.b;
+#pragma unroll 2
+                for (int dd = 0; dd < kDC; dd += 4) {
+                    float4 av[4], bv[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) av[r] = *reinterpret_cast<const float4*>(&L.a[(ty + 16 * r) * kDCP + dd]);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) bv[c] = *reinterpret_cast<const float4*>(&B[(tx + 16 * c) * kDCP + dd]);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (r >= nrb) continue;
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            if (c >= ncb || (diag && c < r)) continue;
+                            float df;
+                            df = av[r].x - bv[c].x; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                            df = av[r].y - bv[c].y; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                            df = av[r].z - bv[c].z; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                            df = av[r].w - bv[c].w; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+            // distances of the tile -> LDS (mirror the strictly-upper blocks of a diagonal tile)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (r >= nrb || c >= ncb || (diag && c < r)) continue;
+                    const int i = ty + 16 * r, j = tx + 16 * c;
+                    L.dist[i * kDistPitch + j] = acc[r][c];
+                    if (diag && c > r) L.dist[j * kDistPitch + i] = acc[r][c];
+                }
+            __syncthreads();
+            // rows of tile I take the columns of tile J as candidates
+            for (int i = wave; i < rows; i += 4) {
+                const int p = L.ida[i];
+                KnnRow<SL> row;
+                row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+                const bool ok = lane < cols && !(diag && lane == i);
+                const float d = L.dist[i * kDistPitch + lane];
+                row.offer_lanes(ok, L.idb[lane], d);
+                if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+            }
+            if (!diag) {
+                // columns of tile J take the rows of tile I as candidates
+                for (int j = wave; j < cols; j += 4) {
+                    const int p = L.idb[j];
+                    KnnRow<SL> row;
+                    row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+                    const bool ok = lane < rows;
+                    const float d = L.dist[lane * kDistPitch + j];
+                    row.offer_lanes(ok, L.ida[lane], d);
+                    if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+                }
+            }
+        }
+    }
+}
+
+// Host launcher.  All pointers are device pointers.
+int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
+                      const int* sizes, int n_buckets, int stride, int* knn_idx, float* knn_dist,
+                      hipStream_t stream)
+{
+    (void)N;
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
+    RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    dim3 grid((unsigned)n_buckets), block(256);
+    if (K <= 64)
+        hipLaunchKernelGGL(k_bucket_knn<1>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx, knn_dist);
+    else if (K <= 128)
+        hipLaunchKernelGGL(k_bucket_knn<2>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx, knn_dist);
+    else
+        hipLaunchKernelGGL(k_bucket_knn<4>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx, knn_dist);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace rsfk

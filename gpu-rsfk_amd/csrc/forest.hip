@@ -1,0 +1,186 @@
+// Host orchestration: the forest loop (trees -> bucket K-NN), the exploration
+// passes, the per-tree log and the single-tree clustering call.  Replaces
+// RSFK::knn_gpu_rsfk_forest (src/rsfk.cu:2033-2183), RSFK::cluster_by_sample_tree
+// (src/rsfk.cu:2185-2228) and RSFK::update_knn_indice_with_buckets
+// (src/rsfk.cu:1967-2030).
+//
+// Differences in schedule: trees are built in batches (all trees of a batch
+// advance one level per launch), device memory is allocated once per call, and
+// the host synchronises once per tree level of a batch instead of after every
+// kernel.
+#include "forest.hpp"
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+namespace rsfk {
+
+namespace {
+std::mutex g_err_mutex;
+std::string g_last_error;
+}  // namespace
+
+void set_last_error(const std::string& msg)
+{
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    g_last_error = msg;
+}
+const char* last_error()
+{
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    return g_last_error.c_str();
+}
+
+namespace {
+
+double now_s()
+{
+    return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+// how many trees to build per batch: as many as fit in a quarter of the free memory
+int choose_batch(int n_trees, int N, int MIN)
+{
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = (size_t)8 << 30;
+    const size_t budget = free_b / 4;
+    int B = std::min(n_trees, 64);
+    while (B > 1 && tree_ws_bytes(N, MIN, B) > budget) --B;
+    return std::max(B, 1);
+}
+
+struct WsGuard {
+    TreeBatchWorkspace* w = nullptr;
+    ~WsGuard() { tree_ws_free(w); }
+};
+struct DevBuf {
+    void* p = nullptr;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+};
+struct EventPair {
+    hipEvent_t a = nullptr, b = nullptr;
+};
+
+}  // namespace
+
+int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                      int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
+                      hipStream_t stream)
+{
+    RSFK_CHECK(N >= 1 && D >= 1 && K >= 1, "forest: N, D and K must be positive");
+    RSFK_CHECK(n_trees >= 0, "forest: n_trees must not be negative");
+    RSFK_CHECK(K <= 256, "forest: K above 256 is not supported");
+    if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
+    const double t_forest0 = now_s();
+
+    if (n_trees > 0) {
+        const int B = choose_batch(n_trees, N, MIN);
+        WsGuard ws;
+        if (tree_ws_alloc(&ws.w, N, MIN, B)) return 1;
+        std::vector<int> stats((size_t)4 * B);
+        std::vector<EventPair> ev((size_t)B);
+        for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        int rc = 0;
+        for (int t0 = 0; t0 < n_trees && rc == 0; t0 += B) {
+            const int nb = std::min(B, n_trees - t0);
+            const double tb0 = now_s();
+            rc = build_tree_batch(ws.w, d_points, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
+            if (rc) break;
+            const double tb = now_s() - tb0;
+            for (int j = 0; j < nb && rc == 0; ++j) {
+                (void)hipEventRecord(ev[j].a, stream);
+                rc = launch_bucket_knn(d_points, N, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                                       tree_ws_leaf_size(ws.w, j), stats[4 * j], 0, d_idx, d_dist, stream);
+                (void)hipEventRecord(ev[j].b, stream);
+            }
+            if (rc) break;
+            RSFK_HIP(hipStreamSynchronize(stream));
+            for (int j = 0; j < nb; ++j) {
+                float ms = 0.0f;
+                (void)hipEventElapsedTime(&ms, ev[j].a, ev[j].b);
+                const int t = t0 + j;
+                if (log_forest) {
+                    log_forest[(size_t)0 * n_trees + t] = (float)stats[4 * j + 1];   // Tree Depth
+                    log_forest[(size_t)1 * n_trees + t] = (float)stats[4 * j + 2];   // Max Leaf Size
+                    log_forest[(size_t)2 * n_trees + t] = (float)stats[4 * j + 3];   // Min Leaf Size
+                    log_forest[(size_t)3 * n_trees + t] = (float)stats[4 * j + 0];   // Total Leaves
+                    log_forest[(size_t)5 * n_trees + t] = (float)(tb / nb);          // Total Tree Building Time
+                    log_forest[(size_t)15 * n_trees + t] = ms * 1e-3f;               // KNN Sets Updates
+                }
+                if (verbose >= 2)
+                    std::printf("tree %d: depth %d, leaves %d, leaf size %d..%d, K-NN update %.6f s\n", t,
+                                stats[4 * j + 1], stats[4 * j + 0], stats[4 * j + 3], stats[4 * j + 2], ms * 1e-3);
+            }
+        }
+        for (auto& e : ev) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+        if (rc) return rc;
+    }
+    const double t_forest = now_s() - t_forest0;
+    if (verbose >= 1) std::printf("Creating RSFK forest takes %lf seconds\n", t_forest);
+
+    const double t_exp0 = now_s();
+    if (nnef > 0) {
+        DevBuf old;
+        RSFK_HIP(hipMalloc(&old.p, sizeof(int) * (size_t)N * (size_t)K));
+        for (int it = 0; it < nnef; ++it) {
+            if (launch_explore(d_points, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), stream)) return 1;
+        }
+        RSFK_HIP(hipStreamSynchronize(stream));
+    }
+    const double t_exp = now_s() - t_exp0;
+    if (verbose >= 1) std::printf("Nearest Neighbors Exploring computation Kernel takes %lf seconds\n", t_exp);
+    if (log_forest) {
+        log_forest[(size_t)16 * n_trees] = (float)t_forest;
+        log_forest[(size_t)16 * n_trees + 1] = (float)t_exp;
+    }
+    return 0;
+}
+
+int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest)
+{
+    RSFK_CHECK(N >= 1 && D >= 1 && K >= 1, "forest: N, D and K must be positive");
+    DevBuf dp, di, dd;
+    const size_t nd = (size_t)N * (size_t)D, nk = (size_t)N * (size_t)K;
+    RSFK_HIP(hipMalloc(&dp.p, nd * sizeof(float)));
+    RSFK_HIP(hipMalloc(&di.p, nk * sizeof(int)));
+    RSFK_HIP(hipMalloc(&dd.p, nk * sizeof(float)));
+    RSFK_HIP(hipMemcpy(dp.p, points, nd * sizeof(float), hipMemcpyHostToDevice));
+    RSFK_HIP(hipMemcpy(di.p, knn_idx, nk * sizeof(int), hipMemcpyHostToDevice));
+    RSFK_HIP(hipMemcpy(dd.p, knn_dist, nk * sizeof(float), hipMemcpyHostToDevice));
+    const int rc = knn_forest_device(n_trees, K, N, D, MIN, MAX, MAX_DEPTH, verbose, seed, nnef,
+                                     static_cast<const float*>(dp.p), static_cast<int*>(di.p),
+                                     static_cast<float*>(dd.p), log_forest, nullptr);
+    if (rc) return rc;
+    RSFK_HIP(hipMemcpy(knn_idx, di.p, nk * sizeof(int), hipMemcpyDeviceToHost));
+    RSFK_HIP(hipMemcpy(knn_dist, dd.p, nk * sizeof(float), hipMemcpyDeviceToHost));
+    return 0;
+}
+
+// One tree; results on the host.  perm: N ints; leaves sorted by start.
+int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int MAX_DEPTH, int seed,
+                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[4])
+{
+    WsGuard ws;
+    if (tree_ws_alloc(&ws.w, N, MIN, 1)) return 1;
+    if (build_tree_batch(ws.w, d_points, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
+    const int nl = stats[0];
+    perm.resize((size_t)N);
+    std::vector<int> ls((size_t)nl), lz((size_t)nl);
+    RSFK_HIP(hipMemcpy(perm.data(), tree_ws_perm(ws.w, 0), sizeof(int) * (size_t)N, hipMemcpyDeviceToHost));
+    if (nl > 0) {
+        RSFK_HIP(hipMemcpy(ls.data(), tree_ws_leaf_start(ws.w, 0), sizeof(int) * (size_t)nl, hipMemcpyDeviceToHost));
+        RSFK_HIP(hipMemcpy(lz.data(), tree_ws_leaf_size(ws.w, 0), sizeof(int) * (size_t)nl, hipMemcpyDeviceToHost));
+    }
+    std::vector<int> order((size_t)nl);
+    for (int i = 0; i < nl; ++i) order[i] = i;
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return ls[a] < ls[b]; });
+    leaf_start.resize((size_t)nl);
+    leaf_size.resize((size_t)nl);
+    for (int i = 0; i < nl; ++i) { leaf_start[i] = ls[order[i]]; leaf_size[i] = lz[order[i]]; }
+    return 0;
+}
+
+}  // namespace rsfk

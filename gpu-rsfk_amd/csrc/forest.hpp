@@ -1,0 +1,40 @@
+// Internal interfaces between the translation units of the library.
+#pragma once
+#include "rsfk_common.hpp"
+#include <vector>
+
+namespace rsfk {
+
+struct TreeBatchWorkspace;
+
+// tree_build.hip
+size_t tree_ws_bytes(int N, int MIN, int B);
+int tree_ws_alloc(TreeBatchWorkspace** out, int N, int MIN, int B);
+void tree_ws_free(TreeBatchWorkspace* w);
+int tree_ws_leaf_cap(const TreeBatchWorkspace* w);
+const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
+const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
+const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
+int tree_small_threshold();
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, int MIN, int MAX, int MAX_DEPTH,
+                     int seed0, int nb, int* host_stats, hipStream_t stream);
+
+// bucket_knn.hip
+int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
+                      const int* sizes, int n_buckets, int stride, int* knn_idx, float* knn_dist,
+                      hipStream_t stream);
+
+// explore.hip
+int launch_explore(const float* points, int N, int D, int K, int* knn_idx, float* knn_dist, int* old_idx,
+                   hipStream_t stream);
+
+// forest.hip
+int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                      int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
+                      hipStream_t stream);
+int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest);
+int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int MAX_DEPTH, int seed,
+                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[4]);
+
+}  // namespace rsfk

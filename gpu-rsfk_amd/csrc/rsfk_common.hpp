@@ -1,0 +1,104 @@
+// Shared definitions of the gfx950 RSFK library: error handling, the
+// counter-based random numbers of the tree build and the record types that
+// travel between the tree-build kernels, the bucket K-NN kernel and the host.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+
+namespace rsfk {
+
+// ---------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------
+void set_last_error(const std::string& msg);
+const char* last_error();
+
+#define RSFK_HIP(call)                                                                   \
+    do {                                                                                 \
+        hipError_t e_ = (call);                                                          \
+        if (e_ != hipSuccess) {                                                          \
+            ::rsfk::set_last_error(std::string(#call) + ": " + hipGetErrorString(e_) +   \
+                                   " (" __FILE__ ":" + std::to_string(__LINE__) + ")");  \
+            return 1;                                                                    \
+        }                                                                                \
+    } while (0)
+
+#define RSFK_CHECK(cond, msg)                      \
+    do {                                           \
+        if (!(cond)) {                             \
+            ::rsfk::set_last_error(msg);           \
+            return 2;                              \
+        }                                          \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// counter-based random numbers.  A node of a tree is identified by a 64-bit key
+// derived from the tree seed and the left/right path to the node, so a tree is
+// a pure function of (points, MIN, MAX, MAX_DEPTH, seed) whatever the launch
+// geometry.  (The reference seeds cuRAND from the thread index:
+// src/kernels/build_tree_create_nodes.cu:64-68.)
+// ---------------------------------------------------------------------------
+__host__ __device__ inline uint64_t mix64(uint64_t z)
+{
+    z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ULL;
+    z ^= z >> 27; z *= 0x94D049BB133111EBULL;
+    z ^= z >> 31;
+    return z;
+}
+__host__ __device__ inline uint64_t root_key(int seed)
+{
+    return mix64((uint64_t)(int64_t)seed ^ 0x5253464B524F4F54ULL);
+}
+__host__ __device__ inline uint64_t child_key(uint64_t key, int side)
+{
+    return mix64(key + 0x9E3779B97F4A7C15ULL * (uint64_t)(side + 1));
+}
+__host__ __device__ inline uint32_t draw_u32(uint64_t key, uint32_t i)
+{
+    return (uint32_t)(mix64(key ^ (0xD6E8FEB86659FD93ULL * (uint64_t)(i + 1))) >> 32);
+}
+// Two member ranks in [0,count); the second is redrawn while equal to the first
+// (src/kernels/build_tree_create_nodes.cu:96-100), bounded so it always ends.
+__host__ __device__ inline void pick_pair(uint64_t key, int count, int& r1, int& r2)
+{
+    uint32_t c = (uint32_t)count;
+    uint32_t a = draw_u32(key, 0) % c;
+    uint32_t b = draw_u32(key, 1) % c;
+    if (count >= 2) {
+        uint32_t i = 2;
+        while (b == a && i < 66) { b = draw_u32(key, i) % c; ++i; }
+        if (b == a) b = (a + 1) % c;
+    }
+    r1 = (int)a; r2 = (int)b;
+}
+
+// ---------------------------------------------------------------------------
+// records
+// ---------------------------------------------------------------------------
+// A node of a tree under construction.  Its members are perm[buf][tree*N + start
+// .. + count); the point pair that defines its hyperplane is drawn from the
+// sub-range [dstart, dstart+dcount) (the larger side, after a min-size merge).
+struct TreeNode {
+    int tree;
+    int start, count;
+    int dstart, dcount;
+    int depth;        // level of the node, root = 0
+    int buf;          // which of the two permutation buffers holds the members
+    int leaf;         // 1 = already decided to be a bucket
+    uint64_t key;
+};
+
+// bit 31 of a permutation entry marks "right side" during a split; ids use the low 31 bits
+constexpr int kIdMask = 0x7fffffff;
+
+// Parameters of one tree-building batch (B trees built level-synchronously).
+struct TreeParams {
+    int N, D;
+    int MIN, MAX, MAX_DEPTH;
+    int small;        // nodes with at most this many points are finished by one workgroup
+    int chunk;        // points per workgroup in the wide (global) passes
+};
+
+}  // namespace rsfk

@@ -1,0 +1,631 @@
+// Random-sample tree building for a batch of trees, level-synchronous.
+//
+// Replaces the reference's per-level kernel chain of
+// RSFK::create_bucket_from_sample_tree (src/rsfk.cu:500-1207):
+// build_tree_init, build_tree_check_active_points, build_tree_check_points_side,
+// build_tree_count_new_nodes, build_tree_accumulate_child_count,
+// build_tree_organize_sample_candidates, build_tree_create_nodes,
+// build_tree_update_parents, build_tree_post_update_parents, build_tree_utils,
+// build_tree_fix, build_tree_max_leaf_size, build_tree_set_leaves_idx and
+// build_tree_bucket_points (src/kernels/build_tree_*.cu, create_node.cu).
+//
+// Representation: every tree keeps a permutation of 0..N-1 in which each node
+// is a contiguous segment; splitting a node is a stable partition of its
+// segment (left members first).  There are no per-point parent/depth arrays
+// and no per-point atomics.
+//
+//   wide phase : nodes larger than `small` points.  Each level is three
+//                launches over all trees of the batch: (1) hyperplane + side
+//                test + per-chunk left counts, (2) stable scatter with
+//                wave64 ballot / mbcnt ranks, child creation by the chunk-0
+//                workgroup of each node, (3) chunk bookkeeping for the next
+//                level.
+//   tail phase : one workgroup finishes the whole subtree of a node with at
+//                most `small` points inside LDS (all the re-draw levels that
+//                the min/max rule causes touch only such nodes).
+//
+// Arithmetic follows the reference bit for bit: the hyperplane offset and the
+// side test are sums of 32 lane-strided partials combined by the xor butterfly
+// (create_node.cu:122-135, build_tree_check_points_side.cu:131-149); a half
+// wavefront plays the role of the 32-lane warp.
+#include "rsfk_common.hpp"
+#include "wave64.hpp"
+#include <vector>
+#include <algorithm>
+#include <cstring>
+
+namespace rsfk {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kHalves = kBlock / 32;     // half wavefronts per workgroup
+
+struct LevelCounters {
+    int n_next;        // nodes appended for the next wide level
+    int n_tail;        // tail tasks appended so far
+    int n_chunks;      // chunks of the current level (written by the scan kernel)
+    int overflow;      // set when a queue capacity is exceeded
+};
+
+// ---------------------------------------------------------------------------
+// helpers
+// ---------------------------------------------------------------------------
+
+// Hyperplane of (x1,x2): normal into LDS nvec[0..D), offset returned to all
+// threads through *b_out (LDS).  Offset order: create_node.cu:122-135.
+__device__ __forceinline__ void make_hyperplane(const float* __restrict__ x1, const float* __restrict__ x2,
+                                                int D, float* nvec, float* b_out)
+{
+    for (int d = threadIdx.x; d < D; d += blockDim.x) nvec[d] = x1[d] - x2[d];
+    if (threadIdx.x < 32) {
+        float s = 0.0f;
+        for (int d = threadIdx.x; d < D; d += 32) {
+            const float t1 = x1[d], t2 = x2[d];
+            const float nd = t1 - t2;
+            const float prod = nd * (t1 + t2);
+            s = s + prod * 0.5f;
+        }
+        s = half_butterfly_sum(s);
+        if (threadIdx.x == 0) *b_out = s;
+    }
+}
+
+// n.x for one point by one half wavefront (32 lanes); every lane of the half
+// returns the same value.  hl = lane within the half.
+__device__ __forceinline__ float half_dot(const float* nvec, const float* __restrict__ x, int D, int hl, bool valid)
+{
+    float s = 0.0f;
+    if (valid)
+        for (int d = hl; d < D; d += 32) s = __builtin_fmaf(nvec[d], x[d], s);
+    return half_butterfly_sum(s);
+}
+
+// Append a child node either to the next wide level or to the tail queue.
+__device__ __forceinline__ void emit_node(const TreeNode& c, const TreeParams& P, TreeNode* next, int next_cap,
+                                          TreeNode* tail, int tail_cap, LevelCounters* ctr)
+{
+    const bool forced = c.depth >= P.MAX_DEPTH - 1;
+    if (!c.leaf && !forced && c.count > P.small) {
+        const int at = atomicAdd(&ctr->n_next, 1);
+        if (at < next_cap) next[at] = c; else ctr->overflow = 1;
+    } else {
+        TreeNode t = c;
+        if (forced) t.leaf = 1;
+        const int at = atomicAdd(&ctr->n_tail, 1);
+        if (at < tail_cap) tail[at] = t; else ctr->overflow = 1;
+    }
+}
+
+// The split / min-size-merge / leaf rules for a node whose left side has `a`
+// members (src/kernels/build_tree_update_parents.cu:64-75,106-134).  Returns the
+// number of children written to c0, c1.
+__device__ __forceinline__ int split_rules(const TreeNode& nd, int a, int MIN, int MAX, int child_buf,
+                                           TreeNode& c0, TreeNode& c1)
+{
+    const int r = nd.count - a;
+    const uint64_t kl = child_key(nd.key, 0), kr = child_key(nd.key, 1);
+    c0.tree = c1.tree = nd.tree;
+    c0.depth = c1.depth = nd.depth + 1;
+    c0.buf = c1.buf = child_buf;
+    if (a == 0 || r == 0) {
+        c0.start = nd.start; c0.count = nd.count; c0.dstart = nd.start; c0.dcount = nd.count;
+        c0.key = a ? kl : kr; c0.leaf = nd.count <= MAX - 2;
+        return 1;
+    }
+    if (min(a, r) < MIN) {
+        const bool left_big = a >= r;
+        c0.start = nd.start; c0.count = nd.count;
+        c0.dstart = left_big ? nd.start : nd.start + a;
+        c0.dcount = left_big ? a : r;
+        c0.key = left_big ? kl : kr; c0.leaf = nd.count <= MAX;
+        return 1;
+    }
+    c0.start = nd.start; c0.count = a; c0.dstart = nd.start; c0.dcount = a;
+    c0.key = kl; c0.leaf = a <= MAX - 2;
+    c1.start = nd.start + a; c1.count = r; c1.dstart = nd.start + a; c1.dcount = r;
+    c1.key = kr; c1.leaf = r <= MAX - 2;
+    return 2;
+}
+
+// ---------------------------------------------------------------------------
+// wide phase kernels
+// ---------------------------------------------------------------------------
+
+__global__ void k_init_perm(int* __restrict__ perm, int N, int B)
+{
+    const size_t total = (size_t)N * (size_t)B;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+        perm[i] = (int)(i % (size_t)N);
+}
+
+__global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr, TreeParams P, int B, int seed0)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= B) return;
+    TreeNode r;
+    r.tree = t; r.start = 0; r.count = P.N; r.dstart = 0; r.dcount = P.N; r.depth = 0; r.buf = 0; r.leaf = 0;
+    r.key = root_key(seed0 + t);
+    // the root is never a leaf (src/kernels/build_tree_init.cu:79) unless the depth limit forces it
+    emit_node(r, P, nodes, B, tail, B, ctr);
+}
+
+// chunk_base[i] = number of chunks of nodes [0,i); one workgroup.
+__global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict__ nodes, int n_nodes, int chunk,
+                                                      int* __restrict__ chunk_base, LevelCounters* ctr)
+{
+    __shared__ int wsum[16];
+    __shared__ int carry_s;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) carry_s = 0;
+    __syncthreads();
+    for (int base = 0; base < n_nodes; base += 1024) {
+        const int i = base + tid;
+        const int v = i < n_nodes ? (nodes[i].count + chunk - 1) / chunk : 0;
+        // inclusive scan inside the wavefront
+        int x = v;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int y = __shfl_up(x, o, 64);
+            if (lane >= o) x += y;
+        }
+        if (lane == 63) wsum[wave] = x;
+        __syncthreads();
+        int woff = 0;
+        for (int w = 0; w < wave; ++w) woff += wsum[w];
+        const int carry = carry_s;
+        if (i < n_nodes) chunk_base[i] = carry + woff + x - v;
+        __syncthreads();
+        if (tid == 1023) carry_s = carry + woff + x;
+        __syncthreads();
+    }
+    if (tid == 0) { chunk_base[n_nodes] = carry_s; ctr->n_chunks = carry_s; }
+}
+
+__global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, int n_chunks, int* __restrict__ chunk2node)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= n_chunks) return;
+    int lo = 0, hi = n_nodes - 1;          // last node with chunk_base <= c
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (chunk_base[mid] <= c) lo = mid; else hi = mid - 1;
+    }
+    chunk2node[c] = lo;
+}
+
+// Side test of one chunk of one node: sets bit 31 of the permutation entry of
+// every member on the right side and counts the members on the left.
+__global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ points, TreeParams P,
+                                                 int* __restrict__ perm0, int* __restrict__ perm1,
+                                                 const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
+                                                 const int* __restrict__ chunk2node, int* __restrict__ chunk_left)
+{
+    extern __shared__ float nvec[];          // D floats
+    __shared__ float b_s;
+    __shared__ int left_s;
+    const int c = blockIdx.x;
+    const int ni = chunk2node[c];
+    const TreeNode nd = nodes[ni];
+    const int k = c - chunk_base[ni];
+    int* perm = (nd.buf ? perm1 : perm0) + (size_t)nd.tree * (size_t)P.N;
+    int r1, r2;
+    pick_pair(nd.key, nd.dcount, r1, r2);
+    const int p1 = perm[nd.dstart + r1] & kIdMask;
+    const int p2 = perm[nd.dstart + r2] & kIdMask;
+    if (threadIdx.x == 0) left_s = 0;
+    // p1/p2 must be read by every workgroup of the node before any of them sets
+    // side bits; masking with kIdMask makes the read independent of that order.
+    make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
+    __syncthreads();
+    const float b = b_s;
+    const int pos0 = nd.start + k * P.chunk;
+    const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
+    const int half = threadIdx.x >> 5, hl = threadIdx.x & 31;
+    const int iters = (pos1 - pos0 + kHalves - 1) / kHalves;
+    int lefts = 0;
+    for (int it = 0; it < iters; ++it) {
+        const int pos = pos0 + it * kHalves + half;
+        const bool valid = pos < pos1;
+        const int id = valid ? (perm[pos] & kIdMask) : 0;
+        const float dot = half_dot(nvec, points + (size_t)id * P.D, P.D, hl, valid);
+        const bool right = dot < b;               // build_tree_check_points_side.cu:149
+        if (valid && hl == 0) {
+            perm[pos] = right ? (id | (int)0x80000000) : id;
+            lefts += right ? 0 : 1;
+        }
+    }
+    if (hl == 0 && lefts) atomicAdd(&left_s, lefts);
+    __syncthreads();
+    if (threadIdx.x == 0) chunk_left[c] = left_s;
+}
+
+// Stable scatter of one chunk into the other permutation buffer; the workgroup
+// of chunk 0 also applies the split rules and appends the children.
+__global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restrict__ perm0, int* __restrict__ perm1,
+                                                    const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
+                                                    const int* __restrict__ chunk2node, const int* __restrict__ chunk_left,
+                                                    TreeNode* __restrict__ next, int next_cap,
+                                                    TreeNode* __restrict__ tail, int tail_cap, LevelCounters* ctr)
+{
+    __shared__ int red[2][kBlock / 64];
+    __shared__ int wcnt[kBlock / 64];
+    const int c = blockIdx.x;
+    const int ni = chunk2node[c];
+    const TreeNode nd = nodes[ni];
+    const int first = chunk_base[ni];
+    const int nch = chunk_base[ni + 1] - first;
+    const int k = c - first;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // lefts in the chunks before this one, and in the whole node
+    int before = 0, all = 0;
+    for (int j = tid; j < nch; j += kBlock) {
+        const int v = chunk_left[first + j];
+        all += v;
+        if (j < k) before += v;
+    }
+    before = wave_sum_i(before);
+    all = wave_sum_i(all);
+    if (lane == 0) { red[0][wave] = before; red[1][wave] = all; }
+    __syncthreads();
+    before = 0; all = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) { before += red[0][w]; all += red[1][w]; }
+
+    const size_t toff = (size_t)nd.tree * (size_t)P.N;
+    const int* src = (nd.buf ? perm1 : perm0) + toff;
+    int* dst = (nd.buf ? perm0 : perm1) + toff;
+    const int pos0 = nd.start + k * P.chunk;
+    const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
+    int lbase = before;                                   // lefts of the node before the current round
+    for (int r0 = pos0; r0 < pos1; r0 += kBlock) {
+        const int pos = r0 + tid;
+        const bool valid = pos < pos1;
+        const int v = valid ? src[pos] : 0;
+        const bool right = v < 0;
+        const bool isl = valid && !right;
+        const uint64_t m = ballot64(isl);
+        if (lane == 0) wcnt[wave] = __popcll(m);
+        __syncthreads();
+        int woff = 0, tot = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; ++w) { const int x = wcnt[w]; if (w < wave) woff += x; tot += x; }
+        const int lrank = lbase + woff + mask_prefix(m);  // lefts of the node before this position
+        if (valid) {
+            const int dest = right ? nd.start + all + (pos - nd.start) - lrank : nd.start + lrank;
+            dst[dest] = v & kIdMask;
+        }
+        lbase += tot;
+        __syncthreads();
+    }
+    if (k == 0 && tid == 0) {
+        TreeNode c0, c1;
+        const int nc = split_rules(nd, all, P.MIN, P.MAX, nd.buf ^ 1, c0, c1);
+        emit_node(c0, P, next, next_cap, tail, tail_cap, ctr);
+        if (nc == 2) emit_node(c1, P, next, next_cap, tail, tail_cap, ctr);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// tail phase: one workgroup per small node, whole subtree in LDS
+// ---------------------------------------------------------------------------
+struct SmallNode {
+    int start, count, dstart, dcount;     // offsets inside the task's segment
+    int depth, leaf;
+    uint64_t key;
+};
+
+struct TreeStats {          // one per tree of the batch
+    int n_leaves;
+    int levels;
+    int max_leaf;
+    int min_leaf;
+};
+
+__device__ __forceinline__ void emit_leaf(int tree, int gstart, int count, int depth, int leaf_cap,
+                                          int* __restrict__ leaf_start, int* __restrict__ leaf_size,
+                                          TreeStats* stats, LevelCounters* ctr)
+{
+    TreeStats* st = stats + tree;
+    const int at = atomicAdd(&st->n_leaves, 1);
+    if (at < leaf_cap) {
+        leaf_start[(size_t)tree * leaf_cap + at] = gstart;
+        leaf_size[(size_t)tree * leaf_cap + at] = count;
+    } else {
+        ctr->overflow = 1;
+    }
+    atomicMax(&st->levels, depth + 1);
+    atomicMax(&st->max_leaf, count);
+    atomicMin(&st->min_leaf, count);
+}
+
+__global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ points, TreeParams P,
+                                                 const int* __restrict__ perm0, const int* __restrict__ perm1,
+                                                 int* __restrict__ perm_out,
+                                                 const TreeNode* __restrict__ tasks, int n_tasks, int stack_cap,
+                                                 int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
+                                                 TreeStats* stats, LevelCounters* ctr)
+{
+    // dynamic LDS: seg[small] | tmp[small] | nvec[D] | stack[stack_cap]
+    extern __shared__ unsigned char lds_raw[];
+    int* seg = reinterpret_cast<int*>(lds_raw);
+    int* tmp = seg + P.small;
+    float* nvec = reinterpret_cast<float*>(tmp + P.small);
+    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + P.D) * 4 + 15) / 16 * 16);
+    __shared__ float b_s;
+    __shared__ int left_s, top_s;
+    __shared__ int wcnt[kBlock / 64];
+
+    const int task = blockIdx.x;
+    if (task >= n_tasks) return;
+    const TreeNode tk = tasks[task];
+    const size_t toff = (size_t)tk.tree * (size_t)P.N;
+    const int* src = (tk.buf ? perm1 : perm0) + toff;
+    int* dst = perm_out + toff;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    if (tk.leaf) {
+        // already a bucket (any size): move it to the output buffer and record it
+        if (src != dst)
+            for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = src[tk.start + i] & kIdMask;
+        if (tid == 0) emit_leaf(tk.tree, tk.start, tk.count, tk.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
+        return;
+    }
+    for (int i = tid; i < tk.count; i += kBlock) seg[i] = src[tk.start + i] & kIdMask;
+    if (tid == 0) {
+        SmallNode r;
+        r.start = 0; r.count = tk.count; r.dstart = tk.dstart - tk.start; r.dcount = tk.dcount;
+        r.depth = tk.depth; r.leaf = 0; r.key = tk.key;
+        stack[0] = r;
+        top_s = 1;
+    }
+    __syncthreads();
+
+    const int half = tid >> 5, hl = tid & 31;
+    while (true) {
+        const int top = top_s;
+        if (top == 0) break;
+        const SmallNode nd = stack[top - 1];
+        __syncthreads();                      // everyone has read the top before it is overwritten
+        if (nd.leaf || nd.depth >= P.MAX_DEPTH - 1) {
+            if (tid == 0) {
+                emit_leaf(tk.tree, tk.start + nd.start, nd.count, nd.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
+                top_s = top - 1;
+            }
+            __syncthreads();
+            continue;
+        }
+        int r1, r2;
+        pick_pair(nd.key, nd.dcount, r1, r2);
+        const int p1 = seg[nd.dstart + r1], p2 = seg[nd.dstart + r2];
+        if (tid == 0) left_s = 0;
+        make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
+        __syncthreads();
+        const float b = b_s;
+        const int iters = (nd.count + kHalves - 1) / kHalves;
+        int lefts = 0;
+        for (int it = 0; it < iters; ++it) {
+            const int i = it * kHalves + half;
+            const bool valid = i < nd.count;
+            const int id = valid ? seg[nd.start + i] : 0;
+            const float dot = half_dot(nvec, points + (size_t)id * P.D, P.D, hl, valid);
+            const bool right = dot < b;
+            if (valid && hl == 0) {
+                if (right) seg[nd.start + i] = id | (int)0x80000000; else ++lefts;
+            }
+        }
+        if (hl == 0 && lefts) atomicAdd(&left_s, lefts);
+        __syncthreads();
+        const int a = left_s;
+        // stable partition seg[start..start+count) -> tmp -> seg
+        int lbase = 0;
+        for (int r0 = 0; r0 < nd.count; r0 += kBlock) {
+            const int i = r0 + tid;
+            const bool valid = i < nd.count;
+            const int v = valid ? seg[nd.start + i] : 0;
+            const bool right = v < 0;
+            const uint64_t m = ballot64(valid && !right);
+            if (lane == 0) wcnt[wave] = __popcll(m);
+            __syncthreads();
+            int woff = 0, tot = 0;
+#pragma unroll
+            for (int w = 0; w < kBlock / 64; ++w) { const int x = wcnt[w]; if (w < wave) woff += x; tot += x; }
+            const int lrank = lbase + woff + mask_prefix(m);
+            if (valid) tmp[right ? a + i - lrank : lrank] = v & kIdMask;
+            lbase += tot;
+            __syncthreads();
+        }
+        for (int i = tid; i < nd.count; i += kBlock) seg[nd.start + i] = tmp[i];
+        if (tid == 0) {
+            TreeNode full, c0, c1;
+            full.tree = tk.tree; full.start = nd.start; full.count = nd.count; full.dstart = nd.dstart;
+            full.dcount = nd.dcount; full.depth = nd.depth; full.buf = 0; full.leaf = 0; full.key = nd.key;
+            const int nc = split_rules(full, a, P.MIN, P.MAX, 0, c0, c1);
+            int t = top - 1;
+            // right child below the left one: leaves come out left to right
+            if (nc == 2) {
+                if (t < stack_cap) {
+                    SmallNode s1; s1.start = c1.start; s1.count = c1.count; s1.dstart = c1.dstart; s1.dcount = c1.dcount;
+                    s1.depth = c1.depth; s1.leaf = c1.leaf; s1.key = c1.key;
+                    stack[t++] = s1;
+                } else ctr->overflow = 1;
+            }
+            if (t < stack_cap) {
+                SmallNode s0; s0.start = c0.start; s0.count = c0.count; s0.dstart = c0.dstart; s0.dcount = c0.dcount;
+                s0.depth = c0.depth; s0.leaf = c0.leaf; s0.key = c0.key;
+                stack[t++] = s0;
+            } else ctr->overflow = 1;
+            top_s = t;
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = seg[i];
+}
+
+template <typename T>
+int dmalloc(T** p, size_t n)
+{
+    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(T)));
+    return 0;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// host driver
+// ---------------------------------------------------------------------------
+struct TreeBatchWorkspace {
+    int B = 0, N = 0;
+    int leaf_cap = 0, node_cap = 0, tail_cap = 0, chunk_cap = 0;
+    int* perm[2] = {nullptr, nullptr};   // perm[0] is also the output
+    TreeNode* nodes[2] = {nullptr, nullptr};
+    TreeNode* tail = nullptr;
+    int* chunk_base = nullptr;
+    int* chunk2node = nullptr;
+    int* chunk_left = nullptr;
+    int* leaf_start = nullptr;
+    int* leaf_size = nullptr;
+    TreeStats* stats = nullptr;
+    LevelCounters* ctr = nullptr;
+    LevelCounters* h_ctr = nullptr;      // pinned
+    TreeStats* h_stats = nullptr;        // pinned
+};
+
+static void free_ws(TreeBatchWorkspace& w)
+{
+    void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
+                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr};
+    for (void* p : dev) if (p) (void)hipFree(p);
+    if (w.h_ctr) (void)hipHostFree(w.h_ctr);
+    if (w.h_stats) (void)hipHostFree(w.h_stats);
+    w = TreeBatchWorkspace();
+}
+
+void tree_ws_free(TreeBatchWorkspace* w)
+{
+    if (!w) return;
+    free_ws(*w);
+    delete w;
+}
+
+int tree_ws_leaf_cap(const TreeBatchWorkspace* w) { return w->leaf_cap; }
+const int* tree_ws_perm(const TreeBatchWorkspace* w, int t) { return w->perm[0] + (size_t)t * w->N; }
+const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t) { return w->leaf_start + (size_t)t * w->leaf_cap; }
+const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t) { return w->leaf_size + (size_t)t * w->leaf_cap; }
+
+int tree_small_threshold() { return 1024; }
+
+// bytes of device memory a batch of B trees needs
+size_t tree_ws_bytes(int N, int MIN, int B)
+{
+    const size_t lc = (size_t)N / (size_t)std::max(MIN, 1) + 2;
+    return (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24));
+}
+
+int tree_ws_alloc(TreeBatchWorkspace** out, int N, int MIN, int B)
+{
+    TreeBatchWorkspace* w = new TreeBatchWorkspace();
+    *out = w;
+    w->B = B; w->N = N;
+    const int small = tree_small_threshold();
+    w->leaf_cap = N / std::max(MIN, 1) + 2;
+    w->node_cap = B * (N / small + 2);
+    w->tail_cap = B * w->leaf_cap;
+    w->chunk_cap = B * (N / small + 2) * 2 + 16;      // sum ceil(count/chunk) <= N/chunk + nodes
+    if (dmalloc(&w->perm[0], (size_t)B * N)) return 1;
+    if (dmalloc(&w->perm[1], (size_t)B * N)) return 1;
+    if (dmalloc(&w->nodes[0], (size_t)w->node_cap)) return 1;
+    if (dmalloc(&w->nodes[1], (size_t)w->node_cap)) return 1;
+    if (dmalloc(&w->tail, (size_t)w->tail_cap)) return 1;
+    if (dmalloc(&w->chunk_base, (size_t)w->node_cap + 1)) return 1;
+    if (dmalloc(&w->chunk2node, (size_t)w->chunk_cap)) return 1;
+    if (dmalloc(&w->chunk_left, (size_t)w->chunk_cap)) return 1;
+    if (dmalloc(&w->leaf_start, (size_t)B * w->leaf_cap)) return 1;
+    if (dmalloc(&w->leaf_size, (size_t)B * w->leaf_cap)) return 1;
+    if (dmalloc(&w->stats, (size_t)B)) return 1;
+    if (dmalloc(&w->ctr, (size_t)1)) return 1;
+    RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_ctr), sizeof(LevelCounters)));
+    RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stats), sizeof(TreeStats) * (size_t)B));
+    return 0;
+}
+
+// Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  On return perm[0] of
+// tree t holds the point ids grouped by bucket and (leaf_start, leaf_size)[t]
+// the buckets, in no particular order.  host_stats receives 4 ints per tree:
+// number of leaves, number of levels, largest and smallest bucket.
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, int MIN, int MAX, int MAX_DEPTH,
+                     int seed0, int nb, int* host_stats, hipStream_t stream)
+{
+    RSFK_CHECK(nb >= 1 && nb <= w->B && N == w->N, "tree batch: workspace does not match the request");
+    RSFK_CHECK(N >= 1 && D >= 1, "tree batch: N and D must be positive");
+    TreeParams P;
+    P.N = N; P.D = D; P.MIN = MIN; P.MAX = MAX; P.MAX_DEPTH = MAX_DEPTH;
+    P.small = tree_small_threshold();
+    P.chunk = P.small;
+
+    {
+        const size_t total = (size_t)N * nb;
+        const int grid = (int)std::min<size_t>((total + 255) / 256, 65536);
+        hipLaunchKernelGGL(k_init_perm, dim3(grid), dim3(256), 0, stream, w->perm[0], N, nb);
+    }
+    std::vector<TreeStats> init((size_t)nb);
+    for (auto& s : init) { s.n_leaves = 0; s.levels = 0; s.max_leaf = 0; s.min_leaf = 0x7fffffff; }
+    std::memcpy(w->h_stats, init.data(), sizeof(TreeStats) * (size_t)nb);
+    RSFK_HIP(hipMemcpyAsync(w->stats, w->h_stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyHostToDevice, stream));
+    RSFK_HIP(hipMemsetAsync(w->ctr, 0, sizeof(LevelCounters), stream));
+    hipLaunchKernelGGL(k_init_roots, dim3((nb + 63) / 64), dim3(64), 0, stream, w->nodes[0], w->tail, w->ctr, P, nb, seed0);
+    RSFK_HIP(hipGetLastError());
+
+    int cur = 0;
+    const size_t side_lds = (size_t)D * sizeof(float);
+    // wide levels
+    while (true) {
+        RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
+        RSFK_HIP(hipStreamSynchronize(stream));
+        RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
+        const int n_nodes = w->h_ctr->n_next;
+        if (n_nodes == 0) break;
+        RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
+        hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], n_nodes, P.chunk, w->chunk_base, w->ctr);
+        RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
+        RSFK_HIP(hipStreamSynchronize(stream));
+        const int n_chunks = w->h_ctr->n_chunks;
+        RSFK_CHECK(n_chunks <= w->chunk_cap, "tree batch: chunk table overflow");
+        // n_next := 0 for the level being produced
+        RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
+        hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
+        hipLaunchKernelGGL(k_side, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, P, w->perm[0], w->perm[1],
+                           w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
+        hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
+                           w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr);
+        RSFK_HIP(hipGetLastError());
+        cur ^= 1;
+    }
+    // tail
+    const int n_tail = w->h_ctr->n_tail;
+    RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
+    if (n_tail > 0) {
+        const int stack_cap = P.small / std::max(MIN, 1) + 4;
+        const size_t lds = ((size_t)(2 * P.small + D) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
+        RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
+        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, P, w->perm[0], w->perm[1], w->perm[0],
+                           w->tail, n_tail, stack_cap, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr);
+        RSFK_HIP(hipGetLastError());
+    }
+    RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
+    RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
+    RSFK_HIP(hipStreamSynchronize(stream));
+    RSFK_CHECK(!w->h_ctr->overflow, "tree batch: queue overflow in the tail phase");
+    for (int t = 0; t < nb; ++t) {
+        host_stats[4 * t + 0] = w->h_stats[t].n_leaves;
+        host_stats[4 * t + 1] = w->h_stats[t].levels;
+        host_stats[4 * t + 2] = w->h_stats[t].max_leaf;
+        host_stats[4 * t + 3] = w->h_stats[t].n_leaves ? w->h_stats[t].min_leaf : 0;
+        RSFK_CHECK(w->h_stats[t].n_leaves <= w->leaf_cap, "tree batch: leaf table overflow");
+    }
+    return 0;
+}
+
+}  // namespace rsfk

@@ -1,0 +1,113 @@
+"""ctypes declarations of every entry point of ``librsfk.so`` (see
+``include/rsfk.h``), plus thin numpy / raw-pointer helpers for the stage-level
+calls.  Device pointers are passed as plain integers (for example
+``tensor.data_ptr()``); this module does not import torch."""
+import ctypes
+import os
+
+import numpy as np
+
+_LIB_DIR = os.path.dirname(os.path.abspath(__file__))
+_f32 = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_i32 = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+_vp = ctypes.c_void_p
+_ci = ctypes.c_int
+
+# name -> (restype, argtypes); the complete list of exported symbols
+SYMBOLS = {
+    "pymodule_rsfk_knn": (None, [_ci] * 10 + [_vp, _vp, _vp, _vp]),
+    "pymodule_rsfk_knn_ann": (None, [_ci] * 11 + [_vp, _vp, _vp, _vp, _vp]),
+    "pymodule_cluster_by_sample_tree": (None, [_ci] * 7 + [_vp, _vp, _vp, _vp, _vp]),
+    "rsfk_knn_forest_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp]),
+    "rsfk_bucket_knn_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _ci, _ci, _vp, _vp, _vp]),
+    "rsfk_explore_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
+    "rsfk_build_tree_host": (_ci, [_f32, _ci, _ci, _ci, _ci, _ci, _ci, _i32, _i32, _i32, _ci, _i32]),
+    "rsfk_bucket_knn_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _ci, _vp, _i32, _ci, _ci, _i32, _f32]),
+    "rsfk_explore_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _f32, _ci]),
+    "rsfk_last_error": (ctypes.c_char_p, []),
+    "rsfk_device_count": (_ci, []),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises OSError when ``librsfk.so`` has not been built."""
+    global _lib
+    if _lib is None:
+        L = ctypes.CDLL(os.path.join(_LIB_DIR, "librsfk.so"))
+        for name, (res, args) in SYMBOLS.items():
+            f = getattr(L, name)
+            f.restype = res
+            f.argtypes = args
+        _lib = L
+    return _lib
+
+
+class RsfkError(RuntimeError):
+    pass
+
+
+def _check(rc):
+    if rc != 0:
+        raise RsfkError(lib().rsfk_last_error().decode("utf-8", "replace"))
+
+
+def _pts(points):
+    return np.require(points, np.float32, ["C_CONTIGUOUS", "ALIGNED"])
+
+
+def build_tree(points, min_children, max_children, max_depth=5000, seed=0):
+    """One tree on the GPU -> (perm, leaf_start, leaf_size, stats[4])."""
+    points = _pts(points)
+    N, D = points.shape
+    cap = N // max(int(min_children), 1) + 2
+    perm = np.empty(N, np.int32)
+    ls = np.empty(cap, np.int32)
+    lz = np.empty(cap, np.int32)
+    stats = np.zeros(4, np.int32)
+    n = lib().rsfk_build_tree_host(points, N, D, int(min_children), int(max_children), int(max_depth), int(seed),
+                                   perm, ls, lz, cap, stats)
+    if n < 0:
+        raise RsfkError(lib().rsfk_last_error().decode("utf-8", "replace"))
+    return perm, ls[:n].copy(), lz[:n].copy(), stats
+
+
+def bucket_knn(points, K, ids, sizes, knn_idx, knn_dist, starts=None, stride=0):
+    """In-place bucket K-NN update on the GPU (host arrays in and out)."""
+    points = _pts(points)
+    N, D = points.shape
+    ids = np.ascontiguousarray(ids, np.int32)
+    sizes = np.ascontiguousarray(sizes, np.int32)
+    sp = None
+    if starts is not None:
+        starts = np.ascontiguousarray(starts, np.int32)
+        sp = starts.ctypes.data_as(_vp)
+    _check(lib().rsfk_bucket_knn_host(points, N, D, int(K), ids, len(ids), sp, sizes, len(sizes), int(stride),
+                                      knn_idx, knn_dist))
+
+
+def explore(points, K, knn_idx, knn_dist, passes=1):
+    points = _pts(points)
+    N, D = points.shape
+    _check(lib().rsfk_explore_host(points, N, D, int(K), knn_idx, knn_dist, int(passes)))
+
+
+def knn_forest_device(n_trees, K, N, D, min_children, max_children, max_depth, verbose, seed, nnef,
+                      d_points, d_idx, d_dist, log=None, stream=0):
+    """Whole K-NN-graph build on device-resident buffers (integer addresses)."""
+    lp = None if log is None else log.ctypes.data_as(_vp)
+    _check(lib().rsfk_knn_forest_device(int(n_trees), int(K), int(N), int(D), int(min_children), int(max_children),
+                                        int(max_depth), int(verbose), int(seed), int(nnef),
+                                        _vp(d_points), _vp(d_idx), _vp(d_dist), lp, _vp(stream)))
+
+
+def bucket_knn_device(d_points, N, D, K, d_ids, d_starts, d_sizes, n_buckets, stride, d_idx, d_dist, stream=0):
+    _check(lib().rsfk_bucket_knn_device(_vp(d_points), int(N), int(D), int(K), _vp(d_ids),
+                                        _vp(d_starts) if d_starts else None, _vp(d_sizes), int(n_buckets),
+                                        int(stride), _vp(d_idx), _vp(d_dist), _vp(stream)))
+
+
+def explore_device(d_points, N, D, K, d_idx, d_dist, d_scratch, stream=0):
+    _check(lib().rsfk_explore_device(_vp(d_points), int(N), int(D), int(K), _vp(d_idx), _vp(d_dist),
+                                     _vp(d_scratch), _vp(stream)))

@@ -1,0 +1,127 @@
+/*
+ * rsfk.h -- C ABI of librsfk.so, the gfx950 (MI355X) implementation of RSFK
+ * K-NN-graph construction.
+ *
+ * The first three functions are the entry points the gpu_rsfk Python package
+ * binds with ctypes (python/gpu_rsfk/RSFK.py:112-168 of the reference); their
+ * names, argument order and meaning are those of the reference's
+ * src/python/pymodule_ext.cu:44-92.  The remaining functions expose the same
+ * path with device-resident buffers and stage by stage; they return 0 on
+ * success and a non-zero code otherwise (rsfk_last_error() has the text).
+ *
+ * Conventions: points are float32, row-major N x D.  K-NN state is int32 N x K
+ * indices and float32 N x K squared distances, same slot <-> same neighbour,
+ * rows unordered, empty slot = (-1, +inf or FLT_MAX).  The library merges into
+ * whatever the K-NN arrays hold on entry; it never resets them.
+ * All calls use the current HIP device and block until their results are
+ * complete.  K is limited to 256.
+ */
+#ifndef RSFK_H
+#define RSFK_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- entry points of the reference's shared library -------------------- */
+
+/* K-NN graph of `points` with a forest of n_trees random-sample trees followed
+ * by nn_exploring_factor exploration passes.  Host buffers.
+ * Replaces pymodule_rsfk_knn (src/python/pymodule_ext.cu:124-147 ->
+ * RSFK::knn_gpu_rsfk_forest, src/rsfk.cu:2033-2183).  Tree t uses seed
+ * RANDOM_STATE + t (src/rsfk.cu:2087).  log_forest: 16*n_trees+2 floats,
+ * series-major (src/rsfk.cu:2148-2173).  On a device error the message goes to
+ * stderr and the process exits with status 1 (src/rsfk.cu:40-50). */
+void pymodule_rsfk_knn(int n_trees, int num_neighbors, int N, int D,
+                       int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                       int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
+                       float* points, int* knn_indices, float* knn_sqr_distances,
+                       float* log_forest);
+
+/* Query-set variant of the reference (src/python/pymodule_ext.cu:149-181).  Not
+ * implemented: the symbol exists because the Python layer binds it on
+ * construction (python/gpu_rsfk/RSFK.py:134); a call prints a message to stderr
+ * and leaves the outputs untouched. */
+void pymodule_rsfk_knn_ann(int n_trees, int num_neighbors, int N, int NQ, int D,
+                           int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                           int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
+                           float* points, float* query_points,
+                           int* knn_indices, float* knn_sqr_distances, float* log_forest);
+
+/* Partition of the points by one random-sample tree.
+ * Replaces pymodule_cluster_by_sample_tree (src/python/pymodule_ext.cu:183-212 ->
+ * RSFK::cluster_by_sample_tree, src/rsfk.cu:2185-2228).
+ * *nodes_buckets = malloc'ed int[total_leaves*max_child], row b = the ids of
+ * bucket b padded with -1; *bucket_sizes = malloc'ed int[total_leaves].  The
+ * caller owns both (free()).  Buckets are ordered by their position in the
+ * tree (left to right), ids inside a bucket ascend. */
+void pymodule_cluster_by_sample_tree(int N, int D,
+                                     int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                                     int VERBOSE, int RANDOM_STATE,
+                                     float* points,
+                                     int** nodes_buckets, int** bucket_sizes,
+                                     int* total_leaves, int* max_child);
+
+/* ---- the same path, device-resident ------------------------------------ */
+
+/* As pymodule_rsfk_knn but points / knn_indices / knn_sqr_distances are device
+ * pointers (log_forest stays a host pointer, may be NULL) and `stream` is a
+ * hipStream_t (NULL = default stream).  Replaces the body of
+ * RSFK::knn_gpu_rsfk_forest between its host-to-device and device-to-host
+ * copies (src/rsfk.cu:2073-2135). */
+int rsfk_knn_forest_device(int n_trees, int num_neighbors, int N, int D,
+                           int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                           int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
+                           const float* d_points, int* d_knn_indices, float* d_knn_sqr_distances,
+                           float* log_forest, void* stream);
+
+/* Bucket K-NN over a given partition, device pointers.  Bucket b holds
+ * d_ids[start_b .. start_b + d_sizes[b]) with start_b = d_starts ? d_starts[b]
+ * : b*stride (stride = max_child of the padded bucket matrix).  Replaces
+ * RSFK::update_knn_indice_with_buckets and the kernel it launches
+ * (src/rsfk.cu:1967-2030, src/kernels/compute_knn_from_buckets.cu:998-1378). */
+int rsfk_bucket_knn_device(const float* d_points, int N, int D, int num_neighbors,
+                           const int* d_ids, const int* d_starts, const int* d_sizes,
+                           int n_buckets, int stride,
+                           int* d_knn_indices, float* d_knn_sqr_distances, void* stream);
+
+/* One exploration pass, device pointers; d_scratch holds N*K ints (it receives
+ * the snapshot of the indices).  Replaces one iteration of the loop at
+ * src/rsfk.cu:2117-2131 (nearest_neighbors_exploring,
+ * src/kernels/nearest_neighbors_exploring.cu:41-146). */
+int rsfk_explore_device(const float* d_points, int N, int D, int num_neighbors,
+                        int* d_knn_indices, float* d_knn_sqr_distances, int* d_scratch, void* stream);
+
+/* ---- stage-level calls with host buffers (copies in and out) ------------ */
+
+/* One tree (RSFK::create_bucket_from_sample_tree, src/rsfk.cu:500-1207).
+ * perm[N] receives the ids grouped by bucket; leaf_start/leaf_size (capacity
+ * leaf_cap) the buckets in ascending start order; stats[4] = {number of
+ * buckets, number of levels, largest bucket, smallest bucket}.  Returns the
+ * number of buckets or a negative value on error. */
+int rsfk_build_tree_host(const float* points, int N, int D,
+                         int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH, int RANDOM_STATE,
+                         int* perm, int* leaf_start, int* leaf_size, int leaf_cap, int* stats);
+
+/* rsfk_bucket_knn_device with host buffers; n_ids = length of ids. */
+int rsfk_bucket_knn_host(const float* points, int N, int D, int num_neighbors,
+                         const int* ids, int n_ids, const int* starts, const int* sizes,
+                         int n_buckets, int stride,
+                         int* knn_indices, float* knn_sqr_distances);
+
+/* `passes` exploration passes with host buffers. */
+int rsfk_explore_host(const float* points, int N, int D, int num_neighbors,
+                      int* knn_indices, float* knn_sqr_distances, int passes);
+
+/* ---- misc --------------------------------------------------------------- */
+
+/* text of the last error of a call that returned non-zero */
+const char* rsfk_last_error(void);
+
+/* number of HIP devices visible to the library (0 when there is none) */
+int rsfk_device_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RSFK_H */
