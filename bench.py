@@ -1,0 +1,187 @@
+"""Benchmark of the K-NN-graph build on one MI355X.
+
+A step is one complete build (forest of random-sample trees with bucket K-NN,
+then the exploration passes) on inputs that are already resident in HBM, through
+the C-ABI entry point ``rsfk_knn_forest_device``.  Default workload: BASELINE
+config 2, N=1,000,000 x D=100 uniform points, K=32, 50 trees, one exploration
+pass, buckets 33..66.  Prints one JSON line.
+
+The roofline object is for the bucket K-NN kernel: algorithmic bytes per launch
+(one launch = one tree) = N*(4D + 4 + 16K) -- every point row gathered once, every
+id read once, every K-NN row (index + distance) read once and written once --
+divided by the average duration of a launch measured with HIP events recorded on
+the launching stream inside the library (they come back in the per-tree log).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "gpu-rsfk_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def make_points(N, D, workload, seed=0):
+    rng = np.random.default_rng(seed)
+    if workload == "uniform":
+        return rng.random((N, D), dtype=np.float32)
+    if workload == "normal":
+        return rng.standard_normal((N, D), dtype=np.float32)
+    if workload == "gmm64":
+        centres = rng.random((64, D), dtype=np.float32)
+        comp = rng.integers(64, size=N)
+        return (centres[comp] + 0.1 * rng.standard_normal((N, D), dtype=np.float32)).astype(np.float32)
+    if workload == "sparse":
+        X = 1.0 - rng.random((N, D), dtype=np.float32)
+        X[rng.random((N, D), dtype=np.float32) < 0.8] = 0.0
+        return X
+    raise SystemExit("unknown workload %r" % workload)
+
+
+def exact_knn_sample(torch, dX, queries, K, chunk=65536):
+    """Exact K-NN of the query rows against all rows (float64 on the GPU)."""
+    q = dX[queries].double()
+    qn = (q * q).sum(1)
+    nq = q.shape[0]
+    best_d = torch.full((nq, K), float("inf"), dtype=torch.float64, device=dX.device)
+    best_i = torch.full((nq, K), -1, dtype=torch.int64, device=dX.device)
+    for s in range(0, dX.shape[0], chunk):
+        xb = dX[s:s + chunk].double()
+        d2 = qn[:, None] + (xb * xb).sum(1)[None, :] - 2.0 * (q @ xb.T)
+        ids = torch.arange(s, s + xb.shape[0], device=dX.device)[None, :].expand(nq, -1)
+        dd = torch.cat([best_d, d2], 1)
+        ii = torch.cat([best_i, ids], 1)
+        best_d, o = torch.topk(dd, K, dim=1, largest=False)
+        best_i = torch.gather(ii, 1, o)
+    return best_i
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--n", type=int, default=1000000)
+    ap.add_argument("--d", type=int, default=100)
+    ap.add_argument("--k", type=int, default=32)
+    ap.add_argument("--trees", type=int, default=50)
+    ap.add_argument("--explore", type=int, default=1)
+    ap.add_argument("--min-children", type=int, default=-1)
+    ap.add_argument("--max-children", type=int, default=-1)
+    ap.add_argument("--workload", default="uniform", choices=["uniform", "normal", "gmm64", "sparse"])
+    ap.add_argument("--recall-queries", type=int, default=10000)
+    ap.add_argument("--cpu-sample", type=int, default=200000, help="rows of the workload the CPU baseline runs on (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs on one GPU only (--gpus 1); nothing here uses a second GPU")
+
+    import torch
+    from gpu_rsfk import capi
+    from gpu_rsfk.RSFK import ForestLog
+
+    if not torch.cuda.is_available() or capi.lib().rsfk_device_count() < 1:
+        raise SystemExit("bench.py: no GPU visible")
+    N, D, K, T = args.n, args.d, args.k, args.trees
+    mn = K + 1 if args.min_children < 0 else args.min_children
+    mx = 2 * mn if args.max_children < 0 else args.max_children
+    X = make_points(N, D, args.workload)
+    dX = torch.from_numpy(X).cuda()
+    idx = torch.empty((N, K), dtype=torch.int32, device="cuda")
+    dist = torch.empty((N, K), dtype=torch.float32, device="cuda")
+    self_ids = torch.arange(N, dtype=torch.int32, device="cuda")
+
+    def reset_lists():
+        idx.fill_(-1)
+        idx[:, 0] = self_ids
+        dist.fill_(float("inf"))
+        dist[:, 0] = 0.0
+
+    logs = []
+
+    def step(keep):
+        reset_lists()
+        log = np.zeros(16 * T + 2, np.float32)
+        capi.knn_forest_device(T, K, N, D, mn, mx, 5000, 0, 0, args.explore,
+                               dX.data_ptr(), idx.data_ptr(), dist.data_ptr(), log)
+        if keep:
+            logs.append(log)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    sec_per_step = elapsed / max(args.steps, 1)
+
+    # recall against exact K-NN on a seeded sample of query rows
+    nq = min(args.recall_queries, N)
+    queries = torch.from_numpy(np.random.default_rng(1).choice(N, nq, replace=False)).cuda()
+    truth = exact_knn_sample(torch, dX, queries, K)
+    approx = idx[queries].long()
+    hits = (approx[:, :, None] == truth[:, None, :]).any(2).sum().item()
+    recall = hits / float(nq * K)
+
+    # roofline of the bucket K-NN kernel
+    fls = [ForestLog(l) for l in logs]
+    knn_s = float(np.mean([np.mean(f.data["KNN Sets Updates"]) for f in fls])) if fls and T > 0 else 0.0
+    tree_s = float(np.mean([np.mean(f.data["Total Tree Building Time"]) for f in fls])) if fls and T > 0 else 0.0
+    expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
+    alg_bytes = float(N) * (4 * D + 4 + 16 * K)
+    achieved = alg_bytes / knn_s / 1e9 if knn_s > 0 else 0.0
+    roofline = {"kernel": "k_bucket_knn", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4),
+                "launches_per_step": T}
+
+    # CPU baseline: the oracle (a port of the reference algorithm) on a bounded sample
+    cpu = None
+    if args.cpu_sample > 0:
+        from oracle import rsfk_oracle as orc
+        ns = min(args.cpu_sample, N)
+        Xs = np.ascontiguousarray(X[:ns])
+        oi, od = orc.init_lists(ns, K)
+        c0 = time.perf_counter()
+        orc.forest(Xs, K, T, mn, mx, 5000, 0, args.explore, knn_idx=oi, knn_dist=od)
+        cs = time.perf_counter() - c0
+        cpu = {"value": round(ns / cs, 1), "unit": "points/s", "cores": orc.num_threads(), "kind": "port",
+               "seconds": round(cs, 3),
+               "sample": "first %d rows of the same workload, same D, K, %d trees, %d exploration pass(es), OpenMP" % (ns, T, args.explore)}
+
+    out = {
+        "metric": "knng_build_points_per_sec",
+        "value": round(N / sec_per_step, 1),
+        "unit": "points/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "%s N=%d D=%d K=%d n_trees=%d buckets=%d..%d exploration=%d seed=0" % (
+            args.workload, N, D, K, T, mn, mx, args.explore)},
+        "build_seconds": round(sec_per_step, 5),
+        "recall_at_k": round(recall, 4),
+        "recall_queries": nq,
+        "phase_seconds": {"tree_build_per_tree": round(tree_s, 6), "bucket_knn_per_tree": round(knn_s, 6),
+                          "exploration": round(expl_s, 6)},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,306 @@
+"""GPU parity tests: the HIP library, called through its C ABI, against the CPU
+oracle on the same seeded inputs.
+
+Bar: the tree partition (integer work) must be identical; K-NN rows are
+compared as sets and must hold bit-identical distances and identical indices
+except among entries tied at the row's K-th distance (the order in which equal
+candidates arrive is the only freedom the algorithm leaves).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from util import assert_knn_equal, check_partition, exact_knn_numpy, recall, rows_have_no_duplicates, sort_rows
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# ---------------------------------------------------------------------------
+# tree build
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("N,D,MIN,MAX,dist", [
+    (1, 3, 2, 4, "u"), (5, 2, 2, 4, "u"), (40, 1, 3, 8, "u"), (700, 5, 9, 20, "u"),   # tail phase only
+    (1024, 16, 33, 66, "u"), (1025, 16, 33, 66, "u"),                                  # around the wide/tail threshold
+    (5000, 32, 33, 66, "u"), (30000, 100, 33, 66, "u"), (60000, 3, 64, 256, "n"),      # wide phase, several levels
+    (20000, 33, 17, 34, "n"), (8000, 784, 91, 182, "sparse"),
+])
+def test_tree_partition_is_identical(gpu, orc, rng, N, D, MIN, MAX, dist):
+    if dist == "u":
+        X = rng.random((N, D), dtype=np.float32)
+    elif dist == "n":
+        X = rng.standard_normal((N, D)).astype(np.float32)
+    else:
+        X = np.where(rng.random((N, D)) < 0.8, 0.0, 1.0 - rng.random((N, D))).astype(np.float32)
+    for seed in (0, 9):
+        _say("tree", N, D, MIN, MAX, dist, seed)
+        perm, ls, lz, st = orc.build_tree(X, MIN, MAX, 5000, seed)
+        gperm, gls, glz, gst = gpu.build_tree(X, MIN, MAX, 5000, seed)
+        check_partition(gperm, gls, glz, N)
+        assert np.array_equal(gperm, perm)
+        assert np.array_equal(gls, ls) and np.array_equal(glz, lz)
+        assert list(gst) == [len(ls), st[0], st[1], st[2]]
+
+
+def test_tree_edge_cases(gpu, orc, rng):
+    # identical points: re-drawn until the depth limit, then one forced bucket
+    X = np.ones((3000, 4), np.float32)
+    _say("tree identical points")
+    gperm, gls, glz, gst = gpu.build_tree(X, 5, 10, 30, 0)
+    perm, ls, lz, st = orc.build_tree(X, 5, 10, 30, 0)
+    assert list(glz) == [3000] == list(lz) and gst[1] == st[0] == 30
+    # depth limits
+    X = rng.random((5000, 6), dtype=np.float32)
+    for depth in (1, 2, 5, 12):
+        _say("tree depth limit", depth)
+        g = gpu.build_tree(X, 5, 10, depth, 1)
+        o = orc.build_tree(X, 5, 10, depth, 1)
+        assert np.array_equal(g[0], o[0]) and np.array_equal(g[2], o[2]) and g[3][1] == o[3][0] <= depth
+    # duplicated points mixed with distinct ones, N smaller than MIN
+    X = np.repeat(rng.random((300, 3), dtype=np.float32), 7, axis=0)
+    _say("tree duplicates")
+    g = gpu.build_tree(X, 9, 20, 200, 4)
+    o = orc.build_tree(X, 9, 20, 200, 4)
+    assert np.array_equal(g[0], o[0]) and np.array_equal(g[2], o[2])
+    X = rng.random((20, 3), dtype=np.float32)
+    g = gpu.build_tree(X, 33, 66, 5000, 0)
+    assert list(g[2]) == [20]
+
+
+# ---------------------------------------------------------------------------
+# bucket K-NN on a fixed partition
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("N,D,K,MIN,MAX", [
+    (2000, 32, 16, 17, 34), (3000, 100, 32, 33, 66), (3000, 33, 8, 100, 300), (1500, 7, 90, 91, 182),
+    (1200, 1, 4, 5, 10), (2500, 3, 1, 2, 4), (2000, 130, 64, 65, 130), (1500, 20, 65, 66, 140),
+    (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
+])
+def test_bucket_knn_matches_oracle(gpu, orc, rng, N, D, K, MIN, MAX):
+    X = rng.random((N, D), dtype=np.float32)
+    oi, od = orc.init_lists(N, K)
+    gi, gd = orc.init_lists(N, K)
+    for seed in (3, 4):
+        _say("bucket_knn", N, D, K, MIN, MAX, seed)
+        perm, ls, lz, _ = orc.build_tree(X, MIN, MAX, 5000, seed)
+        orc.bucket_knn(X, K, perm, lz, oi, od, starts=ls)
+        gpu.bucket_knn(X, K, perm, lz, gi, gd, starts=ls)
+        assert_knn_equal(gi, gd, oi, od)
+        assert rows_have_no_duplicates(gi)
+
+
+def test_bucket_knn_single_bucket_is_exact_knn(gpu, rng):
+    """One bucket holding every point: the kernel must return exact K-NN."""
+    for N, D, K in [(300, 8, 16), (700, 20, 32)]:
+        _say("bucket_knn all-in-one", N, D, K)
+        X = rng.random((N, D), dtype=np.float32)
+        gi = np.full((N, K), -1, np.int32)
+        gd = np.full((N, K), np.inf, np.float32)
+        gi[:, 0] = np.arange(N)
+        gd[:, 0] = 0
+        gpu.bucket_knn(X, K, np.arange(N, dtype=np.int32), np.array([N], np.int32), gi, gd,
+                       starts=np.array([0], np.int32))
+        ti, td = exact_knn_numpy(X, K)
+        si, sd = sort_rows(gi, gd)
+        assert np.array_equal(np.sort(si, 1), np.sort(ti, 1))
+        assert np.allclose(sd, td, rtol=1e-5, atol=1e-7)          # direct-difference path: 1e-5 relative
+
+
+def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
+    N, D, K = 1500, 10, 8
+    X = rng.random((N, D), dtype=np.float32)
+    perm, ls, lz, _ = orc.build_tree(X, 9, 40, 5000, 2)
+    mc = int(lz.max())
+    # padded matrix with two extra buckets of size 0 and 1 (never produce candidates)
+    nb = len(lz) + 2
+    padded = np.full((nb, mc), -1, np.int32)
+    sizes = np.zeros(nb, np.int32)
+    for b, (s, z) in enumerate(zip(ls, lz)):
+        padded[b, :z] = perm[s:s + z]
+        sizes[b] = z
+    padded[nb - 1, 0] = 5
+    sizes[nb - 1] = 1
+    oi, od = orc.init_lists(N, K)
+    gi, gd = orc.init_lists(N, K)
+    orc.bucket_knn(X, K, padded.ravel(), sizes, oi, od, starts=None, stride=mc)
+    _say("bucket_knn padded")
+    gpu.bucket_knn(X, K, padded.ravel(), sizes, gi, gd, starts=None, stride=mc)
+    assert_knn_equal(gi, gd, oi, od)
+    # FLT_MAX instead of +inf in the empty slots (the reference's CLI initialisation)
+    gi2 = np.full((N, K), -1, np.int32)
+    gd2 = np.full((N, K), np.finfo(np.float32).max, np.float32)
+    oi2, od2 = gi2.copy(), gd2.copy()
+    orc.bucket_knn(X, K, perm, lz, oi2, od2, starts=ls)
+    gpu.bucket_knn(X, K, perm, lz, gi2, gd2, starts=ls)
+    assert_knn_equal(gi2, gd2, oi2, od2)
+    # nothing to do
+    gpu.bucket_knn(X, K, perm, np.zeros(0, np.int32), gi2, gd2, starts=np.zeros(0, np.int32))
+    # bad ids are rejected on the host
+    with pytest.raises(gpu.RsfkError):
+        gpu.bucket_knn(X, K, np.array([0, 1, N], np.int32), np.array([3], np.int32), gi2, gd2,
+                       starts=np.array([0], np.int32))
+
+
+# ---------------------------------------------------------------------------
+# exploration
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("N,D,K,self_in", [(3000, 32, 16, True), (2000, 100, 32, True), (1500, 5, 8, False),
+                                           (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True)])
+def test_explore_matches_oracle(gpu, orc, rng, N, D, K, self_in):
+    X = rng.random((N, D), dtype=np.float32)
+    oi, od = orc.init_lists(N, K, self_in=self_in)
+    MIN = max(2, K // 2)                 # buckets smaller than K+1 leave some rows partly empty
+    for seed in range(2):
+        perm, ls, lz, _ = orc.build_tree(X, MIN, 2 * MIN + 3, 5000, seed)
+        orc.bucket_knn(X, K, perm, lz, oi, od, starts=ls)
+    gi, gd = oi.copy(), od.copy()
+    for _ in range(2):
+        _say("explore", N, D, K, self_in)
+        orc.explore(X, K, oi, od)
+        gpu.explore(X, K, gi, gd, 1)
+        assert_knn_equal(gi, gd, oi, od)
+        assert rows_have_no_duplicates(gi)
+    if not self_in:
+        assert not (gi == np.arange(N)[:, None]).any()
+
+
+# ---------------------------------------------------------------------------
+# the whole call, through the entry points the Python package binds
+# ---------------------------------------------------------------------------
+def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
+    """BASELINE config 1 through RSFK.find_nearest_neighbors."""
+    import gpu_rsfk
+    X = np.random.default_rng(0).random((10000, 32), dtype=np.float32)
+    r = gpu_rsfk.RSFK(random_state=0)
+    _say("forest C1")
+    gi, gd = r.find_nearest_neighbors(X, 16, n_trees=4, min_tree_children=32, max_tree_children=128)
+    oi, od, olog = orc.forest(X, 16, 4, 32, 128, 5000, 0, 1, want_log=True)
+    assert_knn_equal(gi, gd, oi, od)
+    ti, _ = orc.bruteforce(X, 16)
+    assert abs(recall(ti, gi) - recall(ti, oi)) < 1e-9 and recall(ti, gi) > 0.35
+    log = r.log_forest.data
+    assert log["Tree Depth"] == [int(v) for v in olog[0:4]]
+    assert log["Max Leaf Size"] == [int(v) for v in olog[4:8]]
+    assert log["Min Leaf Size"] == [int(v) for v in olog[8:12]]
+    assert log["Total Leaves"] == [int(v) for v in olog[12:16]]
+    assert all(t > 0 for t in log["KNN Sets Updates"]) and r._last_search_time > 0
+    assert (gi >= 0).all()
+
+
+@pytest.mark.parametrize("N,D,K,T,kw", [
+    (20000, 100, 32, 6, {}),
+    (5000, 16, 8, 3, dict(min_tree_children=4, max_tree_children=9)),          # second call with K+1 .. 3(K+1)
+    (6000, 24, 40, 3, dict(nn_exploring_factor=2)),
+    (4000, 12, 10, 2, dict(point_in_self_neigh=False, nn_exploring_factor=0)),
+])
+def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, N, D, K, T, kw):
+    import gpu_rsfk
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    r = gpu_rsfk.RSFK(random_state=17)
+    _say("forest", N, D, K, T, kw)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=T, **kw)
+    mn = kw.get("min_tree_children", K + 1)
+    mx = kw.get("max_tree_children", 2 * mn)
+    nnef = kw.get("nn_exploring_factor", 1 if K <= 32 else 0)
+    oi, od = orc.init_lists(N, K, self_in=kw.get("point_in_self_neigh", True))
+    orc.forest(X, K, T, mn, mx, 5000, 17, nnef, knn_idx=oi, knn_dist=od)
+    if mn < K + 1:
+        orc.forest(X, K, 1, K + 1, 3 * (K + 1), 5000, 17, nnef, knn_idx=oi, knn_dist=od)
+    assert_knn_equal(gi, gd, oi, od)
+
+
+def test_reference_package_smoke_tests(gpu):
+    """The two live smoke tests of the reference package (RSFK.py:841-903)."""
+    import gpu_rsfk
+    np.random.seed(0)
+    _say("package test()")
+    gpu_rsfk.test()
+
+
+def test_cluster_by_sample_tree(gpu, orc, rng):
+    import gpu_rsfk
+    N, D = 4096, 99
+    X = rng.random((N, D), dtype=np.float32)
+    r = gpu_rsfk.RSFK(random_state=5)
+    _say("cluster_by_sample_tree")
+    total_leaves, max_child, nodes_buckets, bucket_sizes = r.cluster_by_sample_tree(
+        X, min_tree_children=N // 30, max_tree_children=3 * (N // 30), verbose=0)
+    perm, ls, lz, st = orc.build_tree(X, N // 30, 3 * (N // 30), 5000, 5)
+    assert total_leaves == len(lz) and max_child == lz.max()
+    assert nodes_buckets.shape == (total_leaves * max_child,) and np.array_equal(bucket_sizes, lz)
+    nb = nodes_buckets.reshape(total_leaves, max_child)
+    for b in range(total_leaves):
+        assert np.array_equal(nb[b, :lz[b]], perm[ls[b]:ls[b] + lz[b]])
+        assert (nb[b, lz[b]:] == -1).all()
+    assert np.array_equal(np.sort(nb[nb >= 0]), np.arange(N))
+    raw = r.cluster_by_sample_tree(X, min_tree_children=64, max_tree_children=256, verbose=0, numpy_result_format=False)
+    assert raw[0].value > 0 and raw[1].value <= 256
+
+
+def test_golden_vectors(gpu):
+    g = np.load(os.path.join(ROOT, "tests", "golden", "small_knng.npz"))
+    N, D, K, MIN, MAX, seed = [int(v) for v in g["params"]]
+    X = g["X"]
+    _say("golden")
+    perm, ls, lz, st = gpu.build_tree(X, MIN, MAX, 5000, seed)
+    assert np.array_equal(perm, g["perm"]) and np.array_equal(ls, g["leaf_start"]) and np.array_equal(lz, g["leaf_size"])
+    gi = np.full((N, K), -1, np.int32)
+    gd = np.full((N, K), np.inf, np.float32)
+    gi[:, 0] = np.arange(N)
+    gd[:, 0] = 0
+    gpu.bucket_knn(X, K, perm, lz, gi, gd, starts=ls)
+    assert_knn_equal(gi, gd, g["bucket_idx"], g["bucket_dist"])
+    import gpu_rsfk
+    fi, fd = gpu_rsfk.RSFK(seed).find_nearest_neighbors(X, K, n_trees=3, min_tree_children=MIN, max_tree_children=MAX)
+    assert_knn_equal(fi, fd, g["forest_idx"], g["forest_dist"])
+
+
+# ---------------------------------------------------------------------------
+# size-independent properties at a size the oracle is not run on
+# ---------------------------------------------------------------------------
+def test_properties_at_scale(gpu, orc):
+    import torch
+    N, D, K, T = 300000, 100, 32, 8
+    rng = np.random.default_rng(0)
+    X = rng.random((N, D), dtype=np.float32)
+    dX = torch.from_numpy(X).cuda()
+    idx = torch.full((N, K), -1, dtype=torch.int32, device="cuda")
+    idx[:, 0] = torch.arange(N, dtype=torch.int32, device="cuda")
+    dist = torch.full((N, K), float("inf"), dtype=torch.float32, device="cuda")
+    dist[:, 0] = 0
+    log = np.zeros(16 * T + 2, np.float32)
+    _say("scale forest")
+    gpu.knn_forest_device(T, K, N, D, K + 1, 2 * (K + 1), 5000, 0, 0, 0, dX.data_ptr(), idx.data_ptr(), dist.data_ptr(), log)
+    torch.cuda.synchronize()
+    gi, gd = idx.cpu().numpy(), dist.cpu().numpy()
+    assert (gi >= 0).all() and (gi < N).all()
+    assert rows_have_no_duplicates(gi)
+    leaves = log[3 * T:4 * T]
+    assert (log[1 * T:2 * T] <= 2 * (K + 1)).all() and (log[2 * T:3 * T] >= K + 1).all()
+    assert (leaves >= N / (2 * (K + 1))).all() and (leaves <= N / (K + 1)).all()
+    # stored distances are the distances of the stored neighbours
+    rows = rng.choice(N, 300, replace=False)
+    for p in rows:
+        for k in range(0, K, 5):
+            assert gd[p, k] == orc.sqdist(X[p], X[gi[p, k]])
+    # one more identical forest cannot change anything (idempotence of the set update)
+    before = gd.max(1).copy()
+    _say("scale forest again")
+    gpu.knn_forest_device(T, K, N, D, K + 1, 2 * (K + 1), 5000, 0, 0, 0, dX.data_ptr(), idx.data_ptr(), dist.data_ptr(), log)
+    torch.cuda.synchronize()
+    gi2, gd2 = idx.cpu().numpy(), dist.cpu().numpy()
+    si, sd = sort_rows(gi, gd)
+    si2, sd2 = sort_rows(gi2, gd2)
+    assert np.array_equal(sd, sd2) and np.array_equal(si, si2)
+    # exploration only lowers the row maximum, and the oracle agrees on a sample of rows
+    scratch = torch.empty((N, K), dtype=torch.int32, device="cuda")
+    _say("scale explore")
+    gpu.explore_device(dX.data_ptr(), N, D, K, idx.data_ptr(), dist.data_ptr(), scratch.data_ptr())
+    torch.cuda.synchronize()
+    gd3 = dist.cpu().numpy()
+    assert (gd3.max(1) <= before).all()
+    assert rows_have_no_duplicates(idx.cpu().numpy())
