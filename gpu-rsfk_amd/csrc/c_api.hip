@@ -5,6 +5,7 @@
 #include <cstring>
 #include <chrono>
 #include <vector>
+#include <algorithm>
 
 using namespace rsfk;
 
@@ -105,7 +106,7 @@ RSFK_API int rsfk_bucket_knn_device(const float* d_points, int N, int D, int num
                                     int* d_knn_indices, float* d_knn_sqr_distances, void* stream)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (launch_bucket_knn(d_points, N, D, num_neighbors, d_ids, d_starts, d_sizes, n_buckets, stride,
+    if (launch_bucket_knn(d_points, N, D, num_neighbors, d_ids, d_starts, d_sizes, n_buckets, stride, -1,
                           d_knn_indices, d_knn_sqr_distances, s))
         return 1;
     RSFK_HIP(hipStreamSynchronize(s));
@@ -151,7 +152,9 @@ RSFK_API int rsfk_bucket_knn_host(const float* points, int N, int D, int num_nei
 {
     RSFK_CHECK(N >= 1 && D >= 1 && num_neighbors >= 1 && n_buckets >= 0 && n_ids >= 0, "bad sizes");
     // host-side validation: every bucket must lie inside ids[] and every id inside [0,N)
+    int max_bucket = 0;
     for (int b = 0; b < n_buckets; ++b) {
+        max_bucket = std::max(max_bucket, sizes[b]);
         const long long st = starts ? (long long)starts[b] : (long long)b * stride;
         RSFK_CHECK(sizes[b] >= 0 && st >= 0 && st + sizes[b] <= n_ids, "bucket outside the id array");
         for (int i = 0; i < sizes[b]; ++i)
@@ -171,7 +174,7 @@ RSFK_API int rsfk_bucket_knn_host(const float* points, int N, int D, int num_nei
     RSFK_HIP(hipMemcpy(dkd.p, knn_sqr_distances, sizeof(float) * nk, hipMemcpyHostToDevice));
     if (launch_bucket_knn(static_cast<const float*>(dp.p), N, D, num_neighbors, static_cast<const int*>(di.p),
                           starts ? static_cast<const int*>(dst.p) : nullptr, static_cast<const int*>(dsz.p),
-                          n_buckets, stride, static_cast<int*>(dki.p), static_cast<float*>(dkd.p), nullptr))
+                          n_buckets, stride, max_bucket, static_cast<int*>(dki.p), static_cast<float*>(dkd.p), nullptr))
         return 1;
     RSFK_HIP(hipDeviceSynchronize());
     RSFK_HIP(hipMemcpy(knn_indices, dki.p, sizeof(int) * nk, hipMemcpyDeviceToHost));

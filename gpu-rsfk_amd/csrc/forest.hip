@@ -92,7 +92,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             for (int j = 0; j < nb && rc == 0; ++j) {
                 (void)hipEventRecord(ev[j].a, stream);
                 rc = launch_bucket_knn(d_points, N, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
-                                       tree_ws_leaf_size(ws.w, j), stats[4 * j], 0, d_idx, d_dist, stream);
+                                       tree_ws_leaf_size(ws.w, j), stats[4 * j], 0, stats[4 * j + 2], d_idx, d_dist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
             }
             if (rc) break;

@@ -21,7 +21,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, i
 
 // bucket_knn.hip
 int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
-                      const int* sizes, int n_buckets, int stride, int* knn_idx, float* knn_dist,
+                      const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream);
 
 // explore.hip
