@@ -1,0 +1,307 @@
+// Bucket K-NN for buckets of at most 64 points and K <= 64: the shape the
+// default parameters (bucket size K+1 .. 2(K+1), K <= 32) produce.  Same function
+// as the general kernel in bucket_knn.hip (see there for the reference kernels it
+// replaces); two wavefronts per bucket.
+//
+//   1. the rows of the bucket, 64 dimensions at a time, are requested from HBM at
+//      once and written to LDS; a row is read by consecutive lanes, 16 bytes each
+//      (coalesced);
+//   2. each thread owns one 4x4 block of the upper triangle of the pair matrix and
+//      accumulates its 16 distances with sequential fused multiply-add chains
+//      (arithmetic of euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
+//      the 6 pairs inside each diagonal block are done one per thread;
+//   3. "already in the row" is answered for all rows at once with a hash table of
+//      the bucket's ids in LDS (two probes, branch-free in the common case) and
+//      kept as a 64-bit mask per point;
+//   4. the distance matrix replaces the rows in LDS; a wavefront owns every second
+//      point: per point, the candidates that are closer than the row's last slot
+//      and not in the mask are inserted into the sorted row (knn_list.hpp); the
+//      rows of the next two points are in flight meanwhile.
+// Registers are kept near 100 and LDS near 20 KB per workgroup so that four
+// wavefronts per SIMD are resident: the kernel alternates between an arithmetic
+// phase and a latency-bound merge phase, and only other resident workgroups can
+// fill the gaps.
+#include "rsfk_common.hpp"
+#include "knn_list.hpp"
+#include "forest.hpp"
+
+namespace rsfk {
+
+namespace {
+
+constexpr int kCap = 64;                    // largest bucket this kernel takes
+constexpr int kThreads = 128;
+constexpr int kWaves = kThreads / 64;
+constexpr int kRowsPerWave = kCap / kWaves;
+constexpr int kHash = 256;                  // open-addressing table of the bucket's ids
+constexpr int kSpacing = 17;                // LDS rows between members 4t, 4t+1, 4t+2, 4t+3
+constexpr int kLdsRows = 15 + 3 * kSpacing + 1;
+constexpr int kDistPitch = kCap + 1;
+constexpr int kMaxChunk = 64;               // dimensions staged at once
+constexpr int kMaxLoads = kCap * (kMaxChunk / 4) / kThreads;   // 16-byte loads per thread and chunk
+
+__device__ __forceinline__ uint32_t bucket_hash(int id)
+{
+    uint32_t h = (uint32_t)id * 0x9E3779B1u;
+    return (h ^ (h >> 15)) & (kHash - 1);
+}
+
+// LDS row of bucket member m: the 4x4 block of thread t reads rows t, t+17, t+34,
+// t+51 -- consecutive t give conflict-free 16-byte reads (the pitch is an odd
+// number of 16-byte units) and the four rows of one block fall in different banks.
+__device__ __forceinline__ int phys_row(int m) { return (m >> 2) + kSpacing * (m & 3); }
+
+__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* __restrict__ points, int D, int K,
+                                                                  const int* __restrict__ ids,
+                                                                  const int* __restrict__ starts,
+                                                                  const int* __restrict__ sizes, int stride,
+                                                                  int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                                  int chunk, int pitch, int region_floats)
+{
+    // dynamic LDS: [rows | dist] (region_floats) | ids[64] | table[256] | present[64][2]
+    extern __shared__ __align__(16) float lds_f[];
+    float* rows = lds_f;
+    float* dist = lds_f;                     // same storage, used after the last read of rows
+    int* lids = reinterpret_cast<int*>(lds_f + region_floats);
+    int* table = lids + kCap;
+    uint32_t* present = reinterpret_cast<uint32_t*>(table + kHash);
+
+    const int bkt = blockIdx.x;
+    const int s = sizes[bkt];
+    if (s < 2 || s > kCap) return;
+    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+
+    table[tid] = -1;
+    table[tid + kThreads] = -1;
+    present[tid] = 0;
+    if (tid < kCap) lids[tid] = tid < s ? bid[tid] : -1;
+    __syncthreads();
+
+    // hash table of the bucket
+    if (tid < s) {
+        uint32_t h = bucket_hash(lids[tid]);
+        for (int probe = 0; probe < kHash; ++probe) {
+            if (atomicCAS(&table[h], -1, tid) == -1) break;
+            h = (h + 1) & (kHash - 1);
+        }
+    }
+
+    // work assignment: off-diagonal 4x4 blocks (ti < tj) one per thread, then the 6 pairs of each diagonal block
+    const int n = (s + 3) >> 2;
+    const int noff = n * (n - 1) / 2;
+    int ti = 0, tj = 0;
+    const bool has_tile = tid < noff;
+    if (has_tile) {
+        int rem = tid;
+        while (rem >= n - 1 - ti) { rem -= n - 1 - ti; ++ti; }
+        tj = ti + 1 + rem;
+    }
+    const bool has_diag = tid < 6 * n;
+    const int dt = tid / 6, dq = tid - 6 * dt;
+    const int dr = dq < 3 ? 0 : (dq < 5 ? 1 : 2);
+    const int dc = dq < 3 ? dq + 1 : (dq < 5 ? dq - 1 : 3);
+
+    float acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+    float dacc = 0.0f;
+
+    for (int d0 = 0; d0 < D; d0 += chunk) {
+        const int np = min(chunk, (D - d0 + 3) & ~3) >> 2;      // 16-byte pieces per row in this chunk
+        const int items = s * np;
+        // request everything, then move it to LDS
+        float4 pre[kMaxLoads];
+#pragma unroll
+        for (int i = 0; i < kMaxLoads; ++i) {
+            const int it = tid + i * kThreads;
+            pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (it < items) {
+                const int m = it / np, pc = it - m * np;
+                const float* src = points + (size_t)lids[m] * (size_t)D + d0 + 4 * pc;
+                if (vec_ok) {
+                    pre[i] = *reinterpret_cast<const float4*>(src);
+                } else {
+                    const int left = D - d0 - 4 * pc;
+                    pre[i].x = src[0];
+                    if (left > 1) pre[i].y = src[1];
+                    if (left > 2) pre[i].z = src[2];
+                    if (left > 3) pre[i].w = src[3];
+                }
+            }
+        }
+        if (d0 > 0) __syncthreads();                 // the previous chunk has been consumed
+#pragma unroll
+        for (int i = 0; i < kMaxLoads; ++i) {
+            const int it = tid + i * kThreads;
+            if (it < items) {
+                const int m = it / np, pc = it - m * np;
+                *reinterpret_cast<float4*>(&rows[phys_row(m) * pitch + 4 * pc]) = pre[i];
+            }
+        }
+        __syncthreads();
+        if (has_tile) {
+            const float* ra = &rows[ti * pitch];
+            const float* rb = &rows[tj * pitch];
+            for (int q = 0; q < np; ++q) {
+                float4 av[4], bv[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) av[r] = *reinterpret_cast<const float4*>(ra + kSpacing * r * pitch + 4 * q);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) bv[c] = *reinterpret_cast<const float4*>(rb + kSpacing * c * pitch + 4 * q);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float df;
+                        df = av[r].x - bv[c].x; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                        df = av[r].y - bv[c].y; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                        df = av[r].z - bv[c].z; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                        df = av[r].w - bv[c].w; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                    }
+            }
+        }
+        if (has_diag) {
+            const float* ra = &rows[(dt + kSpacing * dr) * pitch];
+            const float* rb = &rows[(dt + kSpacing * dc) * pitch];
+            for (int q = 0; q < np; ++q) {
+                const float4 a = *reinterpret_cast<const float4*>(ra + 4 * q);
+                const float4 b = *reinterpret_cast<const float4*>(rb + 4 * q);
+                float df;
+                df = a.x - b.x; dacc = __builtin_fmaf(df, df, dacc);
+                df = a.y - b.y; dacc = __builtin_fmaf(df, df, dacc);
+                df = a.z - b.z; dacc = __builtin_fmaf(df, df, dacc);
+                df = a.w - b.w; dacc = __builtin_fmaf(df, df, dacc);
+            }
+        }
+    }
+    __syncthreads();                           // rows no longer needed: the region becomes the distance matrix
+    if (has_tile) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int i = 4 * ti + r, j = 4 * tj + c;
+                if (i < s && j < s) {
+                    dist[i * kDistPitch + j] = acc[r][c];
+                    dist[j * kDistPitch + i] = acc[r][c];
+                }
+            }
+    }
+    if (has_diag) {
+        const int i = 4 * dt + dr, j = 4 * dt + dc;
+        if (j < s) {
+            dist[i * kDistPitch + j] = dacc;
+            dist[j * kDistPitch + i] = dacc;
+        }
+    }
+
+    // Which members of the bucket does each row already hold?  All lookups of the wavefront
+    // are independent: two probes each without branching, a loop only for the rare longer run.
+    // present[i] is touched by the owning wavefront only.
+    bool unsorted = false;
+#pragma unroll
+    for (int u = 0; u < kRowsPerWave; ++u) {
+        const int i = wave + kWaves * u;
+        int mine = -2;
+        float mined = INFINITY;
+        if (i < s && lane < K) {
+            const size_t at = (size_t)lids[i] * (size_t)K + lane;
+            mine = knn_idx[at];
+            mined = knn_dist[at];
+        }
+        const bool want = i < s && mine >= 0;
+        const uint32_t h = bucket_hash(mine);
+        const int e0 = table[h], e1 = table[(h + 1) & (kHash - 1)];
+        const int id0 = lids[e0 < 0 ? 0 : e0], id1 = lids[e1 < 0 ? 0 : e1];
+        int hit = -1;
+        if (want && e0 >= 0) {
+            if (id0 == mine) hit = e0;
+            else if (e1 >= 0) {
+                if (id1 == mine) hit = e1;
+                else {
+                    uint32_t hh = (h + 2) & (kHash - 1);
+                    for (int probe = 2; probe < kHash; ++probe) {
+                        const int e = table[hh];
+                        if (e < 0) break;
+                        if (lids[e] == mine) { hit = e; break; }
+                        hh = (hh + 1) & (kHash - 1);
+                    }
+                }
+            }
+        }
+        if (hit >= 0) atomicOr(&present[2 * i + (hit >> 5)], 1u << (hit & 31));
+        // rows must be sorted by distance; anything else is rebuilt below
+        unsorted |= mined < wave_shr1_f(mined);
+    }
+    const bool any_unsorted = ballot64(unsorted) != 0;
+    __syncthreads();                           // distance matrix and present[] complete
+
+    // top-K update, one member at a time per wavefront; the LDS reads of the next member are
+    // issued before the current one is merged
+    const int my_id = lids[lane];
+    float d_next = dist[wave * kDistPitch + lane];
+    uint32_t f_next = present[2 * wave + (lane >> 5)];
+    auto load_row = [&](int i, int& ri, float& rd) {
+        ri = -2;
+        rd = INFINITY;
+        if (i < s && lane < K) {
+            const size_t at = (size_t)lids[i] * (size_t)K + lane;
+            ri = knn_idx[at];
+            rd = knn_dist[at];
+        }
+    };
+    int ri0, ri1, ri2;
+    float rd0, rd1, rd2;
+    load_row(wave, ri0, rd0);
+    load_row(wave + kWaves, ri1, rd1);
+    for (int i = wave; i < s; i += kWaves) {
+        load_row(i + 2 * kWaves, ri2, rd2);
+        const float d = d_next;
+        const bool held = (f_next >> (lane & 31)) & 1u;
+        if (i + kWaves < s) {
+            d_next = dist[(i + kWaves) * kDistPitch + lane];
+            f_next = present[2 * (i + kWaves) + (lane >> 5)];
+        }
+        KnnRow<1> row;
+        row.idx[0] = ri0;
+        row.dist[0] = rd0;
+        ri0 = ri1; rd0 = rd1; ri1 = ri2; rd1 = rd2;
+        if (any_unsorted) row.init_from_regs(K); else row.init_sorted(K);
+        const bool ok = lane < s && lane != i && !held;
+        row.offer_lanes<false>(ok, my_id, d);
+        if (row.changed) {
+            const size_t at = (size_t)lids[i] * (size_t)K;
+            row.store(knn_idx + at, knn_dist + at);
+        }
+    }
+}
+
+}  // namespace
+
+int small_bucket_cap() { return kCap; }
+
+int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                            int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream)
+{
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
+    const int dpad = (D + 3) & ~3;
+    const int chunk = dpad < kMaxChunk ? dpad : kMaxChunk;
+    int pitch = chunk;
+    if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units
+    const int region = std::max(kLdsRows * pitch, kCap * kDistPitch);
+    const int region_floats = (region + 3) & ~3;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(kCap + kHash + 2 * kCap) * 4;
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_small),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k_bucket_knn_small, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, D, K, ids,
+                       starts, sizes, stride, knn_idx, knn_dist, chunk, pitch, region_floats);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace rsfk

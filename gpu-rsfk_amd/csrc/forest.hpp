@@ -24,6 +24,11 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream);
 
+// bucket_knn_small.hip
+int small_bucket_cap();
+int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                            int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream);
+
 // explore.hip
 int launch_explore(const float* points, int N, int D, int K, int* knn_idx, float* knn_dist, int* old_idx,
                    hipStream_t stream);

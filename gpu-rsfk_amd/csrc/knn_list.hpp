@@ -58,6 +58,14 @@ struct KnnRow {
         changed = true;
     }
 
+    // values already in registers and known to be sorted
+    __device__ __forceinline__ void init_sorted(int K)
+    {
+        kk = K;
+        changed = false;
+        tau = last_slot();
+    }
+
     // values already in registers (slot k = lane + 64*s); slots >= K must hold (-2, +inf)
     __device__ __forceinline__ void init_from_regs(int K)
     {
