@@ -41,13 +41,13 @@ double now_s()
 }
 
 // how many trees to build per batch: as many as fit in a quarter of the free memory
-int choose_batch(int n_trees, int N, int MIN)
+int choose_batch(int n_trees, int N, int D, int MIN)
 {
     size_t free_b = 0, total_b = 0;
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = (size_t)8 << 30;
     const size_t budget = free_b / 4;
     int B = std::min(n_trees, 64);
-    while (B > 1 && tree_ws_bytes(N, MIN, B) > budget) --B;
+    while (B > 1 && tree_ws_bytes(N, D, MIN, B) > budget) --B;
     return std::max(B, 1);
 }
 
@@ -76,9 +76,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     const double t_forest0 = now_s();
 
     if (n_trees > 0) {
-        const int B = choose_batch(n_trees, N, MIN);
+        const int B = choose_batch(n_trees, N, D, MIN);
         WsGuard ws;
-        if (tree_ws_alloc(&ws.w, N, MIN, B)) return 1;
+        if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
         std::vector<int> stats((size_t)4 * B);
         std::vector<EventPair> ev((size_t)B);
         for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
@@ -164,7 +164,7 @@ int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int M
                     std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[4])
 {
     WsGuard ws;
-    if (tree_ws_alloc(&ws.w, N, MIN, 1)) return 1;
+    if (tree_ws_alloc(&ws.w, N, D, MIN, 1)) return 1;
     if (build_tree_batch(ws.w, d_points, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
     const int nl = stats[0];
     perm.resize((size_t)N);

@@ -8,8 +8,8 @@ namespace rsfk {
 struct TreeBatchWorkspace;
 
 // tree_build.hip
-size_t tree_ws_bytes(int N, int MIN, int B);
-int tree_ws_alloc(TreeBatchWorkspace** out, int N, int MIN, int B);
+size_t tree_ws_bytes(int N, int D, int MIN, int B);
+int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B);
 void tree_ws_free(TreeBatchWorkspace* w);
 int tree_ws_leaf_cap(const TreeBatchWorkspace* w);
 const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
