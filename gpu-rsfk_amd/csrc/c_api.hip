@@ -117,9 +117,13 @@ RSFK_API int rsfk_explore_device(const float* d_points, int N, int D, int num_ne
                                  float* d_knn_sqr_distances, int* d_scratch, void* stream)
 {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (launch_explore(d_points, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, s)) return 1;
-    RSFK_HIP(hipStreamSynchronize(s));
-    return 0;
+    Bf16Copy bf;
+    int rc = bf16_copy_alloc(&bf, N, D);
+    if (!rc) rc = bf16_copy_fill(bf, d_points, N, D, s);
+    if (!rc) rc = launch_explore(d_points, &bf, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, s);
+    if (!rc && hipStreamSynchronize(s) != hipSuccess) { set_last_error("hipStreamSynchronize failed"); rc = 1; }
+    bf16_copy_free(&bf);
+    return rc;
 }
 
 RSFK_API int rsfk_build_tree_host(const float* points, int N, int D, int MIN_TREE_CHILD, int MAX_TREE_CHILD,
@@ -194,10 +198,15 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
     RSFK_HIP(hipMemcpy(dp.p, points, sizeof(float) * (size_t)N * (size_t)D, hipMemcpyHostToDevice));
     RSFK_HIP(hipMemcpy(dki.p, knn_indices, sizeof(int) * nk, hipMemcpyHostToDevice));
     RSFK_HIP(hipMemcpy(dkd.p, knn_sqr_distances, sizeof(float) * nk, hipMemcpyHostToDevice));
-    for (int it = 0; it < passes; ++it)
-        if (launch_explore(static_cast<const float*>(dp.p), N, D, num_neighbors, static_cast<int*>(dki.p),
-                           static_cast<float*>(dkd.p), static_cast<int*>(dold.p), nullptr))
-            return 1;
+    Bf16Copy bf;
+    int rc = bf16_copy_alloc(&bf, N, D);
+    if (!rc) rc = bf16_copy_fill(bf, static_cast<const float*>(dp.p), N, D, nullptr);
+    for (int it = 0; it < passes && !rc; ++it)
+        rc = launch_explore(static_cast<const float*>(dp.p), &bf, N, D, num_neighbors, static_cast<int*>(dki.p),
+                            static_cast<float*>(dkd.p), static_cast<int*>(dold.p), nullptr);
+    if (!rc && hipDeviceSynchronize() != hipSuccess) { set_last_error("hipDeviceSynchronize failed"); rc = 1; }
+    bf16_copy_free(&bf);
+    if (rc) return rc;
     RSFK_HIP(hipDeviceSynchronize());
     RSFK_HIP(hipMemcpy(knn_indices, dki.p, sizeof(int) * nk, hipMemcpyDeviceToHost));
     RSFK_HIP(hipMemcpy(knn_sqr_distances, dkd.p, sizeof(float) * nk, hipMemcpyDeviceToHost));

@@ -59,6 +59,10 @@ struct DevBuf {
     void* p = nullptr;
     ~DevBuf() { if (p) (void)hipFree(p); }
 };
+struct Bf16Guard {
+    Bf16Copy c;
+    ~Bf16Guard() { bf16_copy_free(&c); }
+};
 struct EventPair {
     hipEvent_t a = nullptr, b = nullptr;
 };
@@ -74,6 +78,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     RSFK_CHECK(K <= 256, "forest: K above 256 is not supported");
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
     const double t_forest0 = now_s();
+    Bf16Guard bf;
+    if (bf16_copy_alloc(&bf.c, N, D)) return 1;
+    if (bf16_copy_fill(bf.c, d_points, N, D, stream)) return 1;
 
     if (n_trees > 0) {
         const int B = choose_batch(n_trees, N, D, MIN);
@@ -86,7 +93,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         for (int t0 = 0; t0 < n_trees && rc == 0; t0 += B) {
             const int nb = std::min(B, n_trees - t0);
             const double tb0 = now_s();
-            rc = build_tree_batch(ws.w, d_points, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
+            rc = build_tree_batch(ws.w, d_points, bf.c.rows, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
             if (rc) break;
             const double tb = now_s() - tb0;
             for (int j = 0; j < nb && rc == 0; ++j) {
@@ -125,7 +132,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         DevBuf old;
         RSFK_HIP(hipMalloc(&old.p, sizeof(int) * (size_t)N * (size_t)K));
         for (int it = 0; it < nnef; ++it) {
-            if (launch_explore(d_points, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), stream)) return 1;
+            if (launch_explore(d_points, &bf.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), stream)) return 1;
         }
         RSFK_HIP(hipStreamSynchronize(stream));
     }
@@ -165,7 +172,10 @@ int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int M
 {
     WsGuard ws;
     if (tree_ws_alloc(&ws.w, N, D, MIN, 1)) return 1;
-    if (build_tree_batch(ws.w, d_points, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
+    Bf16Guard bf;
+    if (bf16_copy_alloc(&bf.c, N, D)) return 1;
+    if (bf16_copy_fill(bf.c, d_points, N, D, nullptr)) return 1;
+    if (build_tree_batch(ws.w, d_points, bf.c.rows, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
     const int nl = stats[0];
     perm.resize((size_t)N);
     std::vector<int> ls((size_t)nl), lz((size_t)nl);

@@ -1,6 +1,7 @@
 // Internal interfaces between the translation units of the library.
 #pragma once
 #include "rsfk_common.hpp"
+#include "bf16.hpp"
 #include <vector>
 
 namespace rsfk {
@@ -16,8 +17,8 @@ const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
 int tree_small_threshold();
-int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, int MIN, int MAX, int MAX_DEPTH,
-                     int seed0, int nb, int* host_stats, hipStream_t stream);
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, int N, int D, int MIN, int MAX,
+                     int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream);
 
 // bucket_knn.hip
 int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
@@ -30,8 +31,8 @@ int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, c
                             int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream);
 
 // explore.hip
-int launch_explore(const float* points, int N, int D, int K, int* knn_idx, float* knn_dist, int* old_idx,
-                   hipStream_t stream);
+int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K, int* knn_idx, float* knn_dist,
+                   int* old_idx, hipStream_t stream);
 
 // forest.hip
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,

@@ -30,6 +30,7 @@
 // wavefront plays the role of the 32-lane warp.
 #include "rsfk_common.hpp"
 #include "wave64.hpp"
+#include "bf16.hpp"
 #include <vector>
 #include <algorithm>
 #include <cstring>
@@ -58,7 +59,7 @@ __device__ __forceinline__ void make_hyperplane(const float* __restrict__ x1, co
                                                 int D, float* nvec, float* b_out)
 {
     for (int d = threadIdx.x; d < D; d += blockDim.x) nvec[d] = x1[d] - x2[d];
-    if (threadIdx.x == 0 && (D & 1)) nvec[D] = 0.0f;       // pad to the even length of the bfloat16 rows
+    if (threadIdx.x < bf16_pitch(D) - D) nvec[D + threadIdx.x] = 0.0f;   // pad to the length of the bfloat16 rows
     if (threadIdx.x < 32) {
         float s = 0.0f;
         for (int d = threadIdx.x; d < D; d += 32) {
@@ -86,10 +87,11 @@ __device__ __forceinline__ float half_dot(const float* nvec, const float* __rest
 //
 // The decision is always the one of the fp32 test above, but most points never
 // touch their fp32 row: a bfloat16 copy of the row (half the bytes) gives an
-// approximate n.x together with S = sum |n_d||x_d|.  Rounding x to bfloat16
-// (round to nearest) changes n.x by at most 2^-9 S, and the fp32 summations of
-// either path are off by a few 2^-24 S, so whenever |approx - b| > 2^-8 S the
-// sign of (n.x - b) is the same for the exact fp32 evaluation.  Only the points
+// approximate n.x together with S~ = sum |n_d||x~_d|.  bfloat16 keeps 8 significant
+// bits: rounding x to x~ (round to nearest) changes n.x by at most
+// 2^-8 sum |n_d||x_d| <= 2^-8 (1+2^-7) S~, and the fp32 summations of either path are
+// off by a few 2^-24 S~, so whenever |approx - b| > 1.02 * 2^-8 S~ the sign of
+// (n.x - b) is the same for the exact fp32 evaluation.  Only the points
 // inside that band (a few per cent) read the fp32 row and repeat the test with
 // the exact arithmetic.  NaN or infinite values fail the band test and take the
 // exact path.
@@ -114,7 +116,7 @@ __device__ __forceinline__ bool side_right(const float* nvec, float b, const flo
     }
     da = half_butterfly_sum(da);
     sa = half_butterfly_sum(sa);
-    const bool certain = fabsf(da - b) > sa * (1.0f / 256.0f) + 1e-30f;
+    const bool certain = fabsf(da - b) > sa * (1.02f / 256.0f) + 1e-30f;
     bool right = da < b;
     const bool redo = valid && !certain;
     if (ballot64(redo) != 0) {
@@ -122,20 +124,6 @@ __device__ __forceinline__ bool side_right(const float* nvec, float b, const flo
         if (redo) right = dot < b;
     }
     return right;
-}
-
-// fp32 -> bfloat16, round to nearest even; rows padded to an even length with zeros
-__global__ void k_to_bf16(const float* __restrict__ points, uint16_t* __restrict__ out, int N, int D, int Db)
-{
-    const size_t total = (size_t)N * (size_t)Db;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t r = i / (size_t)Db;
-        const int d = (int)(i - r * (size_t)Db);
-        uint32_t u = d < D ? __float_as_uint(points[r * (size_t)D + d]) : 0u;
-        if ((u & 0x7f800000u) != 0x7f800000u) u += 0x7fffu + ((u >> 16) & 1u);      // finite: round
-        else if (u & 0x007fffffu) u |= 0x00400000u;                                  // NaN stays NaN
-        out[i] = (uint16_t)(u >> 16);
-    }
 }
 
 // Append a child node either to the next wide level or to the tail queue.
@@ -259,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
                                                  const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
                                                  const int* __restrict__ chunk2node, int* __restrict__ chunk_left)
 {
-    extern __shared__ __align__(16) float nvec[];          // D floats (+1 pad)
+    extern __shared__ __align__(16) float nvec[];          // bf16_pitch(D) floats
     __shared__ float b_s;
     __shared__ int left_s;
     const int c = blockIdx.x;
@@ -286,7 +274,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
         const int pos = pos0 + it * kHalves + half;
         const bool valid = pos < pos1;
         const int id = valid ? (perm[pos] & kIdMask) : 0;
-        const bool right = side_right(nvec, b, points, pb16, (P.D + 1) & ~1, id, P.D, hl, valid);   // build_tree_check_points_side.cu:149
+        const bool right = side_right(nvec, b, points, pb16, bf16_pitch(P.D), id, P.D, hl, valid);   // build_tree_check_points_side.cu:149
         if (valid && hl == 0) {
             perm[pos] = right ? (id | (int)0x80000000) : id;
             lefts += right ? 0 : 1;
@@ -405,12 +393,12 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr)
 {
-    // dynamic LDS: seg[small] | tmp[small] | nvec[D+1] | stack[stack_cap]
+    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_pitch(D)] | stack[stack_cap]
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int* seg = reinterpret_cast<int*>(lds_raw);
     int* tmp = seg + P.small;
     float* nvec = reinterpret_cast<float*>(tmp + P.small);
-    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + P.D + 1) * 4 + 15) / 16 * 16);
+    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + bf16_pitch(P.D)) * 4 + 15) / 16 * 16);
     __shared__ float b_s;
     __shared__ int left_s, top_s;
     __shared__ int wcnt[kBlock / 64];
@@ -467,7 +455,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
             const int i = it * kHalves + half;
             const bool valid = i < nd.count;
             const int id = valid ? seg[nd.start + i] : 0;
-            const bool right = side_right(nvec, b, points, pb16, (P.D + 1) & ~1, id, P.D, hl, valid);
+            const bool right = side_right(nvec, b, points, pb16, bf16_pitch(P.D), id, P.D, hl, valid);
             if (valid && hl == 0) {
                 if (right) seg[nd.start + i] = id | (int)0x80000000; else ++lefts;
             }
@@ -545,8 +533,6 @@ struct TreeBatchWorkspace {
     int* leaf_size = nullptr;
     TreeStats* stats = nullptr;
     LevelCounters* ctr = nullptr;
-    uint16_t* pb16 = nullptr;            // bfloat16 copy of the points, rows padded to even length
-    const float* pb16_src = nullptr;     // the points it was made from
     int D = 0;
     LevelCounters* h_ctr = nullptr;      // pinned
     TreeStats* h_stats = nullptr;        // pinned
@@ -555,7 +541,7 @@ struct TreeBatchWorkspace {
 static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
-                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.pb16};
+                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
@@ -580,7 +566,7 @@ int tree_small_threshold() { return 1024; }
 size_t tree_ws_bytes(int N, int D, int MIN, int B)
 {
     const size_t lc = (size_t)N / (size_t)std::max(MIN, 1) + 2;
-    return (size_t)N * (size_t)((D + 1) & ~1) * 2 + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24));
+    return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24));
 }
 
 int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
@@ -605,18 +591,18 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     if (dmalloc(&w->leaf_size, (size_t)B * w->leaf_cap)) return 1;
     if (dmalloc(&w->stats, (size_t)B)) return 1;
     if (dmalloc(&w->ctr, (size_t)1)) return 1;
-    if (dmalloc(&w->pb16, (size_t)N * (size_t)((D + 1) & ~1))) return 1;
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_ctr), sizeof(LevelCounters)));
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stats), sizeof(TreeStats) * (size_t)B));
     return 0;
 }
 
-// Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  On return perm[0] of
+// Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  pb16 = rows of the bfloat16 copy of the points (may be
+// null: every side test then reads the fp32 row).  On return perm[0] of
 // tree t holds the point ids grouped by bucket and (leaf_start, leaf_size)[t]
 // the buckets, in no particular order.  host_stats receives 4 ints per tree:
 // number of leaves, number of levels, largest and smallest bucket.
-int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, int MIN, int MAX, int MAX_DEPTH,
-                     int seed0, int nb, int* host_stats, hipStream_t stream)
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, int N, int D, int MIN, int MAX,
+                     int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream)
 {
     RSFK_CHECK(nb >= 1 && nb <= w->B && N == w->N && D == w->D, "tree batch: workspace does not match the request");
     RSFK_CHECK(N >= 1 && D >= 1, "tree batch: N and D must be positive");
@@ -638,16 +624,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, i
     hipLaunchKernelGGL(k_init_roots, dim3((nb + 63) / 64), dim3(64), 0, stream, w->nodes[0], w->tail, w->ctr, P, nb, seed0);
     RSFK_HIP(hipGetLastError());
 
-    if (w->pb16_src != points) {
-        const int Db = (D + 1) & ~1;
-        const size_t total = (size_t)N * (size_t)Db;
-        const int grid = (int)std::min<size_t>((total + 255) / 256, 262144);
-        hipLaunchKernelGGL(k_to_bf16, dim3(grid), dim3(256), 0, stream, points, w->pb16, N, D, Db);
-        RSFK_HIP(hipGetLastError());
-        w->pb16_src = points;
-    }
     int cur = 0;
-    const size_t side_lds = (size_t)(D + 1) * sizeof(float);
+    const size_t side_lds = (size_t)bf16_pitch(D) * sizeof(float);
     // wide levels
     while (true) {
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
@@ -664,7 +642,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, i
         // n_next := 0 for the level being produced
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
-        hipLaunchKernelGGL(k_side, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, w->pb16, P, w->perm[0], w->perm[1],
+        hipLaunchKernelGGL(k_side, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, P, w->perm[0], w->perm[1],
                            w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr);
@@ -676,10 +654,10 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, int N, int D, i
     RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
     if (n_tail > 0) {
         const int stack_cap = P.small / std::max(MIN, 1) + 4;
-        const size_t lds = ((size_t)(2 * P.small + D + 1) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
+        const size_t lds = ((size_t)(2 * P.small + bf16_pitch(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, w->pb16, P, w->perm[0], w->perm[1], w->perm[0],
+        hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
                            w->tail, n_tail, stack_cap, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr);
         RSFK_HIP(hipGetLastError());
     }
