@@ -4,26 +4,32 @@
 // (src/kernels/nearest_neighbors_exploring.cu:41-146) and its host loop
 // (src/rsfk.cu:2100-2135).
 //
-// One wavefront per point:
-//   * the K*K candidate ids are read with coalesced row reads of the snapshot,
-//     up to 16 rows of 64 ids in flight at a time;
-//   * a per-wavefront hash set in LDS drops ids that were already seen (the
-//     point itself, its current row, earlier candidates), so each distinct
-//     candidate is looked at once.  The reference re-evaluates repeats; the
-//     result is the same because a rejected candidate stays rejected (the row
-//     maximum only decreases) and an accepted one is found in the row later;
-//   * surviving ids are compacted (ballot + mbcnt ranks) into a queue.  Whenever
-//     64 are queued they are screened on the bfloat16 copy of the points: the
-//     rows are gathered with coalesced 128-byte segments (8 lanes per row, 64
-//     dimensions per step), transposed through LDS, and each lane accumulates for
-//     "its" candidate the approximate squared distance d~ and a bound E on
-//     |d~ - d|; a candidate with d~ - E >= row maximum cannot enter the row and is
-//     dropped without ever touching its fp32 row (most candidates);
-//   * the few that pass go to a second queue and get the exact distance from the
-//     fp32 rows: same gather/transposition, 32 dimensions per step, sequential
-//     fused multiply-add chain per candidate -- the arithmetic of the bucket
-//     kernel (compute_knn_from_buckets.cu:40-54), so a pair has one distance
-//     value everywhere -- and are then offered to the sorted row.
+// One wavefront per point, in three stages:
+//
+//  1. collect.  The K*K candidate ids are read with coalesced row reads of the
+//     snapshot (16 rows of 64 ids in flight at a time) and put into a hash set in
+//     LDS that was seeded with the point itself and its current row.  Only ids
+//     that are new to the set survive, so each distinct candidate is looked at
+//     once.  (The reference re-evaluates repeats; the result is the same because
+//     a rejected candidate stays rejected -- the row maximum only decreases -- and
+//     an accepted one is found in the row afterwards.)  The set is then compacted
+//     in place into the list of candidates.  When the set cannot hold all K*K ids
+//     (large K) the neighbours are processed in groups, each with a fresh set.
+//
+//  2. screen, on the bfloat16 copy of the points.  64 candidates at a time: their
+//     rows (up to 128 dimensions = 256 bytes each) are requested with coalesced
+//     128-byte segments, 8 lanes per row, while the previous 64 are being
+//     evaluated (two batches of loads are in flight per wavefront: the stage is
+//     bound by gather latency, so memory-level parallelism is what counts).  Rows
+//     are transposed through LDS and each lane accumulates for "its" candidate
+//     the approximate squared distance d~ and the quantity T below; a candidate
+//     with d~ - E >= row maximum cannot enter the row and is dropped without its
+//     fp32 row ever being touched.
+//
+//  3. exact.  The few candidates that pass get the exact distance from the fp32
+//     rows (same gather/transposition, sequential fused multiply-add chain per
+//     candidate: the arithmetic of the bucket kernel, compute_knn_from_buckets.cu:40-54,
+//     so a pair has one distance value everywhere) and are offered to the sorted row.
 //
 // Error bound of the screen.  bfloat16 keeps 8 significant bits, so c~ = c + e with
 // |e_d| <= 2^-8 |c_d| <= 2^-8 (1+2^-7) |c~_d| (round to nearest).  From
@@ -41,12 +47,12 @@ namespace rsfk {
 
 namespace {
 
-constexpr int kWavesPerBlock = 4;
 constexpr int kChunk = 32;              // fp32 dimensions per staging step (exact path)
-constexpr int kChunkB = 64;             // bfloat16 dimensions per staging step (screen)
 constexpr int kPitch = kChunk + 4;      // 36 words = 9 x 16 B: conflict-free b128 reads down a column of rows
-constexpr int kQueue = 128;             // entries of each candidate queue per wavefront
+constexpr int kBlockB = 128;            // bfloat16 dimensions per pipeline stage of the screen (2 x 64)
+constexpr int kQueue2 = 128;            // candidates waiting for the exact distance
 constexpr int kIdRows = 16;             // batches of 64 candidate ids loaded back to back
+constexpr int kEmpty = (int)0x80000000; // free slot of the hash set
 
 __device__ __forceinline__ uint32_t hash_id(int c)
 {
@@ -54,33 +60,35 @@ __device__ __forceinline__ uint32_t hash_id(int c)
     return h ^ (h >> 15);
 }
 
-// returns true when c was not in the set (and is now, if there was room)
-__device__ __forceinline__ bool set_insert(int* table, int mask, int c, int max_probe)
+// Set of ids with open addressing.  Seeds (ids that must not become candidates) are
+// stored as -id-1, candidates as id.  Returns true when c was new.  The caller
+// guarantees a free slot exists.
+__device__ __forceinline__ bool set_insert(int* table, int mask, int c, bool seed)
 {
     uint32_t h = hash_id(c) & (uint32_t)mask;
-    for (int i = 0; i < max_probe; ++i) {
-        const int old = atomicCAS(&table[h], -1, c);
-        if (old == -1) return true;
-        if (old == c) return false;
+    const int stored = seed ? -c - 1 : c;
+    for (int i = 0; i <= mask; ++i) {
+        const int old = atomicCAS(&table[h], kEmpty, stored);
+        if (old == kEmpty) return true;
+        if (old == c || old == -c - 1) return false;
         h = (h + 1) & (uint32_t)mask;
     }
-    return true;     // set is crowded: treat as new, the row itself is still checked on insertion
+    return false;
 }
 
 struct ExploreLds {          // per wavefront; sizes fixed at launch
-    int* table;              // hash set, table_size ints
+    int* table;              // hash set / candidate list, table_size ints
     int* srow;               // snapshot of the point's own row, K ints
-    int* queue;              // fresh candidates waiting for the screen
     int* queue2;             // candidates that passed the screen, waiting for the exact distance
     float* xrow;             // the point's coordinates, zero padded to bf16_pitch(D)
     float* tile;             // 64 x kPitch words
 };
 
 // Load one 16-byte piece (4 dimensions) of a candidate row, zero beyond D.
-__device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int d, int D, bool vec_ok, bool live)
+__device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int d, int D, bool vec_ok)
 {
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (live && d < D) {
+    if (d < D) {
         if (vec_ok) {
             v = *reinterpret_cast<const float4*>(row + d);
         } else {
@@ -93,27 +101,24 @@ __device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int 
     return v;
 }
 
-// Exact distances of the first n candidates of `queue` to the point, then offer them.
+// Exact distances of the first n candidates of `list` to the point, then offer them.
 template <int SL>
-__device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* queue, int n,
+__device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
                                             const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row)
 {
     const int lane = lane_id();
     const int sub = lane >> 3;          // which of 8 rows of a load step
     const int piece = lane & 7;         // which 16-byte piece of the 128-byte segment
-    const int my_c = lane < n ? queue[lane] : -1;
+    const int my_c = lane < n ? list[lane] : -1;
     const float* rp[8];
-    bool live[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int r = i * 8 + sub;
-        live[i] = r < n;
-        const int c = live[i] ? queue[r] : 0;
-        rp[i] = points + (size_t)c * (size_t)D;
+        rp[i] = points + (size_t)list[r < n ? r : 0] * (size_t)D;      // rows beyond n repeat row 0 (ignored later)
     }
     float4 pre[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok, live[i]);
+    for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok);
     float acc = 0.0f;
     const float tau0 = row.tau;
     for (int d0 = 0; d0 < D; d0 += kChunk) {
@@ -123,7 +128,7 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* queu
             *reinterpret_cast<float4*>(&L.tile[(i * 8 + sub) * kPitch + piece * 4]) = pre[i];
         if (d0 + kChunk < D) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], d0 + kChunk + piece * 4, D, vec_ok, live[i]);
+            for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], d0 + kChunk + piece * 4, D, vec_ok);
         }
         wave_lds_sync();
         const int pieces = min(8, (D - d0 + 3) >> 2);
@@ -156,47 +161,43 @@ __device__ __forceinline__ void screen_pair(uint32_t w, float x0, float x1, floa
     ta = __builtin_fmaf(fabsf(f1), fabsf(c1), ta);
 }
 
-// Screen the first n candidates of L.queue on the bfloat16 copy.  Returns, per lane,
-// whether its candidate may still enter the row.
-template <int SL>
-__device__ __forceinline__ bool screen_batch(const ExploreLds& L, int n, const Bf16Copy& bf, int D, int Db,
-                                             const KnnRow<SL>& row)
+// One pipeline stage of the screen = 128 bfloat16 dimensions of 64 candidate rows.
+struct ScreenLoads {
+    uint4 v[16];             // v[h*8+i]: half h (64 dimensions), rows i*8+sub, piece lane&7
+};
+
+__device__ __forceinline__ void screen_issue(ScreenLoads& S, const int* list, int n, const uint16_t* __restrict__ rows,
+                                             int Db, int b0)
 {
     const int lane = lane_id();
-    const int sub = lane >> 3;
-    const int piece = lane & 7;          // 16 bytes = 8 bfloat16 values
-    const int my_c = lane < n ? L.queue[lane] : 0;
-    const float qn = bf.norms[my_c];
-    const uint16_t* rp[8];
-    bool live[8];
+    const int sub = lane >> 3, piece = lane & 7;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int r = i * 8 + sub;
-        live[i] = r < n;
-        const int c = live[i] ? L.queue[r] : 0;
-        rp[i] = bf.rows + (size_t)c * (size_t)Db;
-    }
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
-    uint4 pre[8];
+        const uint16_t* rp = rows + (size_t)list[r < n ? r : 0] * (size_t)Db + b0 + piece * 8;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-        pre[i] = (live[i] && piece * 8 < Db) ? *reinterpret_cast<const uint4*>(rp[i] + piece * 8) : zero4;
-    float da = 0.0f, ta = 0.0f;
-    const float tau = row.tau;
-    const float slack = (float)(D + 8) * (1.0f / 4194304.0f);      // (D+8) 2^-22: fp32 summation error of both sums
+        for (int h = 0; h < 2; ++h) {
+            S.v[h * 8 + i] = make_uint4(0, 0, 0, 0);
+            if (b0 + h * 64 + piece * 8 < Db) S.v[h * 8 + i] = *reinterpret_cast<const uint4*>(rp + h * 64);
+        }
+    }
+}
+
+// Accumulate one stage into (da, ta) of this lane's candidate.
+__device__ __forceinline__ void screen_consume(const ScreenLoads& S, const ExploreLds& L, int Db, int b0, float& da,
+                                               float& ta)
+{
+    const int lane = lane_id();
+    const int sub = lane >> 3, piece = lane & 7;
     uint32_t* tile = reinterpret_cast<uint32_t*>(L.tile);
-    bool may = lane < n;
-    for (int d0 = 0; d0 < Db; d0 += kChunkB) {
-        wave_lds_sync();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int d0 = b0 + h * 64;
+        if (d0 >= Db) break;
+        wave_lds_sync();                 // previous reads of the tile are done
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<uint4*>(&tile[(i * 8 + sub) * kPitch + piece * 4]) = pre[i];
-        if (d0 + kChunkB < Db) {
-            const int dn = d0 + kChunkB + piece * 8;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                pre[i] = (live[i] && dn < Db) ? *reinterpret_cast<const uint4*>(rp[i] + dn) : zero4;
-        }
+            *reinterpret_cast<uint4*>(&tile[(i * 8 + sub) * kPitch + piece * 4]) = S.v[h * 8 + i];
         wave_lds_sync();
         const int pieces = min(8, (Db - d0) >> 3);
         const uint32_t* mine = &tile[lane * kPitch];
@@ -210,113 +211,158 @@ __device__ __forceinline__ bool screen_batch(const ExploreLds& L, int n, const B
             screen_pair(w.z, xb.x, xb.y, da, ta);
             screen_pair(w.w, xb.z, xb.w, da, ta);
         }
-        // lower bound of the exact distance from the dimensions seen so far
-        const float e = ta * (1.02f / 128.0f) + qn * (1.05f / 65536.0f) + da * slack;
-        may = lane < n && (da - e < tau);
-        if (ballot64(may) == 0) break;
     }
-    wave_lds_sync();
-    return may;
+}
+
+// Stages are numbered s = batch * nblk + block; list holds U candidates.
+struct ScreenCtx {
+    const int* list;
+    int U, nblk, Db, D;
+};
+
+template <int SL>
+__device__ __forceinline__ void screen_stage_finish(const ScreenCtx& C, const ExploreLds& L, const Bf16Copy& bf, int batch,
+                                                    float da, float ta, KnnRow<SL>& row, int& queued2,
+                                                    const float* __restrict__ points, bool vec_ok)
+{
+    const int lane = lane_id();
+    const int n = min(64, C.U - batch * 64);
+    const int my_c = C.list[batch * 64 + (lane < n ? lane : 0)];
+    const float qn = bf.norms[my_c];
+    const float slack = (float)(C.D + 8) * (1.0f / 4194304.0f);      // (D+8) 2^-22: fp32 summation error of both sums
+    const float e = ta * (1.02f / 128.0f) + qn * (1.05f / 65536.0f) + da * slack;
+    const bool may = lane < n && (da - e < row.tau);
+    const uint64_t pm = ballot64(may);
+    if (pm == 0) return;
+    if (may) L.queue2[queued2 + mask_prefix(pm)] = my_c;
+    queued2 += __popcll(pm);
+    if (queued2 >= 64) {
+        wave_lds_sync();
+        exact_batch<SL>(L, L.queue2, 64, points, C.D, vec_ok, row);
+        const int rest = queued2 - 64;
+        const int mv = lane < rest ? L.queue2[64 + lane] : 0;
+        wave_lds_sync();
+        if (lane < rest) L.queue2[lane] = mv;
+        queued2 = rest;
+        wave_lds_sync();
+    }
 }
 
 template <int SL>
-__global__ __launch_bounds__(64 * kWavesPerBlock) void k_explore(const float* __restrict__ points, Bf16Copy bf, int N,
-                                                                  int D, int K, const int* __restrict__ old_idx,
-                                                                  int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                                  int table_size, int wave_lds_ints, int dpad)
+__device__ __forceinline__ void screen_all(const ScreenCtx& C, const ExploreLds& L, const Bf16Copy& bf, KnnRow<SL>& row,
+                                           int& queued2, const float* __restrict__ points, bool vec_ok)
+{
+    const int nb = (C.U + 63) >> 6;
+    const int stages = nb * C.nblk;
+    ScreenLoads A, B;
+    float da = 0.0f, ta = 0.0f;
+    auto issue = [&](ScreenLoads& S, int s) {
+        const int batch = s / C.nblk, blk = s - batch * C.nblk;
+        screen_issue(S, C.list + batch * 64, min(64, C.U - batch * 64), bf.rows, C.Db, blk * kBlockB);
+    };
+    auto consume = [&](const ScreenLoads& S, int s) {
+        const int batch = s / C.nblk, blk = s - batch * C.nblk;
+        if (blk == 0) { da = 0.0f; ta = 0.0f; }
+        screen_consume(S, L, C.Db, blk * kBlockB, da, ta);
+        if (blk == C.nblk - 1) screen_stage_finish<SL>(C, L, bf, batch, da, ta, row, queued2, points, vec_ok);
+    };
+    if (stages > 0) issue(A, 0);
+    for (int s = 0; s < stages; s += 2) {
+        if (s + 1 < stages) issue(B, s + 1);
+        consume(A, s);
+        if (s + 1 < stages) {
+            if (s + 2 < stages) issue(A, s + 2);
+            consume(B, s + 1);
+        }
+    }
+}
+
+template <int SL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict__ points, Bf16Copy bf, int N, int D, int K,
+                                                         const int* __restrict__ old_idx, int* __restrict__ knn_idx,
+                                                         float* __restrict__ knn_dist, int table_size, int wave_lds_ints,
+                                                         int dpad, int rows_per_group)
 {
     extern __shared__ __align__(16) int lds_i[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int p = blockIdx.x * kWavesPerBlock + wave;
+    const int p = blockIdx.x * WAVES + wave;
     if (p >= N) return;                                   // whole wavefront leaves together
     int* base = lds_i + (size_t)wave * (size_t)wave_lds_ints;
     ExploreLds L;
     L.tile = reinterpret_cast<float*>(base);                        // 64*kPitch words, 16-byte aligned
     L.xrow = reinterpret_cast<float*>(base + 64 * kPitch);          // dpad floats (multiple of 8)
-    L.queue = base + 64 * kPitch + dpad;
-    L.queue2 = L.queue + kQueue;
-    L.table = L.queue2 + kQueue;
+    L.queue2 = base + 64 * kPitch + dpad;
+    L.table = L.queue2 + kQueue2;
     L.srow = L.table + table_size;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const bool use_screen = bf.rows != nullptr;
-    const int Db = bf16_pitch(D);
     const int mask = table_size - 1;
 
-    for (int i = lane; i < table_size; i += 64) L.table[i] = -1;
     KnnRow<SL> row;
     row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
     for (int k = lane; k < K; k += 64) L.srow[k] = old_idx[(size_t)p * K + k];
     const float* xp = points + (size_t)p * D;
     for (int d = lane; d < dpad; d += 64) L.xrow[d] = d < D ? xp[d] : 0.0f;
-    wave_lds_sync();
-    // seed the set with the point itself and its current row
-    if (lane == 0) set_insert(L.table, mask, p, table_size);
-#pragma unroll
-    for (int s = 0; s < SL; ++s)
-        if (row.idx[s] >= 0) set_insert(L.table, mask, row.idx[s], table_size);
 
-    const int total = K * K;
-    int queued = 0, queued2 = 0;                           // wave-uniform
-    for (int g0 = 0; g0 < total; g0 += 64 * kIdRows) {
-        int cand[kIdRows];
-#pragma unroll
-        for (int b = 0; b < kIdRows; ++b) {
-            const int e = g0 + b * 64 + lane;
-            int c = -1;
-            if (e < total) {
-                const int i = e / K, k = e - i * K;
-                const int q = L.srow[i];
-                if (q >= 0 && q < N) c = old_idx[(size_t)q * K + k];
-            }
-            cand[b] = c;
-        }
-#pragma unroll
-        for (int b = 0; b < kIdRows; ++b) {
-            if (g0 + b * 64 >= total) break;
-            const int c = cand[b];
-            bool fresh = c >= 0 && c < N && c != p;
-            if (fresh) fresh = set_insert(L.table, mask, c, 64);
-            const uint64_t m = ballot64(fresh);
-            if (fresh) L.queue[queued + mask_prefix(m)] = c;
-            queued += __popcll(m);
-            if (queued >= 64) {
-                wave_lds_sync();
-                if (use_screen) {
-                    const bool may = screen_batch<SL>(L, 64, bf, D, Db, row);
-                    const uint64_t pm = ballot64(may);
-                    if (may) L.queue2[queued2 + mask_prefix(pm)] = L.queue[lane];
-                    queued2 += __popcll(pm);
-                    if (queued2 >= 64) {
-                        wave_lds_sync();
-                        exact_batch<SL>(L, L.queue2, 64, points, D, vec_ok, row);
-                        const int rest2 = queued2 - 64;
-                        const int mv2 = lane < rest2 ? L.queue2[64 + lane] : 0;
-                        wave_lds_sync();
-                        if (lane < rest2) L.queue2[lane] = mv2;
-                        queued2 = rest2;
-                    }
-                } else {
-                    exact_batch<SL>(L, L.queue, 64, points, D, vec_ok, row);
-                }
-                wave_lds_sync();
-                // move the overflow to the front
-                const int rest = queued - 64;
-                const int mv = lane < rest ? L.queue[64 + lane] : 0;
-                wave_lds_sync();
-                if (lane < rest) L.queue[lane] = mv;
-                queued = rest;
-            }
-        }
-    }
-    if (queued > 0) {
+    ScreenCtx C;
+    C.list = L.table;
+    C.Db = bf16_pitch(D);
+    C.D = D;
+    C.nblk = (C.Db + kBlockB - 1) / kBlockB;
+    int queued2 = 0;                                       // wave-uniform
+
+    for (int i0 = 0; i0 < K; i0 += rows_per_group) {
+        const int i1 = min(K, i0 + rows_per_group);
+        // ---- collect -----------------------------------------------------------------
         wave_lds_sync();
+        for (int i = lane; i < table_size; i += 64) L.table[i] = kEmpty;
+        wave_lds_sync();
+        if (lane == 0) set_insert(L.table, mask, p, true);
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+            if (row.idx[s] >= 0) set_insert(L.table, mask, row.idx[s], true);
+        const int e_begin = i0 * K, e_end = i1 * K;
+        for (int g0 = e_begin; g0 < e_end; g0 += 64 * kIdRows) {
+            int cand[kIdRows];
+#pragma unroll
+            for (int b = 0; b < kIdRows; ++b) {
+                const int e = g0 + b * 64 + lane;
+                int c = -1;
+                if (e < e_end) {
+                    const int i = e / K, k = e - i * K;
+                    const int q = L.srow[i];
+                    if (q >= 0 && q < N) c = old_idx[(size_t)q * K + k];
+                }
+                cand[b] = c;
+            }
+#pragma unroll
+            for (int b = 0; b < kIdRows; ++b) {
+                if (g0 + b * 64 >= e_end) break;
+                const int c = cand[b];
+                if (c >= 0 && c < N) set_insert(L.table, mask, c, false);
+            }
+        }
+        wave_lds_sync();
+        // ---- compact the set in place into the candidate list --------------------------
+        int U = 0;
+        for (int t0 = 0; t0 < table_size; t0 += 64) {
+            const int v = L.table[t0 + lane];
+            const bool is_cand = v >= 0;
+            const uint64_t m = ballot64(is_cand);
+            wave_lds_sync();             // all reads of this block are done before the front is overwritten
+            if (is_cand) L.table[U + mask_prefix(m)] = v;
+            U += __popcll(m);
+        }
+        wave_lds_sync();
+        C.U = U;
+        // ---- screen / exact ------------------------------------------------------------
         if (use_screen) {
-            const bool may = screen_batch<SL>(L, queued, bf, D, Db, row);
-            const uint64_t pm = ballot64(may);
-            if (may) L.queue2[queued2 + mask_prefix(pm)] = L.queue[lane];
-            queued2 += __popcll(pm);
+            screen_all<SL>(C, L, bf, row, queued2, points, vec_ok);
         } else {
-            exact_batch<SL>(L, L.queue, queued, points, D, vec_ok, row);
+            for (int off = 0; off < U; off += 64) {
+                wave_lds_sync();
+                exact_batch<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+            }
         }
     }
     // drain the second queue (at most 127 entries)
@@ -334,6 +380,20 @@ int next_pow2(int v)
     return p;
 }
 
+template <int SL, int WAVES>
+int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, const int* old_idx, int* knn_idx,
+               float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, hipStream_t stream)
+{
+    const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore<SL, WAVES>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    dim3 grid((unsigned)((N + WAVES - 1) / WAVES)), block(64 * WAVES);
+    hipLaunchKernelGGL((k_explore<SL, WAVES>), grid, block, lds, stream, points, b, N, D, K, old_idx, knn_idx, knn_dist,
+                       table, wave_ints, dpad, rows_per_group);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
 }  // namespace
 
 // One exploration pass.  old_idx is scratch of N*K ints (receives the snapshot).
@@ -345,33 +405,35 @@ int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K,
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
     const int dpad = bf16_pitch(D);
-    const int fixed = 64 * kPitch + dpad + 2 * kQueue + K;              // ints per wavefront besides the set
-    RSFK_CHECK((fixed + 64) * 4 * kWavesPerBlock <= 150 * 1024, "exploration: D too large for the LDS budget");
-    // set size: at least the number of distinct ids a point can meet, capped by LDS
-    int table = std::max(64, next_pow2(K * K + K + 1));
-    // two workgroups per CU when possible (160 KB of LDS per CU)
-    const int pref_budget = 78 * 1024 / kWavesPerBlock / 4 - fixed;
-    const int max_budget = 150 * 1024 / kWavesPerBlock / 4 - fixed;
-    if (table > pref_budget && (table >> 1) >= K * K / 2 && (table >> 1) <= pref_budget) table >>= 1;
-    while (table > max_budget && table > 64) table >>= 1;
+    const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set
+    const int lds_ints = 150 * 1024 / 4;                                // usable LDS per workgroup
+    // The set must hold the seeds (K+1) and all candidates of a group of neighbours with room to
+    // spare.  Prefer 4 wavefronts per workgroup; shrink the workgroup, then the group of
+    // neighbours, when K is large.
+    // (the kernel walks the set 64 entries at a time: it must never be smaller than 64)
+    const int floor_table = next_pow2(4 * K + 66);
+    const int want = std::max(next_pow2(K * K + K + 2), floor_table);
+    RSFK_CHECK(fixed + floor_table <= lds_ints, "exploration: D or K too large for the LDS budget");
+    int waves = 4;
+    int table = want;
+    while (waves > 1 && fixed + table > lds_ints / waves) waves >>= 1;
+    while (table > floor_table && fixed + table > lds_ints / waves) table >>= 1;
+    int rows_per_group = K;
+    if (table < want) rows_per_group = std::max(1, (table * 3 / 4 - K - 1) / K);
+    RSFK_CHECK(table >= 64 && (table & (table - 1)) == 0 && rows_per_group >= 1, "exploration: bad set size");
     const int wave_ints = (fixed + table + 3) / 4 * 4;
-    const size_t lds = (size_t)kWavesPerBlock * (size_t)wave_ints * sizeof(int);
     Bf16Copy b;
     if (bf) b = *bf;
-    dim3 grid((unsigned)((N + kWavesPerBlock - 1) / kWavesPerBlock)), block(64 * kWavesPerBlock);
-#define RSFK_EXPLORE_LAUNCH(SLV)                                                                                   \
-    do {                                                                                                           \
-        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore<SLV>),                                \
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                       \
-        hipLaunchKernelGGL(k_explore<SLV>, grid, block, lds, stream, points, b, N, D, K, old_idx, knn_idx,         \
-                           knn_dist, table, wave_ints, dpad);                                                      \
-    } while (0)
-    if (K <= 64) RSFK_EXPLORE_LAUNCH(1);
-    else if (K <= 128) RSFK_EXPLORE_LAUNCH(2);
-    else RSFK_EXPLORE_LAUNCH(4);
-#undef RSFK_EXPLORE_LAUNCH
-    RSFK_HIP(hipGetLastError());
-    return 0;
+    const int sl = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
+#define RSFK_EXPLORE_CASE(SLV, WV)                                                                                      \
+    if (sl == SLV && waves == WV)                                                                                       \
+        return launch_one<SLV, WV>(points, b, N, D, K, old_idx, knn_idx, knn_dist, table, wave_ints, dpad,              \
+                                   rows_per_group, stream);
+    RSFK_EXPLORE_CASE(1, 4) RSFK_EXPLORE_CASE(1, 2) RSFK_EXPLORE_CASE(1, 1)
+    RSFK_EXPLORE_CASE(2, 4) RSFK_EXPLORE_CASE(2, 2) RSFK_EXPLORE_CASE(2, 1)
+    RSFK_EXPLORE_CASE(4, 4) RSFK_EXPLORE_CASE(4, 2) RSFK_EXPLORE_CASE(4, 1)
+#undef RSFK_EXPLORE_CASE
+    RSFK_CHECK(false, "exploration: no kernel for this configuration");
 }
 
 }  // namespace rsfk
