@@ -138,8 +138,13 @@ def main():
     expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
     alg_bytes = float(N) * (4 * D + 4 + 16 * K)
     achieved = alg_bytes / knn_s / 1e9 if knn_s > 0 else 0.0
-    roofline = {"kernel": "k_bucket_knn", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload, each scaled by
+    # what the same counter reads for a plain copy of known size (FETCH x2.0, WRITE x1.0); only known for the
+    # default workload
+    default_workload = (args.workload == "uniform" and (N, D, K) == (1000000, 100, 32) and (mn, mx) == (33, 66))
+    traffic = 1.16e9 if default_workload else None
+    roofline = {"kernel": "k_bucket_knn_small + k_bucket_knn", "bound": "hbm", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4),
                 "launches_per_step": T}
 

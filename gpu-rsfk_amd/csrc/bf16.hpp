@@ -13,7 +13,11 @@
 
 namespace rsfk {
 
-__host__ __device__ inline int bf16_pitch(int D) { return (D + 7) & ~7; }
+// Row pitch in values: rows start on 64-byte boundaries so that a row touches the
+// minimum number of memory sectors.  bf16_valid(D) <= bf16_pitch(D) is the length the
+// kernels loop over (whole 16-byte pieces); values between D and the pitch are zero.
+__host__ __device__ inline int bf16_pitch(int D) { return (D + 31) & ~31; }
+__host__ __device__ inline int bf16_valid(int D) { return (D + 7) & ~7; }
 
 struct Bf16Copy {
     uint16_t* rows = nullptr;     // N x bf16_pitch(D)

@@ -80,7 +80,7 @@ struct ExploreLds {          // per wavefront; sizes fixed at launch
     int* table;              // hash set / candidate list, table_size ints
     int* srow;               // snapshot of the point's own row, K ints
     int* queue2;             // candidates that passed the screen, waiting for the exact distance
-    float* xrow;             // the point's coordinates, zero padded to bf16_pitch(D)
+    float* xrow;             // the point's coordinates, zero padded to bf16_valid(D)
     float* tile;             // 64 x kPitch words
 };
 
@@ -167,7 +167,7 @@ struct ScreenLoads {
 };
 
 __device__ __forceinline__ void screen_issue(ScreenLoads& S, const int* list, int n, const uint16_t* __restrict__ rows,
-                                             int Db, int b0)
+                                             int Db, int Dv, int b0)
 {
     const int lane = lane_id();
     const int sub = lane >> 3, piece = lane & 7;
@@ -178,7 +178,7 @@ __device__ __forceinline__ void screen_issue(ScreenLoads& S, const int* list, in
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             S.v[h * 8 + i] = make_uint4(0, 0, 0, 0);
-            if (b0 + h * 64 + piece * 8 < Db) S.v[h * 8 + i] = *reinterpret_cast<const uint4*>(rp + h * 64);
+            if (b0 + h * 64 + piece * 8 < Dv) S.v[h * 8 + i] = *reinterpret_cast<const uint4*>(rp + h * 64);
         }
     }
 }
@@ -217,7 +217,7 @@ __device__ __forceinline__ void screen_consume(const ScreenLoads& S, const Explo
 // Stages are numbered s = batch * nblk + block; list holds U candidates.
 struct ScreenCtx {
     const int* list;
-    int U, nblk, Db, D;
+    int U, nblk, Db, Dv, D;
 };
 
 template <int SL>
@@ -258,12 +258,12 @@ __device__ __forceinline__ void screen_all(const ScreenCtx& C, const ExploreLds&
     float da = 0.0f, ta = 0.0f;
     auto issue = [&](ScreenLoads& S, int s) {
         const int batch = s / C.nblk, blk = s - batch * C.nblk;
-        screen_issue(S, C.list + batch * 64, min(64, C.U - batch * 64), bf.rows, C.Db, blk * kBlockB);
+        screen_issue(S, C.list + batch * 64, min(64, C.U - batch * 64), bf.rows, C.Db, C.Dv, blk * kBlockB);
     };
     auto consume = [&](const ScreenLoads& S, int s) {
         const int batch = s / C.nblk, blk = s - batch * C.nblk;
         if (blk == 0) { da = 0.0f; ta = 0.0f; }
-        screen_consume(S, L, C.Db, blk * kBlockB, da, ta);
+        screen_consume(S, L, C.Dv, blk * kBlockB, da, ta);
         if (blk == C.nblk - 1) screen_stage_finish<SL>(C, L, bf, batch, da, ta, row, queued2, points, vec_ok);
     };
     if (stages > 0) issue(A, 0);
@@ -307,8 +307,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     ScreenCtx C;
     C.list = L.table;
     C.Db = bf16_pitch(D);
+    C.Dv = bf16_valid(D);
     C.D = D;
-    C.nblk = (C.Db + kBlockB - 1) / kBlockB;
+    C.nblk = (C.Dv + kBlockB - 1) / kBlockB;
     int queued2 = 0;                                       // wave-uniform
 
     for (int i0 = 0; i0 < K; i0 += rows_per_group) {
@@ -404,7 +405,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K,
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
-    const int dpad = bf16_pitch(D);
+    const int dpad = bf16_valid(D);
     const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set
     const int lds_ints = 150 * 1024 / 4;                                // usable LDS per workgroup
     // The set must hold the seeds (K+1) and all candidates of a group of neighbours with room to

@@ -59,7 +59,7 @@ __device__ __forceinline__ void make_hyperplane(const float* __restrict__ x1, co
                                                 int D, float* nvec, float* b_out)
 {
     for (int d = threadIdx.x; d < D; d += blockDim.x) nvec[d] = x1[d] - x2[d];
-    if (threadIdx.x < bf16_pitch(D) - D) nvec[D + threadIdx.x] = 0.0f;   // pad to the length of the bfloat16 rows
+    if (threadIdx.x < bf16_valid(D) - D) nvec[D + threadIdx.x] = 0.0f;   // pad to whole 16-byte pieces of the bfloat16 rows
     if (threadIdx.x < 32) {
         float s = 0.0f;
         for (int d = threadIdx.x; d < D; d += 32) {
@@ -103,7 +103,7 @@ __device__ __forceinline__ bool side_right(const float* nvec, float b, const flo
     const uint32_t* row = reinterpret_cast<const uint32_t*>(pb16 + (size_t)id * (size_t)Db);
     float da = 0.0f, sa = 0.0f;
     if (valid) {
-        for (int e = 2 * hl; e < Db; e += 64) {
+        for (int e = 2 * hl; e < bf16_valid(D); e += 64) {
             const uint32_t w = row[e >> 1];
             const float x0 = __uint_as_float(w << 16);
             const float x1 = __uint_as_float(w & 0xffff0000u);
@@ -247,7 +247,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
                                                  const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
                                                  const int* __restrict__ chunk2node, int* __restrict__ chunk_left)
 {
-    extern __shared__ __align__(16) float nvec[];          // bf16_pitch(D) floats
+    extern __shared__ __align__(16) float nvec[];          // bf16_valid(D) floats
     __shared__ float b_s;
     __shared__ int left_s;
     const int c = blockIdx.x;
@@ -393,12 +393,12 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr)
 {
-    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_pitch(D)] | stack[stack_cap]
+    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_valid(D)] | stack[stack_cap]
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int* seg = reinterpret_cast<int*>(lds_raw);
     int* tmp = seg + P.small;
     float* nvec = reinterpret_cast<float*>(tmp + P.small);
-    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + bf16_pitch(P.D)) * 4 + 15) / 16 * 16);
+    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + bf16_valid(P.D)) * 4 + 15) / 16 * 16);
     __shared__ float b_s;
     __shared__ int left_s, top_s;
     __shared__ int wcnt[kBlock / 64];
@@ -625,7 +625,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_HIP(hipGetLastError());
 
     int cur = 0;
-    const size_t side_lds = (size_t)bf16_pitch(D) * sizeof(float);
+    const size_t side_lds = (size_t)bf16_valid(D) * sizeof(float);
     // wide levels
     while (true) {
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
@@ -654,7 +654,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
     if (n_tail > 0) {
         const int stack_cap = P.small / std::max(MIN, 1) + 4;
-        const size_t lds = ((size_t)(2 * P.small + bf16_pitch(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
+        const size_t lds = ((size_t)(2 * P.small + bf16_valid(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
