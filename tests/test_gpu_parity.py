@@ -304,3 +304,69 @@ def test_properties_at_scale(gpu, orc):
     gd3 = dist.cpu().numpy()
     assert (gd3.max(1) <= before).all()
     assert rows_have_no_duplicates(idx.cpu().numpy())
+
+
+# ---------------------------------------------------------------------------
+# inputs chosen to stress the bfloat16 screens (tree side test, exploration)
+# ---------------------------------------------------------------------------
+def _hard_inputs(rng, kind, N, D):
+    if kind == "offset":          # large common offset: bfloat16 keeps almost nothing of the differences
+        return (1000.0 + rng.random((N, D))).astype(np.float32)
+    if kind == "grid":            # coarse lattice: many points exactly on bisecting hyperplanes, many equal distances
+        return rng.integers(0, 4, size=(N, D)).astype(np.float32)
+    if kind == "tiny":            # values near the bottom of the normal range
+        return (rng.random((N, D)) * 1e-30).astype(np.float32)
+    if kind == "mixed":           # wildly different scales per dimension, both signs
+        scale = np.logspace(-6, 6, D).astype(np.float32)
+        return (rng.standard_normal((N, D)) * scale).astype(np.float32)
+    if kind == "clusters":        # tight clusters: candidate distances crowd around the row maximum
+        centres = rng.random((20, D))
+        return (centres[rng.integers(20, size=N)] + 1e-3 * rng.standard_normal((N, D))).astype(np.float32)
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["offset", "grid", "tiny", "mixed", "clusters"])
+def test_screens_never_change_a_result(gpu, orc, rng, kind):
+    """The bfloat16 screens only skip work whose outcome is certain: trees, bucket K-NN and exploration on inputs
+    that defeat a 8-bit mantissa must still be identical to the fp32 oracle."""
+    import gpu_rsfk
+    N, D, K = 6000, 24, 10
+    X = _hard_inputs(rng, kind, N, D)
+    _say("hard tree", kind)
+    perm, ls, lz, st = orc.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
+    gperm, gls, glz, gst = gpu.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
+    assert np.array_equal(gperm, perm) and np.array_equal(glz, lz)
+    _say("hard forest", kind)
+    r = gpu_rsfk.RSFK(random_state=2)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=3, max_tree_depth=300, nn_exploring_factor=2)
+    oi, od = orc.forest(X, K, 3, K + 1, 2 * (K + 1), 300, 2, 2)
+    if kind == "grid":
+        # equal distances everywhere: which of several tied neighbours survives is arrival order; exploration then
+        # walks different (equally good) neighbours, so only the distance profile of each row is comparable
+        from util import sort_rows
+        assert np.array_equal(sort_rows(gi, gd)[1][:, :1], sort_rows(oi, od)[1][:, :1])
+        assert rows_have_no_duplicates(gi) and (gi >= 0).all()
+        for p in rng.choice(N, 60, replace=False):
+            for k in range(K):
+                assert gd[p, k] == orc.sqdist(X[p], X[gi[p, k]])
+    else:
+        assert_knn_equal(gi, gd, oi, od)
+
+
+def test_rows_come_back_sorted_and_unsorted_input_is_accepted(gpu, orc, rng):
+    """Rows handed in unsorted (the reference keeps them unordered) are merged correctly; rows come back ascending."""
+    N, D, K = 3000, 12, 16
+    X = rng.random((N, D), dtype=np.float32)
+    oi, od = orc.forest(X, K, 2, nnef=0, seed=3)              # oracle rows are in arrival order (unsorted)
+    assert (np.diff(od, axis=1) < 0).any()
+    gi, gd = oi.copy(), od.copy()
+    perm, ls, lz, _ = orc.build_tree(X, K + 1, 2 * (K + 1), 5000, 77)
+    orc.bucket_knn(X, K, perm, lz, oi, od, starts=ls)
+    _say("unsorted rows in")
+    gpu.bucket_knn(X, K, perm, lz, gi, gd, starts=ls)
+    assert_knn_equal(gi, gd, oi, od)
+    changed = (np.sort(gi, 1) != np.sort(oi.copy(), 1)).any(1)     # rows identical as sets
+    assert not changed.any()
+    gi2, gd2 = gi.copy(), gd.copy()
+    gpu.explore(X, K, gi2, gd2, 1)
+    assert (np.diff(gd2, axis=1) >= 0).all()                       # every row ascending after a full pass
