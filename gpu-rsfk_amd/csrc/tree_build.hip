@@ -40,7 +40,7 @@ namespace rsfk {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kHalves = kBlock / 32;     // half wavefronts per workgroup
+constexpr int kGroups = kBlock / 8;      // groups of 8 lanes per workgroup: one point each per iteration
 
 struct LevelCounters {
     int n_next;        // nodes appended for the next wide level
@@ -83,45 +83,75 @@ __device__ __forceinline__ float half_dot(const float* nvec, const float* __rest
     return half_butterfly_sum(s);
 }
 
-// Side of one point (true = right, n.x < b) decided by one half wavefront.
+// Sides of eight points per wavefront (true = right, n.x < b): lanes 8g..8g+7 work on
+// the point of group g; all lanes of a group return its answer.
 //
-// The decision is always the one of the fp32 test above, but most points never
-// touch their fp32 row: a bfloat16 copy of the row (half the bytes) gives an
+// The decision is always the one of the fp32 test above (half_dot), but most points
+// never touch their fp32 row: a bfloat16 copy of the row (half the bytes) gives an
 // approximate n.x together with S~ = sum |n_d||x~_d|.  bfloat16 keeps 8 significant
 // bits: rounding x to x~ (round to nearest) changes n.x by at most
 // 2^-8 sum |n_d||x_d| <= 2^-8 (1+2^-7) S~, and the fp32 summations of either path are
 // off by a few 2^-24 S~, so whenever |approx - b| > 1.02 * 2^-8 S~ the sign of
-// (n.x - b) is the same for the exact fp32 evaluation.  Only the points
-// inside that band (a few per cent) read the fp32 row and repeat the test with
-// the exact arithmetic.  NaN or infinite values fail the band test and take the
-// exact path.
-__device__ __forceinline__ bool side_right(const float* nvec, float b, const float* __restrict__ points,
-                                           const uint16_t* __restrict__ pb16, int Db, int id, int D, int hl,
-                                           bool valid)
+// (n.x - b) is the same for the exact fp32 evaluation.  Only the points inside that
+// band (a few per cent) read the fp32 row and repeat the test with the exact
+// arithmetic, two at a time (one per half wavefront).  NaN or infinite values fail
+// the band test and take the exact path.  Without a bfloat16 copy every point takes
+// the exact path.
+__device__ __forceinline__ bool side_right8(const float* nvec, float b, const float* __restrict__ points,
+                                            const uint16_t* __restrict__ pb16, int id, int D, bool valid)
 {
-    if (pb16 == nullptr) return half_dot(nvec, points + (size_t)id * D, D, hl, valid) < b;
-    const uint32_t* row = reinterpret_cast<const uint32_t*>(pb16 + (size_t)id * (size_t)Db);
-    float da = 0.0f, sa = 0.0f;
-    if (valid) {
-        for (int e = 2 * hl; e < bf16_valid(D); e += 64) {
-            const uint32_t w = row[e >> 1];
-            const float x0 = __uint_as_float(w << 16);
-            const float x1 = __uint_as_float(w & 0xffff0000u);
-            const float2 n = *reinterpret_cast<const float2*>(&nvec[e]);
-            da = __builtin_fmaf(n.x, x0, da);
-            da = __builtin_fmaf(n.y, x1, da);
-            sa = __builtin_fmaf(fabsf(n.x), fabsf(x0), sa);
-            sa = __builtin_fmaf(fabsf(n.y), fabsf(x1), sa);
+    const int lane = lane_id();
+    const int sub = lane & 7;
+    bool right = false;
+    bool redo = valid;
+    if (pb16 != nullptr) {
+        const int Dv = bf16_valid(D);
+        const uint16_t* row = pb16 + (size_t)id * (size_t)bf16_pitch(D);
+        float da = 0.0f, sa = 0.0f;
+        if (valid) {
+            for (int e = sub * 8; e < Dv; e += 64) {
+                const uint4 w = *reinterpret_cast<const uint4*>(row + e);
+                const float4 n0 = *reinterpret_cast<const float4*>(&nvec[e]);
+                const float4 n1 = *reinterpret_cast<const float4*>(&nvec[e + 4]);
+                const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+                const float nn[8] = {n0.x, n0.y, n0.z, n0.w, n1.x, n1.y, n1.z, n1.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float x0 = __uint_as_float(ww[q] << 16);
+                    const float x1 = __uint_as_float(ww[q] & 0xffff0000u);
+                    da = __builtin_fmaf(nn[2 * q], x0, da);
+                    da = __builtin_fmaf(nn[2 * q + 1], x1, da);
+                    sa = __builtin_fmaf(fabsf(nn[2 * q]), fabsf(x0), sa);
+                    sa = __builtin_fmaf(fabsf(nn[2 * q + 1]), fabsf(x1), sa);
+                }
+            }
         }
+        // sum over the 8 lanes of the group (any order will do for the screen)
+        da += dpp_f<kDppXor1>(da); da += dpp_f<kDppXor2>(da); da += dpp_f<kDppHalfMirror>(da);
+        sa += dpp_f<kDppXor1>(sa); sa += dpp_f<kDppXor2>(sa); sa += dpp_f<kDppHalfMirror>(sa);
+        const bool certain = fabsf(da - b) > sa * (1.02f / 256.0f) + 1e-30f;
+        right = da < b;
+        redo = valid && !certain;
     }
-    da = half_butterfly_sum(da);
-    sa = half_butterfly_sum(sa);
-    const bool certain = fabsf(da - b) > sa * (1.02f / 256.0f) + 1e-30f;
-    bool right = da < b;
-    const bool redo = valid && !certain;
-    if (ballot64(redo) != 0) {
-        const float dot = half_dot(nvec, points + (size_t)id * D, D, hl, redo);
-        if (redo) right = dot < b;
+    // exact test for the groups that need it, two per round (one per half wavefront)
+    uint64_t m = ballot64(redo);
+    while (m != 0) {
+        const int g1 = first_lane(m) >> 3;
+        m &= ~(0xffull << (8 * g1));
+        int g2 = -1;
+        if (m != 0) {
+            g2 = first_lane(m) >> 3;
+            m &= ~(0xffull << (8 * g2));
+        }
+        const int id1 = read_lane_i(id, 8 * g1);
+        const int id2 = g2 >= 0 ? read_lane_i(id, 8 * g2) : id1;
+        const bool upper = lane >= 32;
+        const int my = upper ? id2 : id1;
+        const bool live = upper ? g2 >= 0 : true;
+        const float dot = half_dot(nvec, points + (size_t)my * D, D, lane & 31, live);
+        const uint64_t res = ballot64(dot < b);
+        if ((lane >> 3) == g1) right = (res & 1ull) != 0;
+        if (g2 >= 0 && (lane >> 3) == g2) right = ((res >> 32) & 1ull) != 0;
     }
     return right;
 }
@@ -267,19 +297,20 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     const float b = b_s;
     const int pos0 = nd.start + k * P.chunk;
     const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
-    const int half = threadIdx.x >> 5, hl = threadIdx.x & 31;
-    const int iters = (pos1 - pos0 + kHalves - 1) / kHalves;
+    const int grp = threadIdx.x >> 3, sub8 = threadIdx.x & 7;      // 32 groups of 8 lanes, one point each
+    const int iters = (pos1 - pos0 + kGroups - 1) / kGroups;
     int lefts = 0;
     for (int it = 0; it < iters; ++it) {
-        const int pos = pos0 + it * kHalves + half;
+        const int pos = pos0 + it * kGroups + grp;
         const bool valid = pos < pos1;
         const int id = valid ? (perm[pos] & kIdMask) : 0;
-        const bool right = side_right(nvec, b, points, pb16, bf16_pitch(P.D), id, P.D, hl, valid);   // build_tree_check_points_side.cu:149
-        if (valid && hl == 0) {
+        const bool right = side_right8(nvec, b, points, pb16, id, P.D, valid);   // build_tree_check_points_side.cu:149
+        if (valid && sub8 == 0) {
             perm[pos] = right ? (id | (int)0x80000000) : id;
             lefts += right ? 0 : 1;
         }
     }
+    const int hl = sub8;
     if (hl == 0 && lefts) atomicAdd(&left_s, lefts);
     __syncthreads();
     if (threadIdx.x == 0) chunk_left[c] = left_s;
@@ -428,7 +459,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     }
     __syncthreads();
 
-    const int half = tid >> 5, hl = tid & 31;
+    const int hl = tid & 7;                 // lane within its group of 8
     while (true) {
         const int top = top_s;
         if (top == 0) break;
@@ -449,13 +480,13 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
         __syncthreads();
         const float b = b_s;
-        const int iters = (nd.count + kHalves - 1) / kHalves;
+        const int iters = (nd.count + kGroups - 1) / kGroups;
         int lefts = 0;
         for (int it = 0; it < iters; ++it) {
-            const int i = it * kHalves + half;
+            const int i = it * kGroups + (tid >> 3);
             const bool valid = i < nd.count;
             const int id = valid ? seg[nd.start + i] : 0;
-            const bool right = side_right(nvec, b, points, pb16, bf16_pitch(P.D), id, P.D, hl, valid);
+            const bool right = side_right8(nvec, b, points, pb16, id, P.D, valid);
             if (valid && hl == 0) {
                 if (right) seg[nd.start + i] = id | (int)0x80000000; else ++lefts;
             }
