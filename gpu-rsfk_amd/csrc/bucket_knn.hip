@@ -171,26 +171,13 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
     }
 }
 
-// Host launcher.  All pointers are device pointers.  max_bucket: size of the
-// largest bucket if known, otherwise -1.
-int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
-                      const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
-                      hipStream_t stream)
+namespace {
+
+int launch_general(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
+                   int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream)
 {
-    (void)N;
     if (n_buckets <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
-    RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
-    dim3 grid((unsigned)n_buckets);
-    int skip_upto = 0;
-    if (K <= 64) {
-        // buckets of up to 64 points go to the specialised kernel; the general one skips them
-        if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, knn_idx, knn_dist, stream))
-            return 1;
-        if (max_bucket >= 0 && max_bucket <= small_bucket_cap()) return 0;
-        skip_upto = small_bucket_cap();
-    }
-    dim3 block(256);
+    dim3 grid((unsigned)n_buckets), block(256);
     if (K <= 64)
         hipLaunchKernelGGL(k_bucket_knn<1>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx, knn_dist);
     else if (K <= 128)
@@ -199,6 +186,47 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
         hipLaunchKernelGGL(k_bucket_knn<4>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx, knn_dist);
     RSFK_HIP(hipGetLastError());
     return 0;
+}
+
+}  // namespace
+
+// Host launcher for an arbitrary list of buckets.  All pointers are device pointers.  max_bucket: size of
+// the largest bucket if known, otherwise -1.
+int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
+                      const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
+                      hipStream_t stream)
+{
+    (void)N;
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
+    RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    int skip_upto = 0;
+    if (K <= 64) {
+        // buckets of up to 64 points go to the specialised kernel; the general one skips them
+        if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, knn_idx, knn_dist, stream))
+            return 1;
+        if (max_bucket >= 0 && max_bucket <= small_bucket_cap()) return 0;
+        skip_upto = small_bucket_cap();
+    }
+    return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream);
+}
+
+// Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
+// (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.
+int launch_bucket_knn_tree(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist, hipStream_t stream)
+{
+    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
+    RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    if (n_small > 0) {
+        if (K <= 64) {
+            if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
+        } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream)) {
+            return 1;
+        }
+    }
+    const int off = leaf_cap - n_big;
+    return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, 0, knn_idx, knn_dist, stream);
 }
 
 }  // namespace rsfk

@@ -29,7 +29,8 @@ namespace rsfk {
 
 namespace {
 
-constexpr int kCap = 64;                    // largest bucket this kernel takes
+constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
+static_assert(kCap == 64, "lane-per-candidate merge and 64-bit presence masks assume 64");
 constexpr int kThreads = 128;
 constexpr int kWaves = kThreads / 64;
 constexpr int kRowsPerWave = kCap / kWaves;

@@ -54,7 +54,7 @@ RSFK_API void pymodule_cluster_by_sample_tree(int N, int D, int MIN_TREE_CHILD, 
 {
     const auto t0 = std::chrono::steady_clock::now();
     std::vector<int> perm, ls, lz;
-    int stats[4] = {0, 0, 0, 0};
+    int stats[5] = {0, 0, 0, 0, 0};
     {
         DevMem dp;
         if (N < 1 || D < 1) { set_last_error("N and D must be positive"); die("pymodule_cluster_by_sample_tree"); }
@@ -138,7 +138,7 @@ RSFK_API int rsfk_build_tree_host(const float* points, int N, int D, int MIN_TRE
         return -1;
     }
     std::vector<int> pv, ls, lz;
-    int st[4];
+    int st[5];
     if (build_tree_host(static_cast<const float*>(dp.p), N, D, MIN_TREE_CHILD, MAX_TREE_CHILD, MAX_DEPTH,
                         RANDOM_STATE, pv, ls, lz, st))
         return -1;
@@ -146,7 +146,7 @@ RSFK_API int rsfk_build_tree_host(const float* points, int N, int D, int MIN_TRE
     std::memcpy(perm, pv.data(), sizeof(int) * (size_t)N);
     std::memcpy(leaf_start, ls.data(), sizeof(int) * ls.size());
     std::memcpy(leaf_size, lz.data(), sizeof(int) * lz.size());
-    if (stats) std::memcpy(stats, st, sizeof(st));
+    if (stats) std::memcpy(stats, st, sizeof(int) * 4);
     return st[0];
 }
 

@@ -86,7 +86,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         const int B = choose_batch(n_trees, N, D, MIN);
         WsGuard ws;
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
-        std::vector<int> stats((size_t)4 * B);
+        std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
         for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
         int rc = 0;
@@ -98,8 +98,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             const double tb = now_s() - tb0;
             for (int j = 0; j < nb && rc == 0; ++j) {
                 (void)hipEventRecord(ev[j].a, stream);
-                rc = launch_bucket_knn(d_points, N, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
-                                       tree_ws_leaf_size(ws.w, j), stats[4 * j], 0, stats[4 * j + 2], d_idx, d_dist, stream);
+                rc = launch_bucket_knn_tree(d_points, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                                            tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w),
+                                            stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], d_idx, d_dist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
             }
             if (rc) break;
@@ -109,16 +110,16 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 (void)hipEventElapsedTime(&ms, ev[j].a, ev[j].b);
                 const int t = t0 + j;
                 if (log_forest) {
-                    log_forest[(size_t)0 * n_trees + t] = (float)stats[4 * j + 1];   // Tree Depth
-                    log_forest[(size_t)1 * n_trees + t] = (float)stats[4 * j + 2];   // Max Leaf Size
-                    log_forest[(size_t)2 * n_trees + t] = (float)stats[4 * j + 3];   // Min Leaf Size
-                    log_forest[(size_t)3 * n_trees + t] = (float)stats[4 * j + 0];   // Total Leaves
+                    log_forest[(size_t)0 * n_trees + t] = (float)stats[5 * j + 1];   // Tree Depth
+                    log_forest[(size_t)1 * n_trees + t] = (float)stats[5 * j + 2];   // Max Leaf Size
+                    log_forest[(size_t)2 * n_trees + t] = (float)stats[5 * j + 3];   // Min Leaf Size
+                    log_forest[(size_t)3 * n_trees + t] = (float)stats[5 * j + 0];   // Total Leaves
                     log_forest[(size_t)5 * n_trees + t] = (float)(tb / nb);          // Total Tree Building Time
                     log_forest[(size_t)15 * n_trees + t] = ms * 1e-3f;               // KNN Sets Updates
                 }
                 if (verbose >= 2)
                     std::printf("tree %d: depth %d, leaves %d, leaf size %d..%d, K-NN update %.6f s\n", t,
-                                stats[4 * j + 1], stats[4 * j + 0], stats[4 * j + 3], stats[4 * j + 2], ms * 1e-3);
+                                stats[5 * j + 1], stats[5 * j + 0], stats[5 * j + 3], stats[5 * j + 2], ms * 1e-3);
             }
         }
         for (auto& e : ev) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
@@ -168,7 +169,7 @@ int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_
 
 // One tree; results on the host.  perm: N ints; leaves sorted by start.
 int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int MAX_DEPTH, int seed,
-                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[4])
+                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[5])
 {
     WsGuard ws;
     if (tree_ws_alloc(&ws.w, N, D, MIN, 1)) return 1;
@@ -176,13 +177,17 @@ int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int M
     if (bf16_copy_alloc(&bf.c, N, D)) return 1;
     if (bf16_copy_fill(bf.c, d_points, N, D, nullptr)) return 1;
     if (build_tree_batch(ws.w, d_points, bf.c.rows, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
-    const int nl = stats[0];
+    const int nl = stats[0], n_big = stats[4], n_small = nl - n_big, cap = tree_ws_leaf_cap(ws.w);
     perm.resize((size_t)N);
     std::vector<int> ls((size_t)nl), lz((size_t)nl);
     RSFK_HIP(hipMemcpy(perm.data(), tree_ws_perm(ws.w, 0), sizeof(int) * (size_t)N, hipMemcpyDeviceToHost));
-    if (nl > 0) {
-        RSFK_HIP(hipMemcpy(ls.data(), tree_ws_leaf_start(ws.w, 0), sizeof(int) * (size_t)nl, hipMemcpyDeviceToHost));
-        RSFK_HIP(hipMemcpy(lz.data(), tree_ws_leaf_size(ws.w, 0), sizeof(int) * (size_t)nl, hipMemcpyDeviceToHost));
+    if (n_small > 0) {
+        RSFK_HIP(hipMemcpy(ls.data(), tree_ws_leaf_start(ws.w, 0), sizeof(int) * (size_t)n_small, hipMemcpyDeviceToHost));
+        RSFK_HIP(hipMemcpy(lz.data(), tree_ws_leaf_size(ws.w, 0), sizeof(int) * (size_t)n_small, hipMemcpyDeviceToHost));
+    }
+    if (n_big > 0) {
+        RSFK_HIP(hipMemcpy(ls.data() + n_small, tree_ws_leaf_start(ws.w, 0) + (cap - n_big), sizeof(int) * (size_t)n_big, hipMemcpyDeviceToHost));
+        RSFK_HIP(hipMemcpy(lz.data() + n_small, tree_ws_leaf_size(ws.w, 0) + (cap - n_big), sizeof(int) * (size_t)n_big, hipMemcpyDeviceToHost));
     }
     std::vector<int> order((size_t)nl);
     for (int i = 0; i < nl; ++i) order[i] = i;

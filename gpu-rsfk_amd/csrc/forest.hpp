@@ -25,6 +25,9 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream);
 
+int launch_bucket_knn_tree(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist, hipStream_t stream);
+
 // bucket_knn_small.hip
 int small_bucket_cap();
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
@@ -41,6 +44,6 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
 int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                     int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest);
 int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int MAX_DEPTH, int seed,
-                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[4]);
+                    std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[5]);
 
 }  // namespace rsfk

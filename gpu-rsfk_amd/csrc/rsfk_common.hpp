@@ -90,6 +90,10 @@ struct TreeNode {
     uint64_t key;
 };
 
+// Buckets of at most this many points are handled by the small-bucket K-NN kernel; the
+// tree builder keeps them apart from the larger ones.
+constexpr int kBucketSplit = 64;
+
 // bit 31 of a permutation entry marks "right side" during a split; ids use the low 31 bits
 constexpr int kIdMask = 0x7fffffff;
 

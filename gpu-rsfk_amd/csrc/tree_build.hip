@@ -393,24 +393,35 @@ struct SmallNode {
 };
 
 struct TreeStats {          // one per tree of the batch
-    int n_leaves;
+    int n_leaves;           // buckets of at most kBucketSplit points, stored from the front of the leaf table
+    int n_big;              // larger buckets, stored from the back of the leaf table
     int levels;
     int max_leaf;
     int min_leaf;
 };
 
+// Entry of the leaf table that the `at`-th bucket of its kind takes: small buckets fill the table of the tree from the
+// front, large ones from the back, so that each kind can be handed to its own kernel as a plain (start, size) array.
+__device__ __forceinline__ void store_leaf(int tree, int gstart, int count, int at, int leaf_cap,
+                                           int* __restrict__ leaf_start, int* __restrict__ leaf_size, LevelCounters* ctr)
+{
+    if (at < leaf_cap) {
+        const int slot = count > kBucketSplit ? leaf_cap - 1 - at : at;
+        leaf_start[(size_t)tree * leaf_cap + slot] = gstart;
+        leaf_size[(size_t)tree * leaf_cap + slot] = count;
+    } else {
+        ctr->overflow = 1;
+    }
+}
+
+// One bucket straight to the table (nodes that became buckets in the wide phase).
 __device__ __forceinline__ void emit_leaf(int tree, int gstart, int count, int depth, int leaf_cap,
                                           int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                           TreeStats* stats, LevelCounters* ctr)
 {
     TreeStats* st = stats + tree;
-    const int at = atomicAdd(&st->n_leaves, 1);
-    if (at < leaf_cap) {
-        leaf_start[(size_t)tree * leaf_cap + at] = gstart;
-        leaf_size[(size_t)tree * leaf_cap + at] = count;
-    } else {
-        ctr->overflow = 1;
-    }
+    const int at = atomicAdd(count > kBucketSplit ? &st->n_big : &st->n_leaves, 1);
+    store_leaf(tree, gstart, count, at, leaf_cap, leaf_start, leaf_size, ctr);
     atomicMax(&st->levels, depth + 1);
     atomicMax(&st->max_leaf, count);
     atomicMin(&st->min_leaf, count);
@@ -424,14 +435,18 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr)
 {
-    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_valid(D)] | stack[stack_cap]
+    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_valid(D)] | stack[stack_cap] | lrec[small]
     extern __shared__ __align__(16) unsigned char lds_raw[];
     int* seg = reinterpret_cast<int*>(lds_raw);
     int* tmp = seg + P.small;
     float* nvec = reinterpret_cast<float*>(tmp + P.small);
     SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + bf16_valid(P.D)) * 4 + 15) / 16 * 16);
+    // buckets of this subtree, written to the table of the tree together at the end (one reservation per
+    // workgroup instead of one atomic round trip per bucket): x = start, y = size | rank among its kind << 16
+    int2* lrec = reinterpret_cast<int2*>(stack + stack_cap);
     __shared__ float b_s;
-    __shared__ int left_s, top_s;
+    __shared__ int left_s, top_s, base_s[2], nrec_s;
+    int n_small = 0, n_big = 0, lev = 0, mx = 0, mn = 0x7fffffff;      // thread 0 only
     __shared__ int wcnt[kBlock / 64];
 
     const int task = blockIdx.x;
@@ -467,7 +482,11 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         __syncthreads();                      // everyone has read the top before it is overwritten
         if (nd.leaf || nd.depth >= P.MAX_DEPTH - 1) {
             if (tid == 0) {
-                emit_leaf(tk.tree, tk.start + nd.start, nd.count, nd.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
+                const int rank = nd.count > kBucketSplit ? n_big++ : n_small++;
+                lrec[n_small + n_big - 1] = make_int2(tk.start + nd.start, nd.count | (rank << 16));
+                lev = max(lev, nd.depth + 1);
+                mx = max(mx, nd.count);
+                mn = min(mn, nd.count);
                 top_s = top - 1;
             }
             __syncthreads();
@@ -537,6 +556,21 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         __syncthreads();
     }
     for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = seg[i];
+    if (tid == 0) {
+        TreeStats* st = stats + tk.tree;
+        base_s[0] = n_small ? atomicAdd(&st->n_leaves, n_small) : 0;
+        base_s[1] = n_big ? atomicAdd(&st->n_big, n_big) : 0;
+        nrec_s = n_small + n_big;
+        atomicMax(&st->levels, lev);
+        atomicMax(&st->max_leaf, mx);
+        atomicMin(&st->min_leaf, mn);
+    }
+    __syncthreads();
+    for (int i = tid; i < nrec_s; i += kBlock) {
+        const int2 r = lrec[i];
+        const int count = r.y & 0xffff, rank = r.y >> 16;
+        store_leaf(tk.tree, r.x, count, base_s[count > kBucketSplit ? 1 : 0] + rank, leaf_cap, leaf_start, leaf_size, ctr);
+    }
 }
 
 template <typename T>
@@ -630,8 +664,9 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
 // Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  pb16 = rows of the bfloat16 copy of the points (may be
 // null: every side test then reads the fp32 row).  On return perm[0] of
 // tree t holds the point ids grouped by bucket and (leaf_start, leaf_size)[t]
-// the buckets, in no particular order.  host_stats receives 4 ints per tree:
-// number of leaves, number of levels, largest and smallest bucket.
+// the buckets, in no particular order: those of at most kBucketSplit points in entries [0, n_small), the
+// larger ones in entries [leaf_cap - n_big, leaf_cap).  host_stats receives 5 ints per tree: number of
+// buckets, number of levels, largest and smallest bucket, number of large buckets.
 int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, int N, int D, int MIN, int MAX,
                      int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream)
 {
@@ -648,7 +683,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         hipLaunchKernelGGL(k_init_perm, dim3(grid), dim3(256), 0, stream, w->perm[0], N, nb);
     }
     std::vector<TreeStats> init((size_t)nb);
-    for (auto& s : init) { s.n_leaves = 0; s.levels = 0; s.max_leaf = 0; s.min_leaf = 0x7fffffff; }
+    for (auto& s : init) { s.n_leaves = 0; s.n_big = 0; s.levels = 0; s.max_leaf = 0; s.min_leaf = 0x7fffffff; }
     std::memcpy(w->h_stats, init.data(), sizeof(TreeStats) * (size_t)nb);
     RSFK_HIP(hipMemcpyAsync(w->stats, w->h_stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyHostToDevice, stream));
     RSFK_HIP(hipMemsetAsync(w->ctr, 0, sizeof(LevelCounters), stream));
@@ -685,7 +720,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
     if (n_tail > 0) {
         const int stack_cap = P.small / std::max(MIN, 1) + 4;
-        const size_t lds = ((size_t)(2 * P.small + bf16_valid(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode);
+        const size_t lds = ((size_t)(2 * P.small + bf16_valid(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode) + (size_t)P.small * sizeof(int2);
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
@@ -697,11 +732,13 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_HIP(hipStreamSynchronize(stream));
     RSFK_CHECK(!w->h_ctr->overflow, "tree batch: queue overflow in the tail phase");
     for (int t = 0; t < nb; ++t) {
-        host_stats[4 * t + 0] = w->h_stats[t].n_leaves;
-        host_stats[4 * t + 1] = w->h_stats[t].levels;
-        host_stats[4 * t + 2] = w->h_stats[t].max_leaf;
-        host_stats[4 * t + 3] = w->h_stats[t].n_leaves ? w->h_stats[t].min_leaf : 0;
-        RSFK_CHECK(w->h_stats[t].n_leaves <= w->leaf_cap, "tree batch: leaf table overflow");
+        const int total = w->h_stats[t].n_leaves + w->h_stats[t].n_big;
+        host_stats[5 * t + 0] = total;
+        host_stats[5 * t + 1] = w->h_stats[t].levels;
+        host_stats[5 * t + 2] = w->h_stats[t].max_leaf;
+        host_stats[5 * t + 3] = total ? w->h_stats[t].min_leaf : 0;
+        host_stats[5 * t + 4] = w->h_stats[t].n_big;
+        RSFK_CHECK(total <= w->leaf_cap, "tree batch: leaf table overflow");
     }
     return 0;
 }
