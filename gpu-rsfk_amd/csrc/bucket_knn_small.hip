@@ -10,13 +10,10 @@
 //      accumulates its 16 distances with sequential fused multiply-add chains
 //      (arithmetic of euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
 //      the 6 pairs inside each diagonal block are done one per thread;
-//   3. "already in the row" is answered for all rows at once with a hash table of
-//      the bucket's ids in LDS (two probes, branch-free in the common case) and
-//      kept as a 64-bit mask per point;
-//   4. the distance matrix replaces the rows in LDS; a wavefront owns every second
+//   3. the distance matrix replaces the rows in LDS; a wavefront owns every second
 //      point: per point, the candidates that are closer than the row's last slot
-//      and not in the mask are inserted into the sorted row (knn_list.hpp); the
-//      rows of the next two points are in flight meanwhile.
+//      are inserted into the sorted row unless the row holds them already
+//      (knn_list.hpp); the rows of the next two points are in flight meanwhile.
 // Registers are kept near 100 and LDS near 20 KB per workgroup so that four
 // wavefronts per SIMD are resident: the kernel alternates between an arithmetic
 // phase and a latency-bound merge phase, and only other resident workgroups can
@@ -33,19 +30,11 @@ constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
 static_assert(kCap == 64, "lane-per-candidate merge and 64-bit presence masks assume 64");
 constexpr int kThreads = 128;
 constexpr int kWaves = kThreads / 64;
-constexpr int kRowsPerWave = kCap / kWaves;
-constexpr int kHash = 256;                  // open-addressing table of the bucket's ids
 constexpr int kSpacing = 17;                // LDS rows between members 4t, 4t+1, 4t+2, 4t+3
 constexpr int kLdsRows = 15 + 3 * kSpacing + 1;
 constexpr int kDistPitch = kCap + 1;
 constexpr int kMaxChunk = 64;               // dimensions staged at once
 constexpr int kMaxLoads = kCap * (kMaxChunk / 4) / kThreads;   // 16-byte loads per thread and chunk
-
-__device__ __forceinline__ uint32_t bucket_hash(int id)
-{
-    uint32_t h = (uint32_t)id * 0x9E3779B1u;
-    return (h ^ (h >> 15)) & (kHash - 1);
-}
 
 // LDS row of bucket member m: the 4x4 block of thread t reads rows t, t+17, t+34,
 // t+51 -- consecutive t give conflict-free 16-byte reads (the pitch is an odd
@@ -59,13 +48,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
                                                                   int* __restrict__ knn_idx, float* __restrict__ knn_dist,
                                                                   int chunk, int pitch, int region_floats)
 {
-    // dynamic LDS: [rows | dist] (region_floats) | ids[64] | table[256] | present[64][2]
+    // dynamic LDS: [rows | dist] (region_floats) | ids[64]
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
     float* dist = lds_f;                     // same storage, used after the last read of rows
     int* lids = reinterpret_cast<int*>(lds_f + region_floats);
-    int* table = lids + kCap;
-    uint32_t* present = reinterpret_cast<uint32_t*>(table + kHash);
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
@@ -74,20 +61,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
-    table[tid] = -1;
-    table[tid + kThreads] = -1;
-    present[tid] = 0;
     if (tid < kCap) lids[tid] = tid < s ? bid[tid] : -1;
     __syncthreads();
-
-    // hash table of the bucket
-    if (tid < s) {
-        uint32_t h = bucket_hash(lids[tid]);
-        for (int probe = 0; probe < kHash; ++probe) {
-            if (atomicCAS(&table[h], -1, tid) == -1) break;
-            h = (h + 1) & (kHash - 1);
-        }
-    }
 
     // work assignment: off-diagonal 4x4 blocks (ti < tj) one per thread, then the 6 pairs of each diagonal block
     const int n = (s + 3) >> 2;
@@ -200,52 +175,12 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
         }
     }
 
-    // Which members of the bucket does each row already hold?  All lookups of the wavefront
-    // are independent: two probes each without branching, a loop only for the rare longer run.
-    // present[i] is touched by the owning wavefront only.
-    bool unsorted = false;
-#pragma unroll
-    for (int u = 0; u < kRowsPerWave; ++u) {
-        const int i = wave + kWaves * u;
-        int mine = -2;
-        float mined = INFINITY;
-        if (i < s && lane < K) {
-            const size_t at = (size_t)lids[i] * (size_t)K + lane;
-            mine = knn_idx[at];
-            mined = knn_dist[at];
-        }
-        const bool want = i < s && mine >= 0;
-        const uint32_t h = bucket_hash(mine);
-        const int e0 = table[h], e1 = table[(h + 1) & (kHash - 1)];
-        const int id0 = lids[e0 < 0 ? 0 : e0], id1 = lids[e1 < 0 ? 0 : e1];
-        int hit = -1;
-        if (want && e0 >= 0) {
-            if (id0 == mine) hit = e0;
-            else if (e1 >= 0) {
-                if (id1 == mine) hit = e1;
-                else {
-                    uint32_t hh = (h + 2) & (kHash - 1);
-                    for (int probe = 2; probe < kHash; ++probe) {
-                        const int e = table[hh];
-                        if (e < 0) break;
-                        if (lids[e] == mine) { hit = e; break; }
-                        hh = (hh + 1) & (kHash - 1);
-                    }
-                }
-            }
-        }
-        if (hit >= 0) atomicOr(&present[2 * i + (hit >> 5)], 1u << (hit & 31));
-        // rows must be sorted by distance; anything else is rebuilt below
-        unsorted |= mined < wave_shr1_f(mined);
-    }
-    const bool any_unsorted = ballot64(unsorted) != 0;
-    __syncthreads();                           // distance matrix and present[] complete
+    __syncthreads();                           // distance matrix complete
 
     // top-K update, one member at a time per wavefront; the LDS reads of the next member are
     // issued before the current one is merged
     const int my_id = lids[lane];
     float d_next = dist[wave * kDistPitch + lane];
-    uint32_t f_next = present[2 * wave + (lane >> 5)];
     auto load_row = [&](int i, int& ri, float& rd) {
         ri = -2;
         rd = INFINITY;
@@ -262,18 +197,13 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
     for (int i = wave; i < s; i += kWaves) {
         load_row(i + 2 * kWaves, ri2, rd2);
         const float d = d_next;
-        const bool held = (f_next >> (lane & 31)) & 1u;
-        if (i + kWaves < s) {
-            d_next = dist[(i + kWaves) * kDistPitch + lane];
-            f_next = present[2 * (i + kWaves) + (lane >> 5)];
-        }
+        if (i + kWaves < s) d_next = dist[(i + kWaves) * kDistPitch + lane];
         KnnRow<1> row;
         row.idx[0] = ri0;
         row.dist[0] = rd0;
         ri0 = ri1; rd0 = rd1; ri1 = ri2; rd1 = rd2;
-        if (any_unsorted) row.init_from_regs(K); else row.init_sorted(K);
-        const bool ok = lane < s && lane != i && !held;
-        row.offer_lanes<false>(ok, my_id, d);
+        row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
+        row.offer_lanes<true>(lane < s && lane != i, my_id, d);
         if (row.changed) {
             const size_t at = (size_t)lids[i] * (size_t)K;
             row.store(knn_idx + at, knn_dist + at);
@@ -296,7 +226,7 @@ int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, c
     if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units
     const int region = std::max(kLdsRows * pitch, kCap * kDistPitch);
     const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)(kCap + kHash + 2 * kCap) * 4;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)kCap * 4;
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_small),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k_bucket_knn_small, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, D, K, ids,
