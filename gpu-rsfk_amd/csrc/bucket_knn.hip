@@ -212,14 +212,18 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 }
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
-// (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.
-int launch_bucket_knn_tree(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
-                           int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist, hipStream_t stream)
+// (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  bf: bfloat16 copy of the
+// points if the rows are known to be sorted by distance (then the small buckets take the screened kernel), else null.
+int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, int D, int K, const int* ids, const int* starts,
+                           const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist,
+                           hipStream_t stream)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
     if (n_small > 0) {
-        if (K <= 64) {
+        if (K <= 64 && bf != nullptr) {
+            if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;
+        } else if (K <= 64) {
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream)) {
             return 1;

@@ -1,0 +1,355 @@
+// Bucket K-NN for buckets of at most 64 points and K <= 64 when a bfloat16 copy of
+// the points exists: same function and same results as the kernel in
+// bucket_knn_small.hip (see bucket_knn.hip for the reference kernels both replace),
+// but most pair distances are never computed.
+//
+// A pair (i, j) of a bucket changes nothing unless its distance is smaller than
+// the last slot of row i or of row j.  After the first few trees that holds for a
+// small fraction of the pairs, so the kernel first bounds every pair from below:
+//
+//   1. Gram matrix of the bucket's bfloat16 rows with the matrix cores
+//      (v_mfma_f32_32x32x16_bf16, operands straight from global memory, one to
+//      three 32x32 tiles): d~ = n_i + n_j - 2 G_ij approximates the distance, and
+//      a bound E on |d~ - exact fp32 result| follows from the norms alone
+//      (bfloat16 rounding: 2u sqrt(d~ Q) + u^2 Q with u = 2^-8 and Q = 2 (n_i + n_j),
+//      by Cauchy-Schwarz; accumulation errors of the Gram matrix, the norms and the
+//      fp32 chain are relative to n_i + n_j resp. to the distance).  Pairs with
+//      d~ - E >= max(last slot of row i, last slot of row j) are dropped; this never
+//      drops a pair that the exact arithmetic would have inserted;
+//   2. the remaining pairs go to a list in LDS; the fp32 rows are staged through LDS
+//      in slices of at most 48 dimensions and each thread runs the sequential fused
+//      multiply-add chains (arithmetic of euclidean_distance_sqr,
+//      compute_knn_from_buckets.cu:40-54) of its pairs of the list;
+//   3. the exact distances land in a triangular matrix in LDS (+inf elsewhere) and
+//      the rows are updated as in the other kernel; rows without any candidate below
+//      their last slot are neither read nor written.
+//
+// Requires every K-NN row to be sorted by distance on entry (the last slot is the
+// maximum); launch_sort_rows establishes that once per build.
+#include "rsfk_common.hpp"
+#include "knn_list.hpp"
+#include "forest.hpp"
+
+namespace rsfk {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
+static_assert(kCap == 64, "two 32-row operand halves and lane-per-candidate merge assume 64");
+constexpr int kThreads = 128;
+constexpr int kWaves = kThreads / 64;
+constexpr int kMaxChunk = 48;               // dimensions staged at once
+constexpr int kMaxLoads = kCap * (kMaxChunk / 4) / kThreads;   // 16-byte loads per thread and slice
+constexpr int kMaxPairs = kCap * (kCap - 1) / 2;
+constexpr int kPairsPerThread = (kMaxPairs + kThreads - 1) / kThreads;
+
+constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16 (8 significant bits)
+
+// entry of pair (a, b), a < b, in the triangular matrix
+__device__ __forceinline__ int tri_at(int a, int b) { return ((b * (b - 1)) >> 1) + a; }
+
+// Screen one 32x32 tile of the Gram matrix.  Accumulator i of lane l belongs to row member
+// m = mbase + 8 (i / 4) + i % 4 (mbase = first member of the operand half + 4 (l / 32)) and column
+// member n.  Returns the mask of accumulators whose pair (m < n < s) must be computed exactly.
+__device__ __forceinline__ uint32_t screen_tile(const f32x16& g, int mbase, int n, int s, const float* nrm, const float* tau,
+                                                float kappa, float one_minus_gamma)
+{
+    const float nn = nrm[n], tn = tau[n];
+    uint32_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int m = mbase + 8 * (i >> 2) + (i & 3);
+        const float S = nrm[m] + nn;
+        const float limit = fmaxf(tau[m], tn);
+        const float dt = __builtin_fmaf(-2.0f, g[i], S);            // distance of the bfloat16 rows
+        const float e1 = kappa * S;                                 // accumulation errors of G and the norms
+        const float dhi = fmaxf(dt + e1, 0.0f);
+        const float Q = 2.0001f * S;
+        const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);   // rounding to bfloat16
+        const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;                 // <= result of the fp32 chain
+        const bool skip = lower >= limit;                           // false if anything is NaN
+        if (m < n && n < s && !skip) bits |= 1u << i;
+    }
+    return bits;
+}
+
+__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* __restrict__ points,
+                                                                   const uint16_t* __restrict__ brows,
+                                                                   const float* __restrict__ bnorms, int D, int K,
+                                                                   const int* __restrict__ ids,
+                                                                   const int* __restrict__ starts,
+                                                                   const int* __restrict__ sizes,
+                                                                   int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                                   int chunk, int pitch, int region_floats, int bpitch,
+                                                                   int ksteps, float kappa, float one_minus_gamma)
+{
+    // dynamic LDS: [rows | triangular distance matrix] (region_floats) | ids[64] | tau[64] | nrm[64] | n_pairs | list
+    extern __shared__ __align__(16) float lds_f[];
+    float* rows = lds_f;
+    float* tri = lds_f;                      // same storage, used after the last read of rows
+    int* lids = reinterpret_cast<int*>(lds_f + region_floats);
+    float* tau = reinterpret_cast<float*>(lids + kCap);
+    float* nrm = tau + kCap;
+    int* n_pairs = reinterpret_cast<int*>(nrm + kCap);
+    uint16_t* list = reinterpret_cast<uint16_t*>(n_pairs + 4);
+
+    const int bkt = blockIdx.x;
+    const int s = sizes[bkt];
+    if (s < 2 || s > kCap) return;
+    const int* bid = ids + (size_t)starts[bkt];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+
+    if (tid < kCap) {
+        const int id = tid < s ? bid[tid] : -1;
+        lids[tid] = id;
+        tau[tid] = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
+        nrm[tid] = id >= 0 ? bnorms[id] : 0.0f;
+    }
+    if (tid == 0) *n_pairs = 0;
+    __syncthreads();
+
+    // fp32 rows of a slice: requested early, written to LDS when the previous slice has been consumed
+    float4 pre[kMaxLoads];
+    auto request = [&](int d0) {
+        const int np = min(chunk, (D - d0 + 3) & ~3) >> 2;      // 16-byte pieces per row in this slice
+        const int items = s * np;
+#pragma unroll
+        for (int i = 0; i < kMaxLoads; ++i) {
+            const int it = tid + i * kThreads;
+            pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (it < items) {
+                const int m = it / np, pc = it - m * np;
+                const float* src = points + (size_t)lids[m] * (size_t)D + d0 + 4 * pc;
+                if (vec_ok) {
+                    pre[i] = *reinterpret_cast<const float4*>(src);
+                } else {
+                    const int left = D - d0 - 4 * pc;
+                    pre[i].x = src[0];
+                    if (left > 1) pre[i].y = src[1];
+                    if (left > 2) pre[i].z = src[2];
+                    if (left > 3) pre[i].w = src[3];
+                }
+            }
+        }
+        return np;
+    };
+    int np = request(0);
+
+    // ---- 1. screen: wavefront 0 takes the tiles (half 0 x half 0) and (half 0 x half 1), wavefront 1 the
+    //         tile (half 1 x half 1); members beyond s read the row of member 0 and are ignored
+    {
+        const bool two_halves = s > 32;
+        const int hx = wave;                                     // operand half of this wavefront's first tile
+        if (hx == 0 || two_halves) {
+            const int mx = 32 * hx + (lane & 31), my = 32 + (lane & 31);
+            const uint16_t* rx = brows + (size_t)lids[mx < s ? mx : 0] * (size_t)bpitch + 8 * (lane >> 5);
+            const uint16_t* ry = brows + (size_t)lids[my < s ? my : 0] * (size_t)bpitch + 8 * (lane >> 5);
+            const bool second = hx == 0 && two_halves;
+            f32x16 gxx, gxy;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { gxx[i] = 0.0f; gxy[i] = 0.0f; }
+            for (int k0 = 0; k0 < ksteps; k0 += 4) {
+                bf16x8 x[4], y[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (k0 + u < ksteps) {
+                        x[u] = *reinterpret_cast<const bf16x8*>(rx + 16 * (k0 + u));
+                        if (second) y[u] = *reinterpret_cast<const bf16x8*>(ry + 16 * (k0 + u));
+                        else y[u] = x[u];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (k0 + u < ksteps) {
+                        gxx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], x[u], gxx, 0, 0, 0);
+                        if (second) gxy = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], y[u], gxy, 0, 0, 0);
+                    }
+                }
+            }
+            const int mbase = 32 * hx + 4 * (lane >> 5);
+            for (int t = 0; t < (second ? 2 : 1); ++t) {
+                const int n = t == 0 ? mx : my;
+                uint32_t bits = screen_tile(t == 0 ? gxx : gxy, mbase, n, s, nrm, tau, kappa, one_minus_gamma);
+                const int cnt = __popc(bits);
+                int at = cnt ? atomicAdd(n_pairs, cnt) : 0;
+                while (bits) {
+                    const int i = __ffs(bits) - 1;
+                    bits &= bits - 1;
+                    const int m = mbase + 8 * (i >> 2) + (i & 3);
+                    list[at++] = (uint16_t)(m | (n << 6));
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int n_list = *n_pairs;
+    const int rounds = (n_list + kThreads - 1) / kThreads;      // pairs per thread, at most kPairsPerThread
+
+    // ---- 2. exact distances of the listed pairs
+    uint32_t where[kPairsPerThread];          // LDS offsets of the two rows of a pair, 16 bits each
+    float acc[kPairsPerThread];
+#pragma unroll
+    for (int k = 0; k < kPairsPerThread; ++k) {
+        const int p = tid + k * kThreads;
+        const uint32_t e = p < n_list ? list[p] : 0u;
+        where[k] = ((e & 63u) * (uint32_t)pitch) | (((e >> 6) * (uint32_t)pitch) << 16);
+        acc[k] = 0.0f;
+    }
+    for (int d0 = 0; d0 < D; d0 += chunk) {
+        if (d0 > 0) __syncthreads();                 // the previous slice has been consumed
+        const int items = s * np;
+#pragma unroll
+        for (int i = 0; i < kMaxLoads; ++i) {
+            const int it = tid + i * kThreads;
+            if (it < items) {
+                const int m = it / np, pc = it - m * np;
+                *reinterpret_cast<float4*>(&rows[m * pitch + 4 * pc]) = pre[i];
+            }
+        }
+        const int np_now = np;
+        if (d0 + chunk < D) np = request(d0 + chunk);
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < kPairsPerThread; ++k) {
+            if (k < rounds) {
+                const float* ra = rows + (where[k] & 0xffffu);
+                const float* rb = rows + (where[k] >> 16);
+                float a = acc[k];
+                for (int q = 0; q < np_now; ++q) {
+                    const float4 x = *reinterpret_cast<const float4*>(ra + 4 * q);
+                    const float4 y = *reinterpret_cast<const float4*>(rb + 4 * q);
+                    float df;
+                    df = x.x - y.x; a = __builtin_fmaf(df, df, a);
+                    df = x.y - y.y; a = __builtin_fmaf(df, df, a);
+                    df = x.z - y.z; a = __builtin_fmaf(df, df, a);
+                    df = x.w - y.w; a = __builtin_fmaf(df, df, a);
+                }
+                acc[k] = a;
+            }
+        }
+    }
+    __syncthreads();                           // rows no longer needed: the region becomes the distance matrix
+    const int n_tri = (s * (s - 1)) >> 1;
+    for (int i = tid; i < n_tri; i += kThreads) tri[i] = INFINITY;
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < kPairsPerThread; ++k) {
+        const int p = tid + k * kThreads;
+        if (p < n_list) {
+            const uint32_t e = list[p];
+            tri[tri_at((int)(e & 63u), (int)(e >> 6))] = acc[k];
+        }
+    }
+    __syncthreads();
+
+    // ---- 3. top-K update.  A wavefront owns every second member; first find the members that have a
+    //         candidate below their last slot, then walk those with the rows of the next two in flight.
+    const int my_id = lids[lane];
+    auto candidate = [&](int i) {
+        const int a = min(i, lane), b = max(i, lane);
+        return (lane < s && lane != i) ? tri[tri_at(a, b)] : INFINITY;
+    };
+    uint32_t active = 0;
+    for (int u = 0; wave + kWaves * u < s; ++u) {
+        const int i = wave + kWaves * u;
+        if (ballot64(candidate(i) < tau[i]) != 0) active |= 1u << u;
+    }
+    auto next_member = [&]() {
+        if (active == 0) return -1;
+        const int u = __ffs(active) - 1;
+        active &= active - 1;
+        return wave + kWaves * u;
+    };
+    auto load_row = [&](int i, int& ri, float& rd) {
+        ri = -2;
+        rd = INFINITY;
+        if (i >= 0 && lane < K) {
+            const size_t at = (size_t)lids[i] * (size_t)K + lane;
+            ri = knn_idx[at];
+            rd = knn_dist[at];
+        }
+    };
+    int i0 = next_member(), i1 = next_member();
+    int ri0, ri1, ri2;
+    float rd0, rd1, rd2;
+    load_row(i0, ri0, rd0);
+    load_row(i1, ri1, rd1);
+    while (i0 >= 0) {
+        const int i2 = next_member();
+        load_row(i2, ri2, rd2);
+        const float d = candidate(i0);
+        KnnRow<1> row;
+        row.idx[0] = ri0;
+        row.dist[0] = rd0;
+        row.init_sorted(K);
+        row.offer_lanes<true>(lane < s && lane != i0, my_id, d);
+        if (row.changed) {
+            const size_t at = (size_t)lids[i0] * (size_t)K;
+            row.store(knn_idx + at, knn_dist + at);
+        }
+        i0 = i1; ri0 = ri1; rd0 = rd1;
+        i1 = i2; ri1 = ri2; rd1 = rd2;
+    }
+}
+
+// one wavefront per row: rows that are not sorted by distance are rebuilt by insertion
+template <int SL>
+__global__ __launch_bounds__(256) void k_sort_rows(int* __restrict__ knn_idx, float* __restrict__ knn_dist, int N, int K)
+{
+    const int row_id = (int)((blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> 6);
+    if (row_id >= N) return;
+    KnnRow<SL> row;
+    row.load(knn_idx + (size_t)row_id * K, knn_dist + (size_t)row_id * K, K);
+    if (row.changed) row.store(knn_idx + (size_t)row_id * K, knn_dist + (size_t)row_id * K);
+}
+
+}  // namespace
+
+int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream)
+{
+    if (N <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 256, "sort rows: K must be in 1..256");
+    const dim3 grid((unsigned)((N + 3) / 4)), block(256);
+    if (K <= 64) hipLaunchKernelGGL(k_sort_rows<1>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    else if (K <= 128) hipLaunchKernelGGL(k_sort_rows<2>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    else hipLaunchKernelGGL(k_sort_rows<4>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+// Buckets of at most 64 points given by (starts, sizes); rows sorted on entry.
+int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int K, const int* ids, const int* starts,
+                             const int* sizes, int n_buckets, int* knn_idx, float* knn_dist, hipStream_t stream)
+{
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 64, "screened small-bucket kernel: K must be in 1..64");
+    RSFK_CHECK(bf.rows != nullptr && bf.norms != nullptr && starts != nullptr, "screened small-bucket kernel: missing input");
+    const int dpad = (D + 3) & ~3;
+    const int n_slices = (dpad + kMaxChunk - 1) / kMaxChunk;
+    const int chunk = (((dpad + n_slices - 1) / n_slices) + 3) & ~3;
+    RSFK_CHECK(chunk >= 4 && chunk <= kMaxChunk, "screened small-bucket kernel: slice width");
+    int pitch = chunk;
+    if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units: rows start in different banks
+    RSFK_CHECK(kCap * pitch < 65536, "screened small-bucket kernel: LDS offsets must fit 16 bits");
+    const int region = std::max(kCap * pitch, kMaxPairs);
+    const int region_floats = (region + 3) & ~3;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(3 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
+    const int ksteps = (bf16_valid(D) + 15) / 16;
+    RSFK_CHECK(ksteps * 16 <= bf16_pitch(D), "screened small-bucket kernel: bfloat16 rows too short");
+    const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21
+    const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
+    RSFK_CHECK(one_minus_gamma > 0.5f, "screened small-bucket kernel: D too large");
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_screen),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(k_bucket_knn_screen, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, bf.rows,
+                       bf.norms, D, K, ids, starts, sizes, knn_idx, knn_dist, chunk, pitch, region_floats,
+                       bf16_pitch(D), ksteps, kappa, one_minus_gamma);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace rsfk

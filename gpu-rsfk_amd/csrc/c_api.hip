@@ -120,8 +120,11 @@ RSFK_API int rsfk_explore_device(const float* d_points, int N, int D, int num_ne
     Bf16Copy bf;
     int rc = bf16_copy_alloc(&bf, N, D);
     if (!rc) rc = bf16_copy_fill(bf, d_points, N, D, s);
-    if (!rc) rc = launch_explore(d_points, &bf, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, s);
+    ExploreWorkspace* ws = nullptr;
+    if (!rc && explore_join_enabled(N, num_neighbors)) rc = explore_ws_alloc(&ws, N, num_neighbors);
+    if (!rc) rc = launch_explore(d_points, &bf, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, ws, s);
     if (!rc && hipStreamSynchronize(s) != hipSuccess) { set_last_error("hipStreamSynchronize failed"); rc = 1; }
+    explore_ws_free(ws);
     bf16_copy_free(&bf);
     return rc;
 }
@@ -201,10 +204,13 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
     Bf16Copy bf;
     int rc = bf16_copy_alloc(&bf, N, D);
     if (!rc) rc = bf16_copy_fill(bf, static_cast<const float*>(dp.p), N, D, nullptr);
+    ExploreWorkspace* ws = nullptr;
+    if (!rc && explore_join_enabled(N, num_neighbors)) rc = explore_ws_alloc(&ws, N, num_neighbors);
     for (int it = 0; it < passes && !rc; ++it)
         rc = launch_explore(static_cast<const float*>(dp.p), &bf, N, D, num_neighbors, static_cast<int*>(dki.p),
-                            static_cast<float*>(dkd.p), static_cast<int*>(dold.p), nullptr);
+                            static_cast<float*>(dkd.p), static_cast<int*>(dold.p), ws, nullptr);
     if (!rc && hipDeviceSynchronize() != hipSuccess) { set_last_error("hipDeviceSynchronize failed"); rc = 1; }
+    explore_ws_free(ws);
     bf16_copy_free(&bf);
     if (rc) return rc;
     RSFK_HIP(hipDeviceSynchronize());

@@ -281,12 +281,29 @@ template <int SL, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict__ points, Bf16Copy bf, int N, int D, int K,
                                                          const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                          float* __restrict__ knn_dist, int table_size, int wave_lds_ints,
-                                                         int dpad, int rows_per_group)
+                                                         int dpad, int rows_per_group, const int* __restrict__ fwd2rev,
+                                                         const uint32_t* __restrict__ pass)
 {
     extern __shared__ __align__(16) int lds_i[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int p = blockIdx.x * WAVES + wave;
     if (p >= N) return;                                   // whole wavefront leaves together
+    // Candidates marked by the join (explore_join.hip): entry (p, k) of the graph has its mask of
+    // neighbour slots at pass[fwd2rev[p K + k]].  None marked -> nothing to do; more than the set can
+    // take -> this point enumerates its candidates itself, like without the join.
+    const int MW = (K + 31) >> 5;
+    int n_given = -1;
+    if (pass != nullptr) {
+        int bits = 0;
+        for (int k = lane; k < K; k += 64) {
+            const int j = fwd2rev[(size_t)p * K + k];
+            if (j >= 0)
+                for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
+        }
+        n_given = wave_sum_i(bits);
+        if (n_given == 0) return;
+        if (n_given + K + 1 > table_size / 4 * 3) n_given = -1;
+    }
     int* base = lds_i + (size_t)wave * (size_t)wave_lds_ints;
     ExploreLds L;
     L.tile = reinterpret_cast<float*>(base);                        // 64*kPitch words, 16-byte aligned
@@ -296,7 +313,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     L.srow = L.table + table_size;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const bool use_screen = bf.rows != nullptr;
-    const int mask = table_size - 1;
+    int mask = table_size - 1;
 
     KnnRow<SL> row;
     row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
@@ -311,6 +328,54 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     C.D = D;
     C.nblk = (C.Dv + kBlockB - 1) / kBlockB;
     int queued2 = 0;                                       // wave-uniform
+
+    if (n_given > 0) {
+        // several neighbours may name the same candidate, and it may be in the row already: pass the
+        // marked ids through a set sized for them, then exact distances for what is left (the join has
+        // screened already)
+        int ts = 64;
+        while (ts < 2 * (n_given + K + 1)) ts <<= 1;
+        ts = min(ts, table_size);
+        mask = ts - 1;
+        wave_lds_sync();
+        for (int i = lane; i < ts; i += 64) L.table[i] = kEmpty;
+        wave_lds_sync();
+        if (lane == 0) set_insert(L.table, mask, p, true);
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+            if (row.idx[s] >= 0) set_insert(L.table, mask, row.idx[s], true);
+        for (int k = lane; k < K; k += 64) {
+            const int j = fwd2rev[(size_t)p * K + k];
+            if (j < 0) continue;
+            const int* qrow = old_idx + (size_t)L.srow[k] * K;
+            for (int w = 0; w < MW; ++w) {
+                uint32_t m = pass[(size_t)j * MW + w];
+                while (m) {
+                    const int b = __ffs(m) - 1;
+                    m &= m - 1;
+                    const int c = qrow[32 * w + b];
+                    if (c >= 0 && c < N) set_insert(L.table, mask, c, false);
+                }
+            }
+        }
+        wave_lds_sync();
+        int U = 0;
+        for (int t0 = 0; t0 < ts; t0 += 64) {
+            const int v = L.table[t0 + lane];
+            const bool is_cand = v >= 0;
+            const uint64_t m = ballot64(is_cand);
+            wave_lds_sync();
+            if (is_cand) L.table[U + mask_prefix(m)] = v;
+            U += __popcll(m);
+        }
+        wave_lds_sync();
+        for (int off = 0; off < U; off += 64) {
+            wave_lds_sync();
+            exact_batch<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+        }
+        if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
+        return;
+    }
 
     for (int i0 = 0; i0 < K; i0 += rows_per_group) {
         const int i1 = min(K, i0 + rows_per_group);
@@ -383,14 +448,15 @@ int next_pow2(int v)
 
 template <int SL, int WAVES>
 int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, const int* old_idx, int* knn_idx,
-               float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, hipStream_t stream)
+               float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, const int* fwd2rev,
+               const uint32_t* pass, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore<SL, WAVES>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     dim3 grid((unsigned)((N + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore<SL, WAVES>), grid, block, lds, stream, points, b, N, D, K, old_idx, knn_idx, knn_dist,
-                       table, wave_ints, dpad, rows_per_group);
+                       table, wave_ints, dpad, rows_per_group, fwd2rev, pass);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -399,11 +465,15 @@ int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, cons
 
 // One exploration pass.  old_idx is scratch of N*K ints (receives the snapshot).
 // bf may be null (or hold null rows): every candidate then gets the exact distance.
+// ws may be null; with a workspace and a bfloat16 copy the candidates come from the join over the
+// reversed graph (explore_join.hip), which needs rows sorted by distance.
 int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K, int* knn_idx, float* knn_dist,
-                   int* old_idx, hipStream_t stream)
+                   int* old_idx, ExploreWorkspace* ws, hipStream_t stream)
 {
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
+    const bool join = ws != nullptr && bf != nullptr && bf->rows != nullptr;
+    if (join && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
     const int dpad = bf16_valid(D);
     const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set
@@ -425,11 +495,18 @@ int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K,
     const int wave_ints = (fixed + table + 3) / 4 * 4;
     Bf16Copy b;
     if (bf) b = *bf;
+    const int* fwd2rev = nullptr;
+    const uint32_t* pass = nullptr;
+    if (join) {
+        if (launch_explore_join(ws, b, N, D, K, old_idx, knn_dist, stream)) return 1;
+        fwd2rev = explore_ws_fwd2rev(ws);
+        pass = explore_ws_pass(ws);
+    }
     const int sl = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
 #define RSFK_EXPLORE_CASE(SLV, WV)                                                                                      \
     if (sl == SLV && waves == WV)                                                                                       \
         return launch_one<SLV, WV>(points, b, N, D, K, old_idx, knn_idx, knn_dist, table, wave_ints, dpad,              \
-                                   rows_per_group, stream);
+                                   rows_per_group, fwd2rev, pass, stream);
     RSFK_EXPLORE_CASE(1, 4) RSFK_EXPLORE_CASE(1, 2) RSFK_EXPLORE_CASE(1, 1)
     RSFK_EXPLORE_CASE(2, 4) RSFK_EXPLORE_CASE(2, 2) RSFK_EXPLORE_CASE(2, 1)
     RSFK_EXPLORE_CASE(4, 4) RSFK_EXPLORE_CASE(4, 2) RSFK_EXPLORE_CASE(4, 1)

@@ -11,6 +11,7 @@
 #include "forest.hpp"
 #include <algorithm>
 #include <chrono>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <vector>
@@ -63,6 +64,10 @@ struct Bf16Guard {
     Bf16Copy c;
     ~Bf16Guard() { bf16_copy_free(&c); }
 };
+struct ExploreWsGuard {
+    ExploreWorkspace* w = nullptr;
+    ~ExploreWsGuard() { explore_ws_free(w); }
+};
 struct EventPair {
     hipEvent_t a = nullptr, b = nullptr;
 };
@@ -82,7 +87,15 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (bf16_copy_alloc(&bf.c, N, D)) return 1;
     if (bf16_copy_fill(bf.c, d_points, N, D, stream)) return 1;
 
+    // RSFK_BUCKET_SCREEN=1 sends the small buckets to the kernel that screens pairs on the bfloat16 copy
+    // before computing exact distances (same results; not faster on the workloads measured so far)
+    const char* env_screen = std::getenv("RSFK_BUCKET_SCREEN");
+    const bool screen = K <= 64 && env_screen && env_screen[0] == '1';
+
     if (n_trees > 0) {
+        // the screened kernel reads a row's maximum from its last slot: rows the caller passed in unsorted are
+        // put in order once
+        if (screen && launch_sort_rows(d_idx, d_dist, N, K, stream)) return 1;
         const int B = choose_batch(n_trees, N, D, MIN);
         WsGuard ws;
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
@@ -98,7 +111,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             const double tb = now_s() - tb0;
             for (int j = 0; j < nb && rc == 0; ++j) {
                 (void)hipEventRecord(ev[j].a, stream);
-                rc = launch_bucket_knn_tree(d_points, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w),
                                             stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], d_idx, d_dist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
@@ -132,8 +145,10 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (nnef > 0) {
         DevBuf old;
         RSFK_HIP(hipMalloc(&old.p, sizeof(int) * (size_t)N * (size_t)K));
+        ExploreWsGuard ews;      // without a workspace every point enumerates its own candidates
+        if (explore_join_enabled(N, K) && explore_ws_alloc(&ews.w, N, K)) return 1;
         for (int it = 0; it < nnef; ++it) {
-            if (launch_explore(d_points, &bf.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), stream)) return 1;
+            if (launch_explore(d_points, &bf.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream)) return 1;
         }
         RSFK_HIP(hipStreamSynchronize(stream));
     }

@@ -25,17 +25,34 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream);
 
-int launch_bucket_knn_tree(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
-                           int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist, hipStream_t stream);
+int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, int D, int K, const int* ids, const int* starts,
+                           const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist,
+                           hipStream_t stream);
+
+// bucket_knn_screen.hip
+int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);
+int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int K, const int* ids, const int* starts,
+                             const int* sizes, int n_buckets, int* knn_idx, float* knn_dist, hipStream_t stream);
 
 // bucket_knn_small.hip
 int small_bucket_cap();
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
                             int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream);
 
+// explore_join.hip
+struct ExploreWorkspace;
+bool explore_join_enabled(int N, int K);
+size_t explore_ws_bytes(int N, int K);
+int explore_ws_alloc(ExploreWorkspace** out, int N, int K);
+void explore_ws_free(ExploreWorkspace* w);
+const int* explore_ws_fwd2rev(const ExploreWorkspace* w);
+const uint32_t* explore_ws_pass(const ExploreWorkspace* w);
+int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
+                        const float* knn_dist, hipStream_t stream);
+
 // explore.hip
 int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K, int* knn_idx, float* knn_dist,
-                   int* old_idx, hipStream_t stream);
+                   int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
 // forest.hip
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
