@@ -81,7 +81,7 @@ struct ExploreLds {          // per wavefront; sizes fixed at launch
     int* srow;               // snapshot of the point's own row, K ints
     int* queue2;             // candidates that passed the screen, waiting for the exact distance
     float* xrow;             // the point's coordinates, zero padded to bf16_valid(D)
-    float* tile;             // 64 x kPitch words
+    float* tile;             // 64 x (chunk + 4) words
 };
 
 // Load one 16-byte piece (4 dimensions) of a candidate row, zero beyond D.
@@ -101,38 +101,43 @@ __device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int 
     return v;
 }
 
-// Exact distances of the first n candidates of `list` to the point, then offer them.
-template <int SL>
+// Exact distances of the first n candidates of `list` to the point, then offer them.  CH = dimensions
+// staged per step (32 or 16): a step moves 64 rows x CH floats through the tile.
+template <int SL, int CH = kChunk>
 __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
                                             const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row)
 {
+    constexpr int kPieces = CH / 4;         // 16-byte pieces of a row per step = lanes per row
+    constexpr int kRows = 64 / kPieces;     // rows per load instruction
+    constexpr int kLoads = 64 / kRows;      // load instructions per step
+    constexpr int kP = CH + 4;              // tile pitch: odd number of 16-byte units
     const int lane = lane_id();
-    const int sub = lane >> 3;          // which of 8 rows of a load step
-    const int piece = lane & 7;         // which 16-byte piece of the 128-byte segment
+    const int sub = lane / kPieces;         // which of the rows of a load instruction
+    const int piece = lane % kPieces;       // which 16-byte piece of the segment
     const int my_c = lane < n ? list[lane] : -1;
-    const float* rp[8];
+    const float* rp[kLoads];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int r = i * 8 + sub;
+    for (int i = 0; i < kLoads; ++i) {
+        const int r = i * kRows + sub;
         rp[i] = points + (size_t)list[r < n ? r : 0] * (size_t)D;      // rows beyond n repeat row 0 (ignored later)
     }
-    float4 pre[8];
+    float4 pre[kLoads];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok);
+    for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok);
     float acc = 0.0f;
     const float tau0 = row.tau;
-    for (int d0 = 0; d0 < D; d0 += kChunk) {
+    for (int d0 = 0; d0 < D; d0 += CH) {
         wave_lds_sync();                 // previous step's tile reads are done
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            *reinterpret_cast<float4*>(&L.tile[(i * 8 + sub) * kPitch + piece * 4]) = pre[i];
-        if (d0 + kChunk < D) {
+        for (int i = 0; i < kLoads; ++i)
+            *reinterpret_cast<float4*>(&L.tile[(i * kRows + sub) * kP + piece * 4]) = pre[i];
+        if (d0 + CH < D) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) pre[i] = load_piece(rp[i], d0 + kChunk + piece * 4, D, vec_ok);
+            for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], d0 + CH + piece * 4, D, vec_ok);
         }
         wave_lds_sync();
-        const int pieces = min(8, (D - d0 + 3) >> 2);
-        const float* mine = &L.tile[lane * kPitch];
+        const int pieces = min(kPieces, (D - d0 + 3) >> 2);
+        const float* mine = &L.tile[lane * kP];
         const float* xs = &L.xrow[d0];
         for (int q = 0; q < pieces; ++q) {
             const float4 a = *reinterpret_cast<const float4*>(mine + 4 * q);
@@ -281,29 +286,14 @@ template <int SL, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict__ points, Bf16Copy bf, int N, int D, int K,
                                                          const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                          float* __restrict__ knn_dist, int table_size, int wave_lds_ints,
-                                                         int dpad, int rows_per_group, const int* __restrict__ fwd2rev,
-                                                         const uint32_t* __restrict__ pass)
+                                                         int dpad, int rows_per_group, const int* __restrict__ todo,
+                                                         int n_todo)
 {
     extern __shared__ __align__(16) int lds_i[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int p = blockIdx.x * WAVES + wave;
-    if (p >= N) return;                                   // whole wavefront leaves together
-    // Candidates marked by the join (explore_join.hip): entry (p, k) of the graph has its mask of
-    // neighbour slots at pass[fwd2rev[p K + k]].  None marked -> nothing to do; more than the set can
-    // take -> this point enumerates its candidates itself, like without the join.
-    const int MW = (K + 31) >> 5;
-    int n_given = -1;
-    if (pass != nullptr) {
-        int bits = 0;
-        for (int k = lane; k < K; k += 64) {
-            const int j = fwd2rev[(size_t)p * K + k];
-            if (j >= 0)
-                for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
-        }
-        n_given = wave_sum_i(bits);
-        if (n_given == 0) return;
-        if (n_given + K + 1 > table_size / 4 * 3) n_given = -1;
-    }
+    const int slot = blockIdx.x * WAVES + wave;
+    if (slot >= (todo ? n_todo : N)) return;              // whole wavefront leaves together
+    const int p = todo ? todo[slot] : slot;               // all points, or the listed ones
     int* base = lds_i + (size_t)wave * (size_t)wave_lds_ints;
     ExploreLds L;
     L.tile = reinterpret_cast<float*>(base);                        // 64*kPitch words, 16-byte aligned
@@ -313,7 +303,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     L.srow = L.table + table_size;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const bool use_screen = bf.rows != nullptr;
-    int mask = table_size - 1;
+    const int mask = table_size - 1;
 
     KnnRow<SL> row;
     row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
@@ -328,54 +318,6 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     C.D = D;
     C.nblk = (C.Dv + kBlockB - 1) / kBlockB;
     int queued2 = 0;                                       // wave-uniform
-
-    if (n_given > 0) {
-        // several neighbours may name the same candidate, and it may be in the row already: pass the
-        // marked ids through a set sized for them, then exact distances for what is left (the join has
-        // screened already)
-        int ts = 64;
-        while (ts < 2 * (n_given + K + 1)) ts <<= 1;
-        ts = min(ts, table_size);
-        mask = ts - 1;
-        wave_lds_sync();
-        for (int i = lane; i < ts; i += 64) L.table[i] = kEmpty;
-        wave_lds_sync();
-        if (lane == 0) set_insert(L.table, mask, p, true);
-#pragma unroll
-        for (int s = 0; s < SL; ++s)
-            if (row.idx[s] >= 0) set_insert(L.table, mask, row.idx[s], true);
-        for (int k = lane; k < K; k += 64) {
-            const int j = fwd2rev[(size_t)p * K + k];
-            if (j < 0) continue;
-            const int* qrow = old_idx + (size_t)L.srow[k] * K;
-            for (int w = 0; w < MW; ++w) {
-                uint32_t m = pass[(size_t)j * MW + w];
-                while (m) {
-                    const int b = __ffs(m) - 1;
-                    m &= m - 1;
-                    const int c = qrow[32 * w + b];
-                    if (c >= 0 && c < N) set_insert(L.table, mask, c, false);
-                }
-            }
-        }
-        wave_lds_sync();
-        int U = 0;
-        for (int t0 = 0; t0 < ts; t0 += 64) {
-            const int v = L.table[t0 + lane];
-            const bool is_cand = v >= 0;
-            const uint64_t m = ballot64(is_cand);
-            wave_lds_sync();
-            if (is_cand) L.table[U + mask_prefix(m)] = v;
-            U += __popcll(m);
-        }
-        wave_lds_sync();
-        for (int off = 0; off < U; off += 64) {
-            wave_lds_sync();
-            exact_batch<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
-        }
-        if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
-        return;
-    }
 
     for (int i0 = 0; i0 < K; i0 += rows_per_group) {
         const int i1 = min(K, i0 + rows_per_group);
@@ -439,6 +381,120 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
 
+// Exploration of the points whose candidates the join has marked (explore_join.hip): entry (p, k) of
+// the graph has the mask of neighbour slots at pass[fwd2rev[p K + k]].  One wavefront per point: gather
+// the marked ids, drop repeats and ids the row holds (hash set), exact distances, merge.  Points with
+// more marks than the LDS of this launch takes are appended to todo_out (for a launch with more LDS
+// per wavefront, or for the general kernel).  todo_in: the points to work on, or null for all.
+// Per-wavefront LDS (ints): tile[64*20] | xrow[dpad] | table[table_size] | srow[K] | marked[3/4 table_size].
+constexpr int kMergeChunk = 16;
+constexpr int kMergeTile = 64 * (kMergeChunk + 4);
+
+template <int SL, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __restrict__ points, int N, int D, int K,
+                                                               const int* __restrict__ old_idx, int* __restrict__ knn_idx,
+                                                               float* __restrict__ knn_dist, int table_size,
+                                                               int wave_lds_ints, int dpad,
+                                                               const int* __restrict__ fwd2rev,
+                                                               const uint32_t* __restrict__ pass,
+                                                               const int* __restrict__ todo_in, int n_in,
+                                                               int* __restrict__ todo_out, int* __restrict__ n_out)
+{
+    extern __shared__ __align__(16) int lds_m[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = blockIdx.x * WAVES + wave;
+    if (slot >= (todo_in ? n_in : N)) return;             // whole wavefront leaves together
+    const int p = todo_in ? todo_in[slot] : slot;
+    const int MW = (K + 31) >> 5;
+    int bits = 0;
+    for (int k = lane; k < K; k += 64) {
+        const int j = fwd2rev[(size_t)p * K + k];
+        if (j >= 0)
+            for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
+    }
+    const int n_given = wave_sum_i(bits);
+    if (n_given == 0) return;
+    if (n_given + K + 1 > table_size / 4 * 3) {
+        if (lane == 0) todo_out[atomicAdd(n_out, 1)] = p;
+        return;
+    }
+    int* base = lds_m + (size_t)wave * (size_t)wave_lds_ints;
+    ExploreLds L;
+    L.tile = reinterpret_cast<float*>(base);
+    L.xrow = reinterpret_cast<float*>(base + kMergeTile);
+    L.queue2 = nullptr;
+    L.table = base + kMergeTile + dpad;
+    L.srow = L.table + table_size;
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+
+    KnnRow<SL> row;
+    row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+    for (int k = lane; k < K; k += 64) L.srow[k] = old_idx[(size_t)p * K + k];
+    const float* xp = points + (size_t)p * D;
+    for (int d = lane; d < dpad; d += 64) L.xrow[d] = d < D ? xp[d] : 0.0f;
+
+    int ts = 64;
+    while (ts < 2 * (n_given + K + 1)) ts <<= 1;
+    ts = min(ts, table_size);
+    const int mask = ts - 1;
+    for (int i = lane; i < ts; i += 64) L.table[i] = kEmpty;
+    wave_lds_sync();
+    if (lane == 0) set_insert(L.table, mask, p, true);
+#pragma unroll
+    for (int s = 0; s < SL; ++s)
+        if (row.idx[s] >= 0) set_insert(L.table, mask, row.idx[s], true);
+    // list of the marked (neighbour, slot) pairs, so that the ids can be gathered by all lanes at once
+    // instead of one after the other per neighbour
+    int* marked = L.srow + K;
+    int n_marked = 0;                                     // wave-uniform
+    for (int k0 = 0; k0 < K; k0 += 64) {
+        const int k = k0 + lane;
+        const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
+        int mine = 0;
+        if (j >= 0)
+            for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
+        int at = n_marked + wave_excl_scan_i(mine);
+        if (j >= 0) {
+            for (int w = 0; w < MW; ++w) {
+                uint32_t m = pass[(size_t)j * MW + w];
+                while (m) {
+                    const int b = __ffs(m) - 1;
+                    m &= m - 1;
+                    marked[at++] = k | ((32 * w + b) << 8);
+                }
+            }
+        }
+        n_marked += wave_sum_i(mine);
+    }
+    wave_lds_sync();
+    for (int i0 = 0; i0 < n_marked; i0 += 64) {
+        const int i = i0 + lane;
+        int c = -1;
+        if (i < n_marked) {
+            const int e = marked[i];
+            c = old_idx[(size_t)L.srow[e & 255] * K + (e >> 8)];
+        }
+        if (c >= 0 && c < N) set_insert(L.table, mask, c, false);
+    }
+    wave_lds_sync();
+    // compact the set in place into the candidate list
+    int U = 0;
+    for (int t0 = 0; t0 < ts; t0 += 64) {
+        const int v = L.table[t0 + lane];
+        const bool is_cand = v >= 0;
+        const uint64_t m = ballot64(is_cand);
+        wave_lds_sync();
+        if (is_cand) L.table[U + mask_prefix(m)] = v;
+        U += __popcll(m);
+    }
+    wave_lds_sync();
+    for (int off = 0; off < U; off += 64) {
+        wave_lds_sync();
+        exact_batch<SL, kMergeChunk>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+    }
+    if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
+}
+
 int next_pow2(int v)
 {
     int p = 1;
@@ -447,16 +503,52 @@ int next_pow2(int v)
 }
 
 template <int SL, int WAVES>
+int launch_merge(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
+                 int wave_ints, int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in, int n_in,
+                 int* todo_out, int* n_out, hipStream_t stream)
+{
+    const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int n_work = todo_in ? n_in : N;
+    dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
+    hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
+                       knn_dist, table, wave_ints, dpad, fwd2rev, pass, todo_in, n_in, todo_out, n_out);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+// ints of LDS a wavefront of the merge kernel needs for a set of `table` entries
+int merge_wave_ints(int table, int dpad, int K) { return (kMergeTile + dpad + table + K + table / 4 * 3 + 3) / 4 * 4; }
+
+int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
+                   float* knn_dist, int table, int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in,
+                   int n_in, int* todo_out, int* n_out, hipStream_t stream)
+{
+    const int wi = merge_wave_ints(table, dpad, K);
+#define RSFK_MERGE_CASE(SLV, WV)                                                                                        \
+    if (sl == SLV && waves == WV)                                                                                       \
+        return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, fwd2rev, pass,       \
+                                     todo_in, n_in, todo_out, n_out, stream);
+    RSFK_MERGE_CASE(1, 4) RSFK_MERGE_CASE(1, 2) RSFK_MERGE_CASE(1, 1)
+    RSFK_MERGE_CASE(2, 4) RSFK_MERGE_CASE(2, 2) RSFK_MERGE_CASE(2, 1)
+    RSFK_MERGE_CASE(4, 4) RSFK_MERGE_CASE(4, 2) RSFK_MERGE_CASE(4, 1)
+#undef RSFK_MERGE_CASE
+    RSFK_CHECK(false, "exploration: no merge kernel for this configuration");
+}
+
+template <int SL, int WAVES>
 int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, const int* old_idx, int* knn_idx,
-               float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, const int* fwd2rev,
-               const uint32_t* pass, hipStream_t stream)
+               float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, const int* todo, int n_todo,
+               hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore<SL, WAVES>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    dim3 grid((unsigned)((N + WAVES - 1) / WAVES)), block(64 * WAVES);
+    const int n_work = todo ? n_todo : N;
+    dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore<SL, WAVES>), grid, block, lds, stream, points, b, N, D, K, old_idx, knn_idx, knn_dist,
-                       table, wave_ints, dpad, rows_per_group, fwd2rev, pass);
+                       table, wave_ints, dpad, rows_per_group, todo, n_todo);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -495,18 +587,47 @@ int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K,
     const int wave_ints = (fixed + table + 3) / 4 * 4;
     Bf16Copy b;
     if (bf) b = *bf;
-    const int* fwd2rev = nullptr;
-    const uint32_t* pass = nullptr;
-    if (join) {
-        if (launch_explore_join(ws, b, N, D, K, old_idx, knn_dist, stream)) return 1;
-        fwd2rev = explore_ws_fwd2rev(ws);
-        pass = explore_ws_pass(ws);
-    }
     const int sl = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
+    const int* todo = nullptr;
+    int n_todo = 0;
+    if (join) {
+        // Marks from the join, then the merge kernel with a small set (little LDS, many wavefronts per CU).
+        // The points it cannot take come back in a list and get a second launch with the largest set that
+        // fits; what is left after that goes to the general kernel below.
+        if (launch_explore_join(ws, b, N, D, K, old_idx, knn_dist, stream)) return 1;
+        const int* f2r = explore_ws_fwd2rev(ws);
+        const uint32_t* pass = explore_ws_pass(ws);
+        int* listA = explore_ws_todo(ws, 0);
+        int* listB = explore_ws_todo(ws, 1);
+        int* host_n = explore_ws_host_count(ws);
+        const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
+        RSFK_CHECK(4 * merge_wave_ints(small_table, dpad, K) <= lds_ints, "exploration: D too large for the merge kernel");
+        if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, f2r, pass, nullptr, 0,
+                           listA, listA + N, stream))
+            return 1;
+        RSFK_HIP(hipMemcpyAsync(host_n, listA + N, sizeof(int), hipMemcpyDeviceToHost, stream));
+        RSFK_HIP(hipStreamSynchronize(stream));
+        n_todo = *host_n;
+        if (n_todo == 0) return 0;
+        todo = listA;
+        int big_table = want, big_waves = 4;
+        while (big_waves > 1 && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_waves >>= 1;
+        while (big_table > small_table && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_table >>= 1;
+        if (big_table > small_table) {
+            if (dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass,
+                               listA, n_todo, listB, listB + N, stream))
+                return 1;
+            RSFK_HIP(hipMemcpyAsync(host_n, listB + N, sizeof(int), hipMemcpyDeviceToHost, stream));
+            RSFK_HIP(hipStreamSynchronize(stream));
+            n_todo = *host_n;
+            if (n_todo == 0) return 0;
+            todo = listB;
+        }
+    }
 #define RSFK_EXPLORE_CASE(SLV, WV)                                                                                      \
     if (sl == SLV && waves == WV)                                                                                       \
         return launch_one<SLV, WV>(points, b, N, D, K, old_idx, knn_idx, knn_dist, table, wave_ints, dpad,              \
-                                   rows_per_group, fwd2rev, pass, stream);
+                                   rows_per_group, todo, n_todo, stream);
     RSFK_EXPLORE_CASE(1, 4) RSFK_EXPLORE_CASE(1, 2) RSFK_EXPLORE_CASE(1, 1)
     RSFK_EXPLORE_CASE(2, 4) RSFK_EXPLORE_CASE(2, 2) RSFK_EXPLORE_CASE(2, 1)
     RSFK_EXPLORE_CASE(4, 4) RSFK_EXPLORE_CASE(4, 2) RSFK_EXPLORE_CASE(4, 1)

@@ -35,6 +35,8 @@ struct ExploreWorkspace {
     int* deg = nullptr;        // N: in-degree (counted, then consumed by the fill)
     int* totals = nullptr;     // per scan block
     uint32_t* pass = nullptr;  // N*K*MW
+    int* todo = nullptr;       // two lists of N+1 ints: points left over by a launch; entry N = their number
+    int* host_count = nullptr; // pinned
     int n_blocks = 0;
 };
 namespace {
@@ -45,10 +47,11 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kScanBlock = 1024;            // elements per workgroup of the scan (256 threads x 4)
 constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16
 
-__global__ void k_zero(int* a, int n)
+__global__ void k_zero(int* a, int n, int* counter0, int* counter1)
 {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) a[i] = 0;
+    if (i == 0) { *counter0 = 0; *counter1 = 0; }
 }
 
 __global__ void k_degree(const int* __restrict__ old_idx, size_t total, int N, int* __restrict__ deg)
@@ -232,7 +235,7 @@ bool explore_join_enabled(int N, int K)
 size_t explore_ws_bytes(int N, int K)
 {
     const size_t mw = (size_t)((K + 31) / 32);
-    return (size_t)N * ((size_t)K * 4 * (2 + mw) + 16) + 4096;
+    return (size_t)N * ((size_t)K * 4 * (2 + mw) + 24) + 4096;
 }
 
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
@@ -246,7 +249,9 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
     auto dm = [](void* p, size_t n) { return hipMalloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)); };
     if (dm(&w->rev, (size_t)N * K) != hipSuccess || dm(&w->fwd2rev, (size_t)N * K) != hipSuccess ||
         dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->deg, (size_t)N) != hipSuccess ||
-        dm(&w->totals, (size_t)w->n_blocks + 1) != hipSuccess || dm(&w->pass, (size_t)N * K * w->MW) != hipSuccess) {
+        dm(&w->totals, (size_t)w->n_blocks + 1) != hipSuccess || dm(&w->pass, (size_t)N * K * w->MW) != hipSuccess ||
+        dm(&w->todo, 2 * ((size_t)N + 1)) != hipSuccess ||
+        hipHostMalloc(reinterpret_cast<void**>(&w->host_count), sizeof(int)) != hipSuccess) {
         explore_ws_free(w);
         set_last_error("exploration workspace: out of device memory");
         return 1;
@@ -258,14 +263,17 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass};
+    void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass, w->todo};
     for (void* b : bufs)
         if (b) (void)hipFree(b);
+    if (w->host_count) (void)hipHostFree(w->host_count);
     delete w;
 }
 
 const int* explore_ws_fwd2rev(const ExploreWorkspace* w) { return w->fwd2rev; }
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w) { return w->pass; }
+int* explore_ws_todo(ExploreWorkspace* w, int which) { return w->todo + (size_t)which * ((size_t)w->N + 1); }
+int* explore_ws_host_count(ExploreWorkspace* w) { return w->host_count; }
 
 // Fill pass and fwd2rev from the snapshot old_idx and the current last slots of knn_dist (rows sorted by distance).
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
@@ -277,7 +285,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     const size_t total = (size_t)N * (size_t)K;
     const int nb = w->n_blocks;
     const unsigned wide = (unsigned)std::min<size_t>((total + 255) / 256, 65536);
-    hipLaunchKernelGGL(k_zero, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, w->deg, N);
+    hipLaunchKernelGGL(k_zero, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, w->deg, N, w->todo + N, w->todo + 2 * (size_t)N + 1);
     hipLaunchKernelGGL(k_degree, dim3(wide), dim3(256), 0, stream, old_idx, total, N, w->deg);
     hipLaunchKernelGGL(k_scan_blocks, dim3((unsigned)nb), dim3(256), 0, stream, w->deg, N, w->offs, w->totals);
     hipLaunchKernelGGL(k_scan_totals, dim3(1), dim3(256), 0, stream, w->totals, nb, w->offs + N);

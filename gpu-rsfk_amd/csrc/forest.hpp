@@ -47,6 +47,8 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K);
 void explore_ws_free(ExploreWorkspace* w);
 const int* explore_ws_fwd2rev(const ExploreWorkspace* w);
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w);
+int* explore_ws_todo(ExploreWorkspace* w, int which);
+int* explore_ws_host_count(ExploreWorkspace* w);
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
                         const float* knn_dist, hipStream_t stream);
 

@@ -111,4 +111,17 @@ __device__ __forceinline__ int wave_sum_i(int v)
     return read_lane_i(v, 0) + read_lane_i(v, 16) + read_lane_i(v, 32) + read_lane_i(v, 48);
 }
 
+// exclusive prefix sum over the lanes of the wavefront
+__device__ __forceinline__ int wave_excl_scan_i(int v)
+{
+    const int lane = lane_id();
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int t = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += t;
+    }
+    return incl - v;
+}
+
 }  // namespace rsfk
