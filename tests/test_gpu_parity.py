@@ -148,9 +148,16 @@ def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
 # ---------------------------------------------------------------------------
 # exploration
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("join", ["join", "plain"])
 @pytest.mark.parametrize("N,D,K,self_in", [(3000, 32, 16, True), (2000, 100, 32, True), (1500, 5, 8, False),
-                                           (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True)])
-def test_explore_matches_oracle(gpu, orc, rng, N, D, K, self_in):
+                                           (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True),
+                                           (1300, 6, 200, True), (40, 7, 33, True), (5000, 130, 12, True)])
+def test_explore_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, self_in, join):
+    """Both ways of enumerating the candidates: the join over the reversed graph (default; with partly empty
+    rows and a large K its marks overflow the small set, then the large one, and the general kernel finishes)
+    and every point for itself (RSFK_EXPLORE_JOIN=0)."""
+    if join == "plain":
+        monkeypatch.setenv("RSFK_EXPLORE_JOIN", "0")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K, self_in=self_in)
     MIN = max(2, K // 2)                 # buckets smaller than K+1 leave some rows partly empty
@@ -197,8 +204,11 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
     (6000, 24, 40, 3, dict(nn_exploring_factor=2)),
     (4000, 12, 10, 2, dict(point_in_self_neigh=False, nn_exploring_factor=0)),
 ])
-def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, N, D, K, T, kw):
+@pytest.mark.parametrize("variant", ["default", "bucket_screen"])
+def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, T, kw, variant):
     import gpu_rsfk
+    if variant == "bucket_screen":
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
     X = rng.standard_normal((N, D)).astype(np.float32)
     r = gpu_rsfk.RSFK(random_state=17)
     _say("forest", N, D, K, T, kw)
@@ -325,11 +335,15 @@ def _hard_inputs(rng, kind, N, D):
     raise ValueError(kind)
 
 
+@pytest.mark.parametrize("variant", ["default", "bucket_screen"])
 @pytest.mark.parametrize("kind", ["offset", "grid", "tiny", "mixed", "clusters"])
-def test_screens_never_change_a_result(gpu, orc, rng, kind):
+def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant):
     """The bfloat16 screens only skip work whose outcome is certain: trees, bucket K-NN and exploration on inputs
-    that defeat a 8-bit mantissa must still be identical to the fp32 oracle."""
+    that defeat a 8-bit mantissa must still be identical to the fp32 oracle.  "bucket_screen" also switches the
+    small buckets to the kernel that screens pairs with the matrix cores (RSFK_BUCKET_SCREEN=1)."""
     import gpu_rsfk
+    if variant == "bucket_screen":
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
     N, D, K = 6000, 24, 10
     X = _hard_inputs(rng, kind, N, D)
     _say("hard tree", kind)
