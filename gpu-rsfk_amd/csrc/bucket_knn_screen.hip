@@ -10,14 +10,17 @@
 //   1. Gram matrix of the bucket's bfloat16 rows with the matrix cores
 //      (v_mfma_f32_32x32x16_bf16, operands straight from global memory, one to
 //      three 32x32 tiles): d~ = n_i + n_j - 2 G_ij approximates the distance, and
-//      a bound E on |d~ - exact fp32 result| follows from the norms alone
-//      (bfloat16 rounding: 2u sqrt(d~ Q) + u^2 Q with u = 2^-8 and Q = 2 (n_i + n_j),
-//      by Cauchy-Schwarz; accumulation errors of the Gram matrix, the norms and the
-//      fp32 chain are relative to n_i + n_j resp. to the distance).  Pairs with
-//      d~ - E >= max(last slot of row i, last slot of row j) are dropped; this never
-//      drops a pair that the exact arithmetic would have inserted;
+//      a bound on |d~ - exact fp32 result| follows from the norms alone.  With
+//      S = n_i + n_j (norms of the bfloat16 rows), u = 2^-8:
+//        rounding to bfloat16:   |d(real) - d~(real)| <= 2u sqrt(d~ Q) + u^2 Q,  Q = 2 S  (Cauchy-Schwarz)
+//        Gram matrix and norms:  |d~(computed) - d~(real)| <= E1 = (D' + 16) 2^-21 S
+//        fp32 chain:             result >= d(real) (1 - gamma),  gamma = (D + 8) 2^-22
+//      so the pair is dropped iff  d~ - E1 - 1.01 (2u sqrt((d~ + E1) Q) + u^2 Q) >= (limit + 1e-30) / (1 - gamma),
+//      limit = max(last slot of row i, last slot of row j); the inequality is evaluated
+//      without the square root (both sides squared when the left side is not negative).
+//      This never drops a pair that the exact arithmetic would have inserted;
 //   2. the remaining pairs go to a list in LDS; the fp32 rows are staged through LDS
-//      in slices of at most 48 dimensions and each thread runs the sequential fused
+//      in slices of at most 52 dimensions and each thread runs the sequential fused
 //      multiply-add chains (arithmetic of euclidean_distance_sqr,
 //      compute_knn_from_buckets.cu:40-54) of its pairs of the list;
 //   3. the exact distances land in a triangular matrix in LDS (+inf elsewhere) and
@@ -41,12 +44,17 @@ constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
 static_assert(kCap == 64, "two 32-row operand halves and lane-per-candidate merge assume 64");
 constexpr int kThreads = 128;
 constexpr int kWaves = kThreads / 64;
-constexpr int kMaxChunk = 48;               // dimensions staged at once
-constexpr int kMaxLoads = kCap * (kMaxChunk / 4) / kThreads;   // 16-byte loads per thread and slice
+constexpr int kMaxChunk = 52;               // dimensions staged at once
+constexpr int kLanesPerRow = 16;            // a row of a slice is loaded by 16 lanes, 16 bytes each (13 used at most)
+constexpr int kRowsPerStep = kThreads / kLanesPerRow;
+constexpr int kLoads = kCap / kRowsPerStep; // 16-byte loads per thread and slice
 constexpr int kMaxPairs = kCap * (kCap - 1) / 2;
 constexpr int kPairsPerThread = (kMaxPairs + kThreads - 1) / kThreads;
+static_assert(kMaxChunk / 4 <= kLanesPerRow, "a slice must fit the lanes of a row");
 
-constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16 (8 significant bits)
+constexpr float kU = 1.0f / 256.0f;                           // unit roundoff of bfloat16 (8 significant bits)
+constexpr float kC2 = 1.01f * kU * kU * 2.0001f;              // coefficient of S in the u^2 Q term
+constexpr float kC3 = (2.02f * kU) * (2.02f * kU) * 2.0001f;  // (1.01 2u)^2 Q / S
 
 // entry of pair (a, b), a < b, in the triangular matrix
 __device__ __forceinline__ int tri_at(int a, int b) { return ((b * (b - 1)) >> 1) + a; }
@@ -54,23 +62,22 @@ __device__ __forceinline__ int tri_at(int a, int b) { return ((b * (b - 1)) >> 1
 // Screen one 32x32 tile of the Gram matrix.  Accumulator i of lane l belongs to row member
 // m = mbase + 8 (i / 4) + i % 4 (mbase = first member of the operand half + 4 (l / 32)) and column
 // member n.  Returns the mask of accumulators whose pair (m < n < s) must be computed exactly.
-__device__ __forceinline__ uint32_t screen_tile(const f32x16& g, int mbase, int n, int s, const float* nrm, const float* tau,
-                                                float kappa, float one_minus_gamma)
+// taup = (last slot + 1e-30) / (1 - gamma) per member.
+__device__ __forceinline__ uint32_t screen_tile(const f32x16& g, int mbase, int n, int s, const float* nrm,
+                                                const float* taup, float kappa)
 {
-    const float nn = nrm[n], tn = tau[n];
+    const float nn = nrm[n], tn = taup[n];
     uint32_t bits = 0;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         const int m = mbase + 8 * (i >> 2) + (i & 3);
         const float S = nrm[m] + nn;
-        const float limit = fmaxf(tau[m], tn);
+        const float limit = fmaxf(taup[m], tn);
         const float dt = __builtin_fmaf(-2.0f, g[i], S);            // distance of the bfloat16 rows
         const float e1 = kappa * S;                                 // accumulation errors of G and the norms
         const float dhi = fmaxf(dt + e1, 0.0f);
-        const float Q = 2.0001f * S;
-        const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);   // rounding to bfloat16
-        const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;                 // <= result of the fp32 chain
-        const bool skip = lower >= limit;                           // false if anything is NaN
+        const float a = dt - e1 - kC2 * S - limit;
+        const bool skip = a >= 0.0f && a * a >= kC3 * dhi * S;      // false if anything is NaN
         if (m < n && n < s && !skip) bits |= 1u << i;
     }
     return bits;
@@ -84,16 +91,19 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                                                                    const int* __restrict__ sizes,
                                                                    int* __restrict__ knn_idx, float* __restrict__ knn_dist,
                                                                    int chunk, int pitch, int region_floats, int bpitch,
-                                                                   int ksteps, float kappa, float one_minus_gamma)
+                                                                   int ksteps, float kappa, float inv_one_minus_gamma)
 {
-    // dynamic LDS: [rows | triangular distance matrix] (region_floats) | ids[64] | tau[64] | nrm[64] | n_pairs | list
+    // dynamic LDS: [rows | triangular distance matrix] (region_floats) | ids[64] | tau[64] | taup[64] | nrm[64] |
+    //              n_pairs, active[2] | list
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
     float* tri = lds_f;                      // same storage, used after the last read of rows
     int* lids = reinterpret_cast<int*>(lds_f + region_floats);
     float* tau = reinterpret_cast<float*>(lids + kCap);
-    float* nrm = tau + kCap;
+    float* taup = tau + kCap;
+    float* nrm = taup + kCap;
     int* n_pairs = reinterpret_cast<int*>(nrm + kCap);
+    uint32_t* active_s = reinterpret_cast<uint32_t*>(n_pairs + 1);      // per wavefront: members with a candidate
     uint16_t* list = reinterpret_cast<uint16_t*>(n_pairs + 4);
 
     const int bkt = blockIdx.x;
@@ -105,25 +115,32 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
 
     if (tid < kCap) {
         const int id = tid < s ? bid[tid] : -1;
+        const float t = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
         lids[tid] = id;
-        tau[tid] = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
+        tau[tid] = t;
+        taup[tid] = (t + 1e-30f) * inv_one_minus_gamma;
         nrm[tid] = id >= 0 ? bnorms[id] : 0.0f;
     }
-    if (tid == 0) *n_pairs = 0;
+    if (tid < 4) n_pairs[tid] = 0;           // n_pairs, active[0], active[1]
     __syncthreads();
 
-    // fp32 rows of a slice: requested early, written to LDS when the previous slice has been consumed
-    float4 pre[kMaxLoads];
+    // fp32 rows of a slice: lane pc of a group of 16 loads piece pc of rows rg, rg + 8, ...; requested early,
+    // written to LDS when the previous slice has been consumed
+    const int pc = tid & (kLanesPerRow - 1), rg = tid / kLanesPerRow;
+    const float* rowp[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+        const int m = rg + kRowsPerStep * i;
+        rowp[i] = points + (size_t)lids[m < s ? m : 0] * (size_t)D + 4 * pc;
+    }
+    float4 pre[kLoads];
     auto request = [&](int d0) {
         const int np = min(chunk, (D - d0 + 3) & ~3) >> 2;      // 16-byte pieces per row in this slice
-        const int items = s * np;
 #pragma unroll
-        for (int i = 0; i < kMaxLoads; ++i) {
-            const int it = tid + i * kThreads;
+        for (int i = 0; i < kLoads; ++i) {
             pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (it < items) {
-                const int m = it / np, pc = it - m * np;
-                const float* src = points + (size_t)lids[m] * (size_t)D + d0 + 4 * pc;
+            if (pc < np && rg + kRowsPerStep * i < s) {
+                const float* src = rowp[i] + d0;
                 if (vec_ok) {
                     pre[i] = *reinterpret_cast<const float4*>(src);
                 } else {
@@ -173,7 +190,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             const int mbase = 32 * hx + 4 * (lane >> 5);
             for (int t = 0; t < (second ? 2 : 1); ++t) {
                 const int n = t == 0 ? mx : my;
-                uint32_t bits = screen_tile(t == 0 ? gxx : gxy, mbase, n, s, nrm, tau, kappa, one_minus_gamma);
+                uint32_t bits = screen_tile(t == 0 ? gxx : gxy, mbase, n, s, nrm, taup, kappa);
                 const int cnt = __popc(bits);
                 int at = cnt ? atomicAdd(n_pairs, cnt) : 0;
                 while (bits) {
@@ -201,13 +218,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     }
     for (int d0 = 0; d0 < D; d0 += chunk) {
         if (d0 > 0) __syncthreads();                 // the previous slice has been consumed
-        const int items = s * np;
+        if (pc < np) {
 #pragma unroll
-        for (int i = 0; i < kMaxLoads; ++i) {
-            const int it = tid + i * kThreads;
-            if (it < items) {
-                const int m = it / np, pc = it - m * np;
-                *reinterpret_cast<float4*>(&rows[m * pitch + 4 * pc]) = pre[i];
+            for (int i = 0; i < kLoads; ++i) {
+                const int m = rg + kRowsPerStep * i;
+                if (m < s) *reinterpret_cast<float4*>(&rows[m * pitch + 4 * pc]) = pre[i];
             }
         }
         const int np_now = np;
@@ -241,23 +256,24 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         const int p = tid + k * kThreads;
         if (p < n_list) {
             const uint32_t e = list[p];
-            tri[tri_at((int)(e & 63u), (int)(e >> 6))] = acc[k];
+            const int r = (int)(e & 63u), c = (int)(e >> 6);
+            const float d = acc[k];
+            tri[tri_at(r, c)] = d;
+            // member i belongs to wavefront i % 2 and is its bit i / 2
+            if (d < tau[r]) atomicOr(&active_s[r & 1], 1u << (r >> 1));
+            if (d < tau[c]) atomicOr(&active_s[c & 1], 1u << (c >> 1));
         }
     }
     __syncthreads();
 
-    // ---- 3. top-K update.  A wavefront owns every second member; first find the members that have a
-    //         candidate below their last slot, then walk those with the rows of the next two in flight.
+    // ---- 3. top-K update.  A wavefront owns every second member and walks those that have a candidate below
+    //         their last slot, with the rows of the next two in flight.
     const int my_id = lids[lane];
+    uint32_t active = active_s[wave];
     auto candidate = [&](int i) {
         const int a = min(i, lane), b = max(i, lane);
         return (lane < s && lane != i) ? tri[tri_at(a, b)] : INFINITY;
     };
-    uint32_t active = 0;
-    for (int u = 0; wave + kWaves * u < s; ++u) {
-        const int i = wave + kWaves * u;
-        if (ballot64(candidate(i) < tau[i]) != 0) active |= 1u << u;
-    }
     auto next_member = [&]() {
         if (active == 0) return -1;
         const int u = __ffs(active) - 1;
@@ -337,17 +353,18 @@ int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int
     RSFK_CHECK(kCap * pitch < 65536, "screened small-bucket kernel: LDS offsets must fit 16 bits");
     const int region = std::max(kCap * pitch, kMaxPairs);
     const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)(3 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(4 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
     const int ksteps = (bf16_valid(D) + 15) / 16;
     RSFK_CHECK(ksteps * 16 <= bf16_pitch(D), "screened small-bucket kernel: bfloat16 rows too short");
     const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21
     const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
     RSFK_CHECK(one_minus_gamma > 0.5f, "screened small-bucket kernel: D too large");
+    const float inv_one_minus_gamma = 1.000001f / one_minus_gamma;                  // rounded up
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_screen),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k_bucket_knn_screen, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, bf.rows,
                        bf.norms, D, K, ids, starts, sizes, knn_idx, knn_dist, chunk, pitch, region_floats,
-                       bf16_pitch(D), ksteps, kappa, one_minus_gamma);
+                       bf16_pitch(D), ksteps, kappa, inv_one_minus_gamma);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

@@ -73,13 +73,43 @@ __device__ __forceinline__ void make_hyperplane(const float* __restrict__ x1, co
     }
 }
 
+// The same by one wavefront (all 64 lanes call): normal zero padded to bf16_valid(D) values.
+__device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x1, const float* __restrict__ x2,
+                                                     int D, float* nvec, float* b_out)
+{
+    const int lane = lane_id();
+    const int Dv = bf16_valid(D);
+    for (int d = lane; d < Dv; d += 64) nvec[d] = d < D ? x1[d] - x2[d] : 0.0f;
+    float s = 0.0f;
+    if (lane < 32) {
+        for (int d = lane; d < D; d += 32) {
+            const float t1 = x1[d], t2 = x2[d];
+            const float nd = t1 - t2;
+            const float prod = nd * (t1 + t2);
+            s = s + prod * 0.5f;
+        }
+    }
+    s = half_butterfly_sum(s);
+    if (lane == 0) *b_out = s;
+}
+
 // n.x for one point by one half wavefront (32 lanes); every lane of the half
 // returns the same value.  hl = lane within the half.
 __device__ __forceinline__ float half_dot(const float* nvec, const float* __restrict__ x, int D, int hl, bool valid)
 {
+    // the chain of a lane runs over d = hl, hl + 32, ...; its loads are issued eight at a time so that the
+    // chain does not wait for memory once per element
     float s = 0.0f;
-    if (valid)
-        for (int d = hl; d < D; d += 32) s = __builtin_fmaf(nvec[d], x[d], s);
+    if (valid) {
+        for (int d0 = hl; d0 < D; d0 += 256) {
+            float xv[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) xv[k] = d0 + 32 * k < D ? x[d0 + 32 * k] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (d0 + 32 * k < D) s = __builtin_fmaf(nvec[d0 + 32 * k], xv[k], s);
+        }
+    }
     return half_butterfly_sum(s);
 }
 
@@ -97,64 +127,89 @@ __device__ __forceinline__ float half_dot(const float* nvec, const float* __rest
 // arithmetic, two at a time (one per half wavefront).  NaN or infinite values fail
 // the band test and take the exact path.  Without a bfloat16 copy every point takes
 // the exact path.
-__device__ __forceinline__ bool side_right8(const float* nvec, float b, const float* __restrict__ points,
-                                            const uint16_t* __restrict__ pb16, int id, int D, bool valid)
+//
+// NB points per group are handled per call, so that NB row gathers per lane are in flight before the
+// first is needed (the loop over points is bound by the latency of these gathers otherwise).
+template <int NB>
+__device__ __forceinline__ void side_right8(const float* nvec0, int nstride, const int (&j)[NB], const float (&b)[NB],
+                                            const float* __restrict__ points, const uint16_t* __restrict__ pb16,
+                                            const int (&id)[NB], int D, const bool (&valid)[NB], bool (&right)[NB])
 {
+    // hyperplane of point u of this group: normal nvec0 + j[u] * nstride, offset b[u] (groups may differ)
     const int lane = lane_id();
     const int sub = lane & 7;
-    bool right = false;
-    bool redo = valid;
+    bool redo[NB];
+#pragma unroll
+    for (int u = 0; u < NB; ++u) { right[u] = false; redo[u] = valid[u]; }
     if (pb16 != nullptr) {
         const int Dv = bf16_valid(D);
-        const uint16_t* row = pb16 + (size_t)id * (size_t)bf16_pitch(D);
-        float da = 0.0f, sa = 0.0f;
-        if (valid) {
-            for (int e = sub * 8; e < Dv; e += 64) {
-                const uint4 w = *reinterpret_cast<const uint4*>(row + e);
+        const size_t pitch = (size_t)bf16_pitch(D);
+        float da[NB], sa[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) { da[u] = 0.0f; sa[u] = 0.0f; }
+        for (int e = sub * 8; e < Dv; e += 64) {
+            uint4 w[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                w[u] = make_uint4(0u, 0u, 0u, 0u);
+                if (valid[u]) w[u] = *reinterpret_cast<const uint4*>(pb16 + (size_t)id[u] * pitch + e);
+            }
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const float* nvec = nvec0 + (size_t)j[u] * nstride;
                 const float4 n0 = *reinterpret_cast<const float4*>(&nvec[e]);
                 const float4 n1 = *reinterpret_cast<const float4*>(&nvec[e + 4]);
-                const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+                const uint32_t ww[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
                 const float nn[8] = {n0.x, n0.y, n0.z, n0.w, n1.x, n1.y, n1.z, n1.w};
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const float x0 = __uint_as_float(ww[q] << 16);
                     const float x1 = __uint_as_float(ww[q] & 0xffff0000u);
-                    da = __builtin_fmaf(nn[2 * q], x0, da);
-                    da = __builtin_fmaf(nn[2 * q + 1], x1, da);
-                    sa = __builtin_fmaf(fabsf(nn[2 * q]), fabsf(x0), sa);
-                    sa = __builtin_fmaf(fabsf(nn[2 * q + 1]), fabsf(x1), sa);
+                    da[u] = __builtin_fmaf(nn[2 * q], x0, da[u]);
+                    da[u] = __builtin_fmaf(nn[2 * q + 1], x1, da[u]);
+                    sa[u] = __builtin_fmaf(fabsf(nn[2 * q]), fabsf(x0), sa[u]);
+                    sa[u] = __builtin_fmaf(fabsf(nn[2 * q + 1]), fabsf(x1), sa[u]);
                 }
             }
         }
-        // sum over the 8 lanes of the group (any order will do for the screen)
-        da += dpp_f<kDppXor1>(da); da += dpp_f<kDppXor2>(da); da += dpp_f<kDppHalfMirror>(da);
-        sa += dpp_f<kDppXor1>(sa); sa += dpp_f<kDppXor2>(sa); sa += dpp_f<kDppHalfMirror>(sa);
-        const bool certain = fabsf(da - b) > sa * (1.02f / 256.0f) + 1e-30f;
-        right = da < b;
-        redo = valid && !certain;
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            // sum over the 8 lanes of the group (any order will do for the screen)
+            float d = da[u], a = sa[u];
+            d += dpp_f<kDppXor1>(d); d += dpp_f<kDppXor2>(d); d += dpp_f<kDppHalfMirror>(d);
+            a += dpp_f<kDppXor1>(a); a += dpp_f<kDppXor2>(a); a += dpp_f<kDppHalfMirror>(a);
+            const bool certain = fabsf(d - b[u]) > a * (1.02f / 256.0f) + 1e-30f;
+            right[u] = d < b[u];
+            redo[u] = valid[u] && !certain;
+        }
     }
     // exact test for the groups that need it, two per round (one per half wavefront)
-    uint64_t m = ballot64(redo);
-    while (m != 0) {
-        const int g1 = first_lane(m) >> 3;
-        m &= ~(0xffull << (8 * g1));
-        int g2 = -1;
-        if (m != 0) {
-            g2 = first_lane(m) >> 3;
-            m &= ~(0xffull << (8 * g2));
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+        uint64_t m = ballot64(redo[u]);
+        while (m != 0) {
+            const int g1 = first_lane(m) >> 3;
+            m &= ~(0xffull << (8 * g1));
+            int g2 = -1;
+            if (m != 0) {
+                g2 = first_lane(m) >> 3;
+                m &= ~(0xffull << (8 * g2));
+            }
+            const int l1 = 8 * g1, l2 = g2 >= 0 ? 8 * g2 : l1;
+            const bool upper = lane >= 32;
+            const int my = upper ? read_lane_i(id[u], l2) : read_lane_i(id[u], l1);
+            const int myj = upper ? read_lane_i(j[u], l2) : read_lane_i(j[u], l1);
+            const float myb = upper ? read_lane_f(b[u], l2) : read_lane_f(b[u], l1);
+            const bool live = upper ? g2 >= 0 : true;
+            const float dot = half_dot(nvec0 + (size_t)myj * nstride, points + (size_t)my * D, D, lane & 31, live);
+            const uint64_t res = ballot64(dot < myb);
+            if ((lane >> 3) == g1) right[u] = (res & 1ull) != 0;
+            if (g2 >= 0 && (lane >> 3) == g2) right[u] = ((res >> 32) & 1ull) != 0;
         }
-        const int id1 = read_lane_i(id, 8 * g1);
-        const int id2 = g2 >= 0 ? read_lane_i(id, 8 * g2) : id1;
-        const bool upper = lane >= 32;
-        const int my = upper ? id2 : id1;
-        const bool live = upper ? g2 >= 0 : true;
-        const float dot = half_dot(nvec, points + (size_t)my * D, D, lane & 31, live);
-        const uint64_t res = ballot64(dot < b);
-        if ((lane >> 3) == g1) right = (res & 1ull) != 0;
-        if (g2 >= 0 && (lane >> 3) == g2) right = ((res >> 32) & 1ull) != 0;
     }
-    return right;
 }
+
+constexpr int kSideBatch = 4;        // points per group and call of side_right8
 
 // Append a child node either to the next wide level or to the tail queue.
 __device__ __forceinline__ void emit_node(const TreeNode& c, const TreeParams& P, TreeNode* next, int next_cap,
@@ -300,14 +355,25 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     const int grp = threadIdx.x >> 3, sub8 = threadIdx.x & 7;      // 32 groups of 8 lanes, one point each
     const int iters = (pos1 - pos0 + kGroups - 1) / kGroups;
     int lefts = 0;
-    for (int it = 0; it < iters; ++it) {
-        const int pos = pos0 + it * kGroups + grp;
-        const bool valid = pos < pos1;
-        const int id = valid ? (perm[pos] & kIdMask) : 0;
-        const bool right = side_right8(nvec, b, points, pb16, id, P.D, valid);   // build_tree_check_points_side.cu:149
-        if (valid && sub8 == 0) {
-            perm[pos] = right ? (id | (int)0x80000000) : id;
-            lefts += right ? 0 : 1;
+    for (int it = 0; it < iters; it += kSideBatch) {
+        int id[kSideBatch], jz[kSideBatch], pos[kSideBatch];
+        float bb[kSideBatch];
+        bool valid[kSideBatch], right[kSideBatch];
+#pragma unroll
+        for (int u = 0; u < kSideBatch; ++u) {
+            pos[u] = pos0 + (it + u) * kGroups + grp;
+            valid[u] = pos[u] < pos1;
+            id[u] = valid[u] ? (perm[pos[u]] & kIdMask) : 0;
+            jz[u] = 0;
+            bb[u] = b;
+        }
+        side_right8<kSideBatch>(nvec, 0, jz, bb, points, pb16, id, P.D, valid, right);   // build_tree_check_points_side.cu:149
+#pragma unroll
+        for (int u = 0; u < kSideBatch; ++u) {
+            if (valid[u] && sub8 == 0) {
+                perm[pos[u]] = right[u] ? (id[u] | (int)0x80000000) : id[u];
+                lefts += right[u] ? 0 : 1;
+            }
         }
     }
     const int hl = sub8;
@@ -427,27 +493,35 @@ __device__ __forceinline__ void emit_leaf(int tree, int gstart, int count, int d
     atomicMin(&st->min_leaf, count);
 }
 
+constexpr int kMaxGroup = 16;        // nodes of one level of a subtree worked on together
+
+// One workgroup finishes the subtree of a task level by level: the nodes of a level are taken kMaxGroup (or
+// fewer, G) at a time -- their hyperplanes are made together (one wavefront each), all their points are tested in
+// one sweep, and each node is partitioned by one wavefront -- so the number of dependent trips to memory per
+// subtree is a few per level instead of a few per node.
 __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ points,
                                                  const uint16_t* __restrict__ pb16, TreeParams P,
                                                  const int* __restrict__ perm0, const int* __restrict__ perm1,
                                                  int* __restrict__ perm_out,
-                                                 const TreeNode* __restrict__ tasks, int n_tasks, int stack_cap,
+                                                 const TreeNode* __restrict__ tasks, int n_tasks, int node_cap, int G,
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr)
 {
-    // dynamic LDS: seg[small] | tmp[small] | nvec[bf16_valid(D)] | stack[stack_cap] | lrec[small]
+    // dynamic LDS: seg[small] | tmp[small] | nvec[G][bf16_valid(D)] | lrec[node_cap] | level lists 2 x node_cap | fmap[small]
     extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int Dv = bf16_valid(P.D);
     int* seg = reinterpret_cast<int*>(lds_raw);
     int* tmp = seg + P.small;
     float* nvec = reinterpret_cast<float*>(tmp + P.small);
-    SmallNode* stack = reinterpret_cast<SmallNode*>(lds_raw + ((size_t)(2 * P.small + bf16_valid(P.D)) * 4 + 15) / 16 * 16);
     // buckets of this subtree, written to the table of the tree together at the end (one reservation per
     // workgroup instead of one atomic round trip per bucket): x = start, y = size | rank among its kind << 16
-    int2* lrec = reinterpret_cast<int2*>(stack + stack_cap);
-    __shared__ float b_s;
-    __shared__ int left_s, top_s, base_s[2], nrec_s;
-    int n_small = 0, n_big = 0, lev = 0, mx = 0, mn = 0x7fffffff;      // thread 0 only
-    __shared__ int wcnt[kBlock / 64];
+    int2* lrec = reinterpret_cast<int2*>(nvec + (size_t)G * Dv);
+    SmallNode* cur = reinterpret_cast<SmallNode*>(lrec + node_cap);
+    SmallNode* nxt = cur + node_cap;
+    unsigned char* fmap = reinterpret_cast<unsigned char*>(nxt + node_cap);
+    __shared__ float b_s[kMaxGroup];
+    __shared__ int left_s[kMaxGroup], pre_s[kMaxGroup + 1], start_s[kMaxGroup], pair_s[kMaxGroup][2];
+    __shared__ int n_cur_s, n_nxt_s, nrec_s, kind_s[2], base_s[2], lev_s, mx_s, mn_s;
 
     const int task = blockIdx.x;
     if (task >= n_tasks) return;
@@ -469,104 +543,133 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         SmallNode r;
         r.start = 0; r.count = tk.count; r.dstart = tk.dstart - tk.start; r.dcount = tk.dcount;
         r.depth = tk.depth; r.leaf = 0; r.key = tk.key;
-        stack[0] = r;
-        top_s = 1;
+        cur[0] = r;
+        n_cur_s = 1; n_nxt_s = 0; nrec_s = 0; kind_s[0] = 0; kind_s[1] = 0; lev_s = 0; mx_s = 0; mn_s = 0x7fffffff;
     }
     __syncthreads();
 
-    const int hl = tid & 7;                 // lane within its group of 8
+    auto record_leaf = [&](int start, int count, int depth) {
+        const int at = atomicAdd(&nrec_s, 1);
+        const int rank = atomicAdd(&kind_s[count > kBucketSplit ? 1 : 0], 1);
+        if (at < node_cap) lrec[at] = make_int2(tk.start + start, count | (rank << 16)); else ctr->overflow = 1;
+        atomicMax(&lev_s, depth + 1);
+        atomicMax(&mx_s, count);
+        atomicMin(&mn_s, count);
+    };
+
+    const int grp = tid >> 3, sub8 = tid & 7;       // 32 groups of 8 lanes, one point each per iteration
     while (true) {
-        const int top = top_s;
-        if (top == 0) break;
-        const SmallNode nd = stack[top - 1];
-        __syncthreads();                      // everyone has read the top before it is overwritten
-        if (nd.leaf || nd.depth >= P.MAX_DEPTH - 1) {
+        const int n_cur = n_cur_s;
+        if (n_cur == 0) break;
+        for (int b0 = 0; b0 < n_cur; b0 += G) {
+            const int nb = min(G, n_cur - b0);
+            // the drawn pairs of the nodes of the group, and where their points sit in the flat numbering
+            if (tid < nb) {
+                const SmallNode nd = cur[b0 + tid];
+                int r1, r2;
+                pick_pair(nd.key, nd.dcount, r1, r2);
+                pair_s[tid][0] = seg[nd.dstart + r1];
+                pair_s[tid][1] = seg[nd.dstart + r2];
+                start_s[tid] = nd.start;
+            }
             if (tid == 0) {
-                const int rank = nd.count > kBucketSplit ? n_big++ : n_small++;
-                lrec[n_small + n_big - 1] = make_int2(tk.start + nd.start, nd.count | (rank << 16));
-                lev = max(lev, nd.depth + 1);
-                mx = max(mx, nd.count);
-                mn = min(mn, nd.count);
-                top_s = top - 1;
+                int run = 0;
+                for (int j = 0; j < nb; ++j) { pre_s[j] = run; run += cur[b0 + j].count; }
+                pre_s[nb] = run;
             }
             __syncthreads();
-            continue;
-        }
-        int r1, r2;
-        pick_pair(nd.key, nd.dcount, r1, r2);
-        const int p1 = seg[nd.dstart + r1], p2 = seg[nd.dstart + r2];
-        if (tid == 0) left_s = 0;
-        make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
-        __syncthreads();
-        const float b = b_s;
-        const int iters = (nd.count + kGroups - 1) / kGroups;
-        int lefts = 0;
-        for (int it = 0; it < iters; ++it) {
-            const int i = it * kGroups + (tid >> 3);
-            const bool valid = i < nd.count;
-            const int id = valid ? seg[nd.start + i] : 0;
-            const bool right = side_right8(nvec, b, points, pb16, id, P.D, valid);
-            if (valid && hl == 0) {
-                if (right) seg[nd.start + i] = id | (int)0x80000000; else ++lefts;
+            for (int j = wave; j < nb; j += kBlock / 64)
+                make_hyperplane_wave(points + (size_t)pair_s[j][0] * P.D, points + (size_t)pair_s[j][1] * P.D, P.D,
+                                     nvec + (size_t)j * Dv, &b_s[j]);
+            for (int j = 0; j < nb; ++j) {
+                const int c = pre_s[j + 1] - pre_s[j];
+                for (int t = tid; t < c; t += kBlock) fmap[pre_s[j] + t] = (unsigned char)j;
             }
-        }
-        if (hl == 0 && lefts) atomicAdd(&left_s, lefts);
-        __syncthreads();
-        const int a = left_s;
-        // stable partition seg[start..start+count) -> tmp -> seg
-        int lbase = 0;
-        for (int r0 = 0; r0 < nd.count; r0 += kBlock) {
-            const int i = r0 + tid;
-            const bool valid = i < nd.count;
-            const int v = valid ? seg[nd.start + i] : 0;
-            const bool right = v < 0;
-            const uint64_t m = ballot64(valid && !right);
-            if (lane == 0) wcnt[wave] = __popcll(m);
             __syncthreads();
-            int woff = 0, tot = 0;
+            // side of every point of the group's nodes
+            const int total = pre_s[nb];
+            const int iters = (total + kGroups - 1) / kGroups;
+            for (int it = 0; it < iters; it += kSideBatch) {
+                int id[kSideBatch], jj[kSideBatch], pos[kSideBatch];
+                float bb[kSideBatch];
+                bool valid[kSideBatch], right[kSideBatch];
 #pragma unroll
-            for (int w = 0; w < kBlock / 64; ++w) { const int x = wcnt[w]; if (w < wave) woff += x; tot += x; }
-            const int lrank = lbase + woff + mask_prefix(m);
-            if (valid) tmp[right ? a + i - lrank : lrank] = v & kIdMask;
-            lbase += tot;
+                for (int u = 0; u < kSideBatch; ++u) {
+                    const int f = (it + u) * kGroups + grp;
+                    valid[u] = f < total;
+                    jj[u] = valid[u] ? fmap[f] : 0;
+                    pos[u] = valid[u] ? start_s[jj[u]] + f - pre_s[jj[u]] : 0;
+                    id[u] = valid[u] ? seg[pos[u]] : 0;
+                    bb[u] = b_s[jj[u]];
+                }
+                side_right8<kSideBatch>(nvec, Dv, jj, bb, points, pb16, id, P.D, valid, right);
+#pragma unroll
+                for (int u = 0; u < kSideBatch; ++u)
+                    if (valid[u] && sub8 == 0 && right[u]) seg[pos[u]] = id[u] | (int)0x80000000;
+            }
+            __syncthreads();
+            // stable partition, one wavefront per node: seg -> tmp -> seg
+            for (int j = wave; j < nb; j += kBlock / 64) {
+                const int st = start_s[j], cnt = pre_s[j + 1] - pre_s[j];
+                int a = 0;
+                for (int r0 = 0; r0 < cnt; r0 += 64) a += __popcll(ballot64(r0 + lane < cnt && seg[st + r0 + lane] >= 0));
+                int lbase = 0;
+                for (int r0 = 0; r0 < cnt; r0 += 64) {
+                    const int i = r0 + lane;
+                    const bool valid = i < cnt;
+                    const int v = valid ? seg[st + i] : 0;
+                    const bool right = v < 0;
+                    const uint64_t m = ballot64(valid && !right);
+                    const int lrank = lbase + mask_prefix(m);
+                    if (valid) tmp[st + (right ? a + i - lrank : lrank)] = v & kIdMask;
+                    lbase += __popcll(m);
+                }
+                wave_lds_sync();
+                for (int i = lane; i < cnt; i += 64) seg[st + i] = tmp[st + i];
+                if (lane == 0) left_s[j] = a;
+            }
+            __syncthreads();
+            // children: buckets are recorded, the others wait for the next level
+            if (tid < nb) {
+                const SmallNode nd = cur[b0 + tid];
+                TreeNode full, c[2];
+                full.tree = tk.tree; full.start = nd.start; full.count = nd.count; full.dstart = nd.dstart;
+                full.dcount = nd.dcount; full.depth = nd.depth; full.buf = 0; full.leaf = 0; full.key = nd.key;
+                const int nc = split_rules(full, left_s[tid], P.MIN, P.MAX, 0, c[0], c[1]);
+                for (int q = 0; q < nc; ++q) {
+                    if (c[q].leaf || c[q].depth >= P.MAX_DEPTH - 1) {
+                        record_leaf(c[q].start, c[q].count, c[q].depth);
+                    } else {
+                        const int at = atomicAdd(&n_nxt_s, 1);
+                        if (at < node_cap) {
+                            SmallNode sn;
+                            sn.start = c[q].start; sn.count = c[q].count; sn.dstart = c[q].dstart; sn.dcount = c[q].dcount;
+                            sn.depth = c[q].depth; sn.leaf = 0; sn.key = c[q].key;
+                            nxt[at] = sn;
+                        } else {
+                            ctr->overflow = 1;
+                        }
+                    }
+                }
+            }
             __syncthreads();
         }
-        for (int i = tid; i < nd.count; i += kBlock) seg[nd.start + i] = tmp[i];
-        if (tid == 0) {
-            TreeNode full, c0, c1;
-            full.tree = tk.tree; full.start = nd.start; full.count = nd.count; full.dstart = nd.dstart;
-            full.dcount = nd.dcount; full.depth = nd.depth; full.buf = 0; full.leaf = 0; full.key = nd.key;
-            const int nc = split_rules(full, a, P.MIN, P.MAX, 0, c0, c1);
-            int t = top - 1;
-            // right child below the left one: leaves come out left to right
-            if (nc == 2) {
-                if (t < stack_cap) {
-                    SmallNode s1; s1.start = c1.start; s1.count = c1.count; s1.dstart = c1.dstart; s1.dcount = c1.dcount;
-                    s1.depth = c1.depth; s1.leaf = c1.leaf; s1.key = c1.key;
-                    stack[t++] = s1;
-                } else ctr->overflow = 1;
-            }
-            if (t < stack_cap) {
-                SmallNode s0; s0.start = c0.start; s0.count = c0.count; s0.dstart = c0.dstart; s0.dcount = c0.dcount;
-                s0.depth = c0.depth; s0.leaf = c0.leaf; s0.key = c0.key;
-                stack[t++] = s0;
-            } else ctr->overflow = 1;
-            top_s = t;
-        }
+        if (tid == 0) { n_cur_s = min(n_nxt_s, node_cap); n_nxt_s = 0; }
+        SmallNode* t = cur; cur = nxt; nxt = t;
         __syncthreads();
     }
     for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = seg[i];
     if (tid == 0) {
         TreeStats* st = stats + tk.tree;
-        base_s[0] = n_small ? atomicAdd(&st->n_leaves, n_small) : 0;
-        base_s[1] = n_big ? atomicAdd(&st->n_big, n_big) : 0;
-        nrec_s = n_small + n_big;
-        atomicMax(&st->levels, lev);
-        atomicMax(&st->max_leaf, mx);
-        atomicMin(&st->min_leaf, mn);
+        base_s[0] = kind_s[0] ? atomicAdd(&st->n_leaves, kind_s[0]) : 0;
+        base_s[1] = kind_s[1] ? atomicAdd(&st->n_big, kind_s[1]) : 0;
+        atomicMax(&st->levels, lev_s);
+        atomicMax(&st->max_leaf, mx_s);
+        atomicMin(&st->min_leaf, mn_s);
     }
     __syncthreads();
-    for (int i = tid; i < nrec_s; i += kBlock) {
+    const int nrec = min(nrec_s, node_cap);
+    for (int i = tid; i < nrec; i += kBlock) {
         const int2 r = lrec[i];
         const int count = r.y & 0xffff, rank = r.y >> 16;
         store_leaf(tk.tree, r.x, count, base_s[count > kBucketSplit ? 1 : 0] + rank, leaf_cap, leaf_start, leaf_size, ctr);
@@ -719,12 +822,16 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     const int n_tail = w->h_ctr->n_tail;
     RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
     if (n_tail > 0) {
-        const int stack_cap = P.small / std::max(MIN, 1) + 4;
-        const size_t lds = ((size_t)(2 * P.small + bf16_valid(D)) * 4 + 15) / 16 * 16 + (size_t)stack_cap * sizeof(SmallNode) + (size_t)P.small * sizeof(int2);
+        // nodes of a level of a subtree (and its buckets): at most small / MIN + 1; hyperplanes kept together:
+        // as many as 24 KB hold, at most kMaxGroup
+        const int node_cap = P.small / std::max(MIN, 1) + 4;
+        const int G = std::max(1, std::min(kMaxGroup, (int)(24 * 1024 / ((size_t)bf16_valid(D) * 4))));
+        const size_t lds = (size_t)(2 * P.small) * 4 + (size_t)G * bf16_valid(D) * 4 + (size_t)node_cap * sizeof(int2) +
+                           2 * (size_t)node_cap * sizeof(SmallNode) + (size_t)P.small;
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
-                           w->tail, n_tail, stack_cap, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr);
+                           w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr);
         RSFK_HIP(hipGetLastError());
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
