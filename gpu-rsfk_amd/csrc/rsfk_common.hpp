@@ -103,6 +103,7 @@ struct TreeParams {
     int MIN, MAX, MAX_DEPTH;
     int small;        // nodes with at most this many points are finished by one workgroup
     int chunk;        // points per workgroup in the wide (global) passes
+    float band;       // half-width of the undecided band of the bfloat16 side screen, relative to sum |n_d||x~_d|
 };
 
 }  // namespace rsfk

@@ -93,52 +93,30 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
     if (lane == 0) *b_out = s;
 }
 
-// n.x for one point by one half wavefront (32 lanes); every lane of the half
-// returns the same value.  hl = lane within the half.
-__device__ __forceinline__ float half_dot(const float* nvec, const float* __restrict__ x, int D, int hl, bool valid)
-{
-    // the chain of a lane runs over d = hl, hl + 32, ...; its loads are issued eight at a time so that the
-    // chain does not wait for memory once per element
-    float s = 0.0f;
-    if (valid) {
-        for (int d0 = hl; d0 < D; d0 += 256) {
-            float xv[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) xv[k] = d0 + 32 * k < D ? x[d0 + 32 * k] : 0.0f;
-#pragma unroll
-            for (int k = 0; k < 8; ++k)
-                if (d0 + 32 * k < D) s = __builtin_fmaf(nvec[d0 + 32 * k], xv[k], s);
-        }
-    }
-    return half_butterfly_sum(s);
-}
-
-// Sides of eight points per wavefront (true = right, n.x < b): lanes 8g..8g+7 work on
+// Screen of the side test for eight points per wavefront (right = n.x < b): lanes 8g..8g+7 work on
 // the point of group g; all lanes of a group return its answer.
 //
-// The decision is always the one of the fp32 test above (half_dot), but most points
-// never touch their fp32 row: a bfloat16 copy of the row (half the bytes) gives an
-// approximate n.x together with S~ = sum |n_d||x~_d|.  bfloat16 keeps 8 significant
-// bits: rounding x to x~ (round to nearest) changes n.x by at most
-// 2^-8 sum |n_d||x_d| <= 2^-8 (1+2^-7) S~, and the fp32 summations of either path are
-// off by a few 2^-24 S~, so whenever |approx - b| > 1.02 * 2^-8 S~ the sign of
-// (n.x - b) is the same for the exact fp32 evaluation.  Only the points inside that
-// band (a few per cent) read the fp32 row and repeat the test with the exact
-// arithmetic, two at a time (one per half wavefront).  NaN or infinite values fail
-// the band test and take the exact path.  Without a bfloat16 copy every point takes
-// the exact path.
+// The decision is always the one of the exact fp32 test (resolve_exact below: 32 lane-strided fused
+// multiply-add chains + xor butterfly, build_tree_check_points_side.cu:131-149), but most points never
+// touch their fp32 row: a bfloat16 copy of the row (half the bytes) gives an approximate n.x together
+// with S~ = sum |n_d||x~_d|.  bfloat16 keeps 8 significant bits: rounding x to x~ (round to nearest)
+// changes n.x by at most 2^-8 sum |n_d||x_d| <= 2^-8 (1+2^-7) S~, and the fp32 summations of the two
+// paths are off by at most (D/8 + D/32 + 16) 2^-24 S~ together, so whenever |approx - b| exceeds
+// `band` * S~ (band = 1.01 (2^-8 (1+2^-7) + (D/8 + D/32 + 16) 2^-24), computed by the caller) the sign of
+// (n.x - b) is the same for the exact evaluation: right[u] is final.  Otherwise (a few per cent of the
+// points; also NaN or infinite values, and every point when there is no bfloat16 copy) redo[u] is set and
+// the caller hands the point to resolve_exact.
 //
 // NB points per group are handled per call, so that NB row gathers per lane are in flight before the
 // first is needed (the loop over points is bound by the latency of these gathers otherwise).
 template <int NB>
-__device__ __forceinline__ void side_right8(const float* nvec0, int nstride, const int (&j)[NB], const float (&b)[NB],
-                                            const float* __restrict__ points, const uint16_t* __restrict__ pb16,
-                                            const int (&id)[NB], int D, const bool (&valid)[NB], bool (&right)[NB])
+__device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, const int (&j)[NB], const float (&b)[NB],
+                                             const uint16_t* __restrict__ pb16, const int (&id)[NB], int D, float band,
+                                             const bool (&valid)[NB], bool (&right)[NB], bool (&redo)[NB])
 {
     // hyperplane of point u of this group: normal nvec0 + j[u] * nstride, offset b[u] (groups may differ)
     const int lane = lane_id();
     const int sub = lane & 7;
-    bool redo[NB];
 #pragma unroll
     for (int u = 0; u < NB; ++u) { right[u] = false; redo[u] = valid[u]; }
     if (pb16 != nullptr) {
@@ -178,33 +156,53 @@ __device__ __forceinline__ void side_right8(const float* nvec0, int nstride, con
             float d = da[u], a = sa[u];
             d += dpp_f<kDppXor1>(d); d += dpp_f<kDppXor2>(d); d += dpp_f<kDppHalfMirror>(d);
             a += dpp_f<kDppXor1>(a); a += dpp_f<kDppXor2>(a); a += dpp_f<kDppHalfMirror>(a);
-            const bool certain = fabsf(d - b[u]) > a * (1.02f / 256.0f) + 1e-30f;
+            const bool certain = fabsf(d - b[u]) > a * band + 1e-30f;
             right[u] = d < b[u];
             redo[u] = valid[u] && !certain;
         }
     }
-    // exact test for the groups that need it, two per round (one per half wavefront)
+}
+
+// Exact side tests for the points the screen could not decide: n.x by one half wavefront (32 lanes, lane hl
+// runs the chain over d = hl, hl + 32, ...; the loads of a chain are issued eight at a time), then the xor butterfly.  list[i] = position of the
+// point (local to the caller) | slot of its node << 16.  One half wavefront per point, two points per half
+// wavefront at a time so that their row loads overlap; all threads of the workgroup call.  id_at(pos) gives the
+// point, apply(pos, right) receives the answer in lane 0 of the half wavefront.
+template <typename IdAt, typename Apply>
+__device__ __forceinline__ void resolve_exact(const int* list, int n, const float* nvec0, int nstride, const float* b_of,
+                                              const float* __restrict__ points, int D, IdAt id_at, Apply apply)
+{
+    const int halves = blockDim.x >> 5;
+    const int h = threadIdx.x >> 5, hl = threadIdx.x & 31;
+    for (int base = 0; base < n; base += 2 * halves) {
+        const int ia = base + h, ib = base + halves + h;
+        const bool va = ia < n, vb = ib < n;
+        const int ea = va ? list[ia] : 0, eb = vb ? list[ib] : 0;
+        const float* xa = points + (size_t)id_at(ea & 0xffff) * D;
+        const float* xb = points + (size_t)id_at(eb & 0xffff) * D;
+        const float* na = nvec0 + (size_t)(ea >> 16) * nstride;
+        const float* nb = nvec0 + (size_t)(eb >> 16) * nstride;
+        float sa = 0.0f, sb = 0.0f;
+        for (int d0 = hl; d0 < D; d0 += 256) {
+            float xv[8], yv[8];
 #pragma unroll
-    for (int u = 0; u < NB; ++u) {
-        uint64_t m = ballot64(redo[u]);
-        while (m != 0) {
-            const int g1 = first_lane(m) >> 3;
-            m &= ~(0xffull << (8 * g1));
-            int g2 = -1;
-            if (m != 0) {
-                g2 = first_lane(m) >> 3;
-                m &= ~(0xffull << (8 * g2));
+            for (int k = 0; k < 8; ++k) {
+                xv[k] = (va && d0 + 32 * k < D) ? xa[d0 + 32 * k] : 0.0f;
+                yv[k] = (vb && d0 + 32 * k < D) ? xb[d0 + 32 * k] : 0.0f;
             }
-            const int l1 = 8 * g1, l2 = g2 >= 0 ? 8 * g2 : l1;
-            const bool upper = lane >= 32;
-            const int my = upper ? read_lane_i(id[u], l2) : read_lane_i(id[u], l1);
-            const int myj = upper ? read_lane_i(j[u], l2) : read_lane_i(j[u], l1);
-            const float myb = upper ? read_lane_f(b[u], l2) : read_lane_f(b[u], l1);
-            const bool live = upper ? g2 >= 0 : true;
-            const float dot = half_dot(nvec0 + (size_t)myj * nstride, points + (size_t)my * D, D, lane & 31, live);
-            const uint64_t res = ballot64(dot < myb);
-            if ((lane >> 3) == g1) right[u] = (res & 1ull) != 0;
-            if (g2 >= 0 && (lane >> 3) == g2) right[u] = ((res >> 32) & 1ull) != 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                if (d0 + 32 * k < D) {
+                    sa = __builtin_fmaf(na[d0 + 32 * k], xv[k], sa);
+                    sb = __builtin_fmaf(nb[d0 + 32 * k], yv[k], sb);
+                }
+            }
+        }
+        sa = half_butterfly_sum(sa);
+        sb = half_butterfly_sum(sb);
+        if (hl == 0) {
+            if (va) apply(ea & 0xffff, sa < b_of[ea >> 16]);
+            if (vb) apply(eb & 0xffff, sb < b_of[eb >> 16]);
         }
     }
 }
@@ -334,7 +332,8 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
 {
     extern __shared__ __align__(16) float nvec[];          // bf16_valid(D) floats
     __shared__ float b_s;
-    __shared__ int left_s;
+    __shared__ int left_s, n_def_s;
+    __shared__ int deferred[1024];                          // points of the chunk left to the exact test (chunk <= 1024)
     const int c = blockIdx.x;
     const int ni = chunk2node[c];
     const TreeNode nd = nodes[ni];
@@ -344,7 +343,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     pick_pair(nd.key, nd.dcount, r1, r2);
     const int p1 = perm[nd.dstart + r1] & kIdMask;
     const int p2 = perm[nd.dstart + r2] & kIdMask;
-    if (threadIdx.x == 0) left_s = 0;
+    if (threadIdx.x == 0) { left_s = 0; n_def_s = 0; }
     // p1/p2 must be read by every workgroup of the node before any of them sets
     // side bits; masking with kIdMask makes the read independent of that order.
     make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
@@ -358,7 +357,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     for (int it = 0; it < iters; it += kSideBatch) {
         int id[kSideBatch], jz[kSideBatch], pos[kSideBatch];
         float bb[kSideBatch];
-        bool valid[kSideBatch], right[kSideBatch];
+        bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
             pos[u] = pos0 + (it + u) * kGroups + grp;
@@ -367,17 +366,28 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
             jz[u] = 0;
             bb[u] = b;
         }
-        side_right8<kSideBatch>(nvec, 0, jz, bb, points, pb16, id, P.D, valid, right);   // build_tree_check_points_side.cu:149
+        side_screen8<kSideBatch>(nvec, 0, jz, bb, pb16, id, P.D, P.band, valid, right, redo);
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
             if (valid[u] && sub8 == 0) {
-                perm[pos[u]] = right[u] ? (id[u] | (int)0x80000000) : id[u];
-                lefts += right[u] ? 0 : 1;
+                if (redo[u]) {
+                    deferred[atomicAdd(&n_def_s, 1)] = pos[u] - pos0;
+                } else {
+                    perm[pos[u]] = right[u] ? (id[u] | (int)0x80000000) : id[u];
+                    lefts += right[u] ? 0 : 1;
+                }
             }
         }
     }
-    const int hl = sub8;
-    if (hl == 0 && lefts) atomicAdd(&left_s, lefts);
+    __syncthreads();
+    resolve_exact(deferred, n_def_s, nvec, 0, &b_s, points, P.D,
+                  [&](int local) { return perm[pos0 + local] & kIdMask; },
+                  [&](int local, bool right) {
+                      const int id = perm[pos0 + local] & kIdMask;
+                      perm[pos0 + local] = right ? (id | (int)0x80000000) : id;      // build_tree_check_points_side.cu:149
+                      lefts += right ? 0 : 1;
+                  });
+    if (lefts) atomicAdd(&left_s, lefts);
     __syncthreads();
     if (threadIdx.x == 0) chunk_left[c] = left_s;
 }
@@ -521,7 +531,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     unsigned char* fmap = reinterpret_cast<unsigned char*>(nxt + node_cap);
     __shared__ float b_s[kMaxGroup];
     __shared__ int left_s[kMaxGroup], pre_s[kMaxGroup + 1], start_s[kMaxGroup], pair_s[kMaxGroup][2];
-    __shared__ int n_cur_s, n_nxt_s, nrec_s, kind_s[2], base_s[2], lev_s, mx_s, mn_s;
+    __shared__ int n_cur_s, n_nxt_s, nrec_s, kind_s[2], base_s[2], lev_s, mx_s, mn_s, n_def_s;
 
     const int task = blockIdx.x;
     if (task >= n_tasks) return;
@@ -573,6 +583,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                 start_s[tid] = nd.start;
             }
             if (tid == 0) {
+                n_def_s = 0;
                 int run = 0;
                 for (int j = 0; j < nb; ++j) { pre_s[j] = run; run += cur[b0 + j].count; }
                 pre_s[nb] = run;
@@ -592,7 +603,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
             for (int it = 0; it < iters; it += kSideBatch) {
                 int id[kSideBatch], jj[kSideBatch], pos[kSideBatch];
                 float bb[kSideBatch];
-                bool valid[kSideBatch], right[kSideBatch];
+                bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
 #pragma unroll
                 for (int u = 0; u < kSideBatch; ++u) {
                     const int f = (it + u) * kGroups + grp;
@@ -602,11 +613,18 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                     id[u] = valid[u] ? seg[pos[u]] : 0;
                     bb[u] = b_s[jj[u]];
                 }
-                side_right8<kSideBatch>(nvec, Dv, jj, bb, points, pb16, id, P.D, valid, right);
+                side_screen8<kSideBatch>(nvec, Dv, jj, bb, pb16, id, P.D, P.band, valid, right, redo);
 #pragma unroll
-                for (int u = 0; u < kSideBatch; ++u)
-                    if (valid[u] && sub8 == 0 && right[u]) seg[pos[u]] = id[u] | (int)0x80000000;
+                for (int u = 0; u < kSideBatch; ++u) {
+                    if (valid[u] && sub8 == 0) {
+                        if (redo[u]) tmp[atomicAdd(&n_def_s, 1)] = pos[u] | (jj[u] << 16);      // tmp is free until the partition
+                        else if (right[u]) seg[pos[u]] = id[u] | (int)0x80000000;
+                    }
+                }
             }
+            __syncthreads();
+            resolve_exact(tmp, n_def_s, nvec, Dv, b_s, points, P.D, [&](int pos) { return seg[pos] & kIdMask; },
+                          [&](int pos, bool right) { if (right) seg[pos] |= (int)0x80000000; });
             __syncthreads();
             // stable partition, one wavefront per node: seg -> tmp -> seg
             for (int j = wave; j < nb; j += kBlock / 64) {
@@ -779,6 +797,10 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     P.N = N; P.D = D; P.MIN = MIN; P.MAX = MAX; P.MAX_DEPTH = MAX_DEPTH;
     P.small = tree_small_threshold();
     P.chunk = P.small;
+    RSFK_CHECK(P.chunk <= 1024, "tree batch: chunk size");
+    // bfloat16 rounding 2^-8 (1 + 2^-7), plus the summation errors of the screen (D/8 terms per lane and a 3-step
+    // tree) and of the exact test (D/32 terms per lane and a 5-step tree), 1 % on top
+    P.band = 1.01f * ((1.0f + 1.0f / 128.0f) / 256.0f + (float)(D / 8 + D / 32 + 16) / 16777216.0f);
 
     {
         const size_t total = (size_t)N * nb;
