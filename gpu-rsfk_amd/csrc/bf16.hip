@@ -33,7 +33,104 @@ __global__ __launch_bounds__(256) void k_to_bf16(const float* __restrict__ point
     }
 }
 
+// one wavefront per row of the 8-bit copy
+__global__ __launch_bounds__(256) void k_to_q8(const float* __restrict__ points, uint8_t* __restrict__ out,
+                                               float* __restrict__ rho_sum, int N, int D, int pitch, float c_d)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int n_waves = (gridDim.x * blockDim.x) >> 6;
+    float rho_acc = 0.0f;
+    for (int r = wave_global; r < N; r += n_waves) {
+        const float* src = points + (size_t)r * (size_t)D;
+        uint8_t* dst = out + (size_t)r * (size_t)pitch;
+        float lo = INFINITY, hi = -INFINITY, sabs = 0.0f;
+        bool bad = false;
+        for (int d = lane; d < D; d += 64) {
+            const float x = src[d];
+            bad |= !(fabsf(x) <= 3.0e38f);                 // NaN or infinite
+            lo = fminf(lo, x);
+            hi = fmaxf(hi, x);
+            sabs += fabsf(x);
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, o, 64));
+            hi = fmaxf(hi, __shfl_xor(hi, o, 64));
+            sabs += __shfl_xor(sabs, o, 64);
+        }
+        bad = __ballot(bad) != 0;
+        const float range = hi - lo;
+        const float scale = range * (1.0f / 255.0f);
+        const float inv = range > 0.0f ? 255.0f / range : 0.0f;
+        float err = 0.0f;
+        for (int d = lane; d < pitch - 16; d += 64) {
+            uint8_t q = 0;
+            if (d < D) {
+                const float x = src[d];
+                float t = __builtin_rintf((x - lo) * inv);
+                t = fminf(fmaxf(t, 0.0f), 255.0f);
+                q = (uint8_t)t;
+                err = fmaxf(err, fabsf(x - __builtin_fmaf(scale, t, lo)));
+            }
+            dst[16 + d] = q;
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) err = fmaxf(err, __shfl_xor(err, o, 64));
+        // err was measured against fl(lo + scale q); the screen evaluates lo sum n + scale sum n q in fp32 and is
+        // compared with an fp32 evaluation of n.x: all of that stays below c_d (|lo| + 255 scale) per unit of ||n||_1
+        const float mag = fabsf(lo) + 255.0f * scale;
+        float e1 = 1.01f * err + c_d * mag + 1e-37f;
+        if (bad || !(range <= 3.0e38f)) e1 = __builtin_nanf("");      // the screen never decides for such a row
+        if (lane == 0) {
+            float* head = reinterpret_cast<float*>(dst);
+            head[0] = 0.0f;
+            head[1] = lo;
+            head[2] = scale;
+            head[3] = e1;
+            const float bf = sabs / (float)D * (1.0f / 256.0f);
+            rho_acc += (e1 == e1 && bf > 0.0f) ? fminf(e1 / bf, 1000.0f) : 1000.0f;
+        }
+    }
+    if (lane == 0 && rho_acc != 0.0f) atomicAdd(rho_sum, rho_acc);
+}
+
 }  // namespace
+
+int q8_copy_alloc(Q8Copy* c, int N, int D)
+{
+    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * q8_pitch(D), 64)));
+    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->rho_sum), 16));
+    return 0;
+}
+
+void q8_copy_free(Q8Copy* c)
+{
+    if (c->rows) (void)hipFree(c->rows);
+    if (c->rho_sum) (void)hipFree(c->rho_sum);
+    c->rows = nullptr;
+    c->rho_sum = nullptr;
+}
+
+int q8_copy_fill(const Q8Copy& c, const float* points, int N, int D, hipStream_t stream)
+{
+    RSFK_HIP(hipMemsetAsync(c.rho_sum, 0, sizeof(float), stream));
+    const int grid = std::min((N + 3) / 4, 65536);
+    // (D/8 + D/32 + D + 32) 2^-24: chains of the screen and of the exact test, sum of the normal, rounding of lo + scale q
+    const float c_d = (float)(D / 8 + D / 32 + D + 32) / 16777216.0f;
+    hipLaunchKernelGGL(k_to_q8, dim3(grid), dim3(256), 0, stream, points, c.rows, c.rho_sum, N, D, q8_pitch(D), c_d);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+int q8_copy_mean_rho(const Q8Copy& c, int N, float* mean_rho, hipStream_t stream)
+{
+    float sum = 0.0f;
+    RSFK_HIP(hipMemcpyAsync(&sum, c.rho_sum, sizeof(float), hipMemcpyDeviceToHost, stream));
+    RSFK_HIP(hipStreamSynchronize(stream));
+    *mean_rho = N > 0 ? sum / (float)N : 0.0f;
+    return 0;
+}
 
 size_t bf16_copy_bytes(int N, int D) { return (size_t)N * ((size_t)bf16_pitch(D) * 2 + 4); }
 

@@ -24,6 +24,29 @@ struct Bf16Copy {
     float* norms = nullptr;       // N
 };
 
+// 8-bit screening copy of the points, used by the side test of the tree build when the rows have a narrow
+// range of values (half the bytes of the bfloat16 copy).
+//
+// Row p, q8_pitch(D) bytes on a 64-byte boundary: a 16-byte header (pad, lo, scale, e1 as four floats), then one
+// byte per coordinate, q_d = round((x_d - lo) / scale) in 0..255 with lo = min_d x_d and scale = (max_d x_d - lo) / 255,
+// zeros up to the end of the row.  e1 bounds what the quantisation can do to a dot product per unit of the
+// 1-norm of the other vector: for any n, |n.x - (lo sum_d n_d + scale sum_d n_d q_d)| <= e1 ||n||_1, including
+// the fp32 evaluation of either side with at most D/8-term chains (see k_to_q8).  mean_rho (host, after
+// q8_copy_fill has completed) compares e1 with the corresponding quantity of the bfloat16 copy,
+// 2^-8 mean_d |x_d|, averaged over the rows: the 8-bit copy pays off while it is below about 6.
+__host__ __device__ inline int q8_pitch(int D) { return (16 + D + 63) & ~63; }
+__host__ __device__ inline int q8_padded(int D) { return (D + 15) & ~15; }      // coordinates in whole 16-byte pieces
+
+struct Q8Copy {
+    uint8_t* rows = nullptr;      // N x q8_pitch(D)
+    float* rho_sum = nullptr;     // device scalar: sum over the rows of e1 / (2^-8 mean |x_d|)
+};
+
+int q8_copy_alloc(Q8Copy* c, int N, int D);
+void q8_copy_free(Q8Copy* c);
+int q8_copy_fill(const Q8Copy& c, const float* points, int N, int D, hipStream_t stream);
+int q8_copy_mean_rho(const Q8Copy& c, int N, float* mean_rho, hipStream_t stream);     // synchronises the stream
+
 size_t bf16_copy_bytes(int N, int D);
 int bf16_copy_alloc(Bf16Copy* c, int N, int D);
 void bf16_copy_free(Bf16Copy* c);

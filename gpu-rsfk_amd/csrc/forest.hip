@@ -68,9 +68,33 @@ struct ExploreWsGuard {
     ExploreWorkspace* w = nullptr;
     ~ExploreWsGuard() { explore_ws_free(w); }
 };
+struct Q8Guard {
+    Q8Copy c;
+    ~Q8Guard() { q8_copy_free(&c); }
+};
 struct EventPair {
     hipEvent_t a = nullptr, b = nullptr;
 };
+
+// Side tests of the trees are screened on the 8-bit copy when its quantisation error is within a small factor
+// of the bfloat16 rounding error on these points (half the bytes per row), else on the bfloat16 copy.
+// RSFK_TREE_SCREEN=q8 / bf16 forces one of them.  *rows = the 8-bit rows, or null for the bfloat16 screen.
+int make_tree_screen(Q8Guard& q8, const float* d_points, int N, int D, int verbose, hipStream_t stream, const uint8_t** rows)
+{
+    *rows = nullptr;
+    const char* env_tree = std::getenv("RSFK_TREE_SCREEN");
+    const bool force_bf16 = env_tree && env_tree[0] == 'b';
+    const bool force_q8 = env_tree && env_tree[0] == 'q';
+    if (force_bf16) return 0;
+    if (q8_copy_alloc(&q8.c, N, D) || q8_copy_fill(q8.c, d_points, N, D, stream)) return 1;
+    float rho = 0.0f;
+    if (q8_copy_mean_rho(q8.c, N, &rho, stream)) return 1;
+    if (force_q8 || rho <= 6.0f) *rows = q8.c.rows;
+    if (verbose >= 2)
+        std::printf("8-bit copy: quantisation error %.2f x bfloat16 rounding error -> %s screen\n", rho,
+                    *rows ? "8-bit" : "bfloat16");
+    return 0;
+}
 
 }  // namespace
 
@@ -92,6 +116,10 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     const char* env_screen = std::getenv("RSFK_BUCKET_SCREEN");
     const bool screen = K <= 64 && env_screen && env_screen[0] == '1';
 
+    Q8Guard q8;
+    const uint8_t* q8_rows = nullptr;
+    if (n_trees > 0 && make_tree_screen(q8, d_points, N, D, verbose, stream, &q8_rows)) return 1;
+
     if (n_trees > 0) {
         // the screened kernel reads a row's maximum from its last slot: rows the caller passed in unsorted are
         // put in order once
@@ -106,7 +134,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         for (int t0 = 0; t0 < n_trees && rc == 0; t0 += B) {
             const int nb = std::min(B, n_trees - t0);
             const double tb0 = now_s();
-            rc = build_tree_batch(ws.w, d_points, bf.c.rows, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
+            rc = build_tree_batch(ws.w, d_points, bf.c.rows, q8_rows, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
             if (rc) break;
             const double tb = now_s() - tb0;
             for (int j = 0; j < nb && rc == 0; ++j) {
@@ -191,7 +219,10 @@ int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int M
     Bf16Guard bf;
     if (bf16_copy_alloc(&bf.c, N, D)) return 1;
     if (bf16_copy_fill(bf.c, d_points, N, D, nullptr)) return 1;
-    if (build_tree_batch(ws.w, d_points, bf.c.rows, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
+    Q8Guard q8;
+    const uint8_t* q8_rows = nullptr;
+    if (make_tree_screen(q8, d_points, N, D, 0, nullptr, &q8_rows)) return 1;
+    if (build_tree_batch(ws.w, d_points, bf.c.rows, q8_rows, N, D, MIN, MAX, MAX_DEPTH, seed, 1, stats, nullptr)) return 1;
     const int nl = stats[0], n_big = stats[4], n_small = nl - n_big, cap = tree_ws_leaf_cap(ws.w);
     perm.resize((size_t)N);
     std::vector<int> ls((size_t)nl), lz((size_t)nl);

@@ -17,7 +17,8 @@ const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
 int tree_small_threshold();
-int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, int N, int D, int MIN, int MAX,
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, const uint8_t* q8, int N, int D,
+                     int MIN, int MAX,
                      int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream);
 
 // bucket_knn.hip

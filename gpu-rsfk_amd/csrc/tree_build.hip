@@ -33,6 +33,7 @@
 #include "bf16.hpp"
 #include <vector>
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 namespace rsfk {
@@ -53,34 +54,20 @@ struct LevelCounters {
 // helpers
 // ---------------------------------------------------------------------------
 
-// Hyperplane of (x1,x2): normal into LDS nvec[0..D), offset returned to all
-// threads through *b_out (LDS).  Offset order: create_node.cu:122-135.
-__device__ __forceinline__ void make_hyperplane(const float* __restrict__ x1, const float* __restrict__ x2,
-                                                int D, float* nvec, float* b_out)
-{
-    for (int d = threadIdx.x; d < D; d += blockDim.x) nvec[d] = x1[d] - x2[d];
-    if (threadIdx.x < bf16_valid(D) - D) nvec[D + threadIdx.x] = 0.0f;   // pad to whole 16-byte pieces of the bfloat16 rows
-    if (threadIdx.x < 32) {
-        float s = 0.0f;
-        for (int d = threadIdx.x; d < D; d += 32) {
-            const float t1 = x1[d], t2 = x2[d];
-            const float nd = t1 - t2;
-            const float prod = nd * (t1 + t2);
-            s = s + prod * 0.5f;
-        }
-        s = half_butterfly_sum(s);
-        if (threadIdx.x == 0) *b_out = s;
-    }
-}
+// Length of a normal in LDS: zero padded to whole 16-byte pieces of either screening copy.
+__host__ __device__ inline int nvec_len(int D) { return (D + 15) & ~15; }
 
-// The same by one wavefront (all 64 lanes call): normal zero padded to bf16_valid(D) values.
+// Hyperplane of (x1,x2) by one wavefront (all 64 lanes call): normal into LDS nvec[0..nvec_len(D)), and
+// hp[0] = offset (order of create_node.cu:122-135: 32 lane-strided partial sums + xor butterfly),
+// hp[1] = an upper bound of the 1-norm of the normal, hp[2] = the sum of its components (any order: only the
+// 8-bit screen uses them, with a margin).
 __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x1, const float* __restrict__ x2,
-                                                     int D, float* nvec, float* b_out)
+                                                     int D, float* nvec, float* hp)
 {
     const int lane = lane_id();
-    const int Dv = bf16_valid(D);
-    for (int d = lane; d < Dv; d += 64) nvec[d] = d < D ? x1[d] - x2[d] : 0.0f;
-    float s = 0.0f;
+    const int Dn = nvec_len(D);
+    for (int d = lane; d < Dn; d += 64) nvec[d] = d < D ? x1[d] - x2[d] : 0.0f;
+    float s = 0.0f, s2 = 0.0f;
     if (lane < 32) {
         for (int d = lane; d < D; d += 32) {
             const float t1 = x1[d], t2 = x2[d];
@@ -88,9 +75,17 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
             const float prod = nd * (t1 + t2);
             s = s + prod * 0.5f;
         }
+    } else {
+        for (int d = lane - 32; d < D; d += 32) {
+            const float nd = x1[d] - x2[d];
+            s += fabsf(nd);
+            s2 += nd;
+        }
     }
     s = half_butterfly_sum(s);
-    if (lane == 0) *b_out = s;
+    s2 = half_butterfly_sum(s2);
+    if (lane == 0) hp[0] = s;
+    if (lane == 32) { hp[1] = s * 1.001f; hp[2] = s2; }
 }
 
 // Screen of the side test for eight points per wavefront (right = n.x < b): lanes 8g..8g+7 work on
@@ -109,16 +104,72 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
 //
 // NB points per group are handled per call, so that NB row gathers per lane are in flight before the
 // first is needed (the loop over points is bound by the latency of these gathers otherwise).
-template <int NB>
+//
+// With the 8-bit copy (bf16.hpp) the row is 16 header bytes + one byte per coordinate: approx = lo sum_d n_d +
+// scale sum_d n_d q_d, undecided band e1 ||n||_1 (hp1 = bound of the 1-norm, hp2 = sum of the components of the
+// normal of the point's node).  Only lane 0 of a group holds the header, so only its right / redo are meaningful
+// (with either copy the callers use lane 0 only).
+template <int NB, bool Q8>
 __device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, const int (&j)[NB], const float (&b)[NB],
-                                             const uint16_t* __restrict__ pb16, const int (&id)[NB], int D, float band,
+                                             const float (&hp1)[NB], const float (&hp2)[NB],
+                                             const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8,
+                                             const int (&id)[NB], int D, float band,
                                              const bool (&valid)[NB], bool (&right)[NB], bool (&redo)[NB])
 {
+    if (Q8) {
+        const int sub = lane_id() & 7;
+#pragma unroll
+        for (int u = 0; u < NB; ++u) { right[u] = false; redo[u] = valid[u]; }
+        const size_t pitch = (size_t)q8_pitch(D);
+        const int pieces = q8_padded(D) >> 4;
+        float da[NB];
+        uint4 head[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            da[u] = 0.0f;
+            head[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (valid[u] && sub == 0) head[u] = *reinterpret_cast<const uint4*>(q8 + (size_t)id[u] * pitch);
+        }
+        for (int k = sub; k < pieces; k += 8) {
+            uint4 w[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                w[u] = make_uint4(0u, 0u, 0u, 0u);
+                if (valid[u]) w[u] = *reinterpret_cast<const uint4*>(q8 + (size_t)id[u] * pitch + 16 + 16 * k);
+            }
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const float* nvec = nvec0 + (size_t)j[u] * nstride + 16 * k;
+                const uint32_t ww[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 nq = *reinterpret_cast<const float4*>(&nvec[4 * q]);
+                    da[u] = __builtin_fmaf(nq.x, (float)((ww[q] >> 0) & 0xffu), da[u]);
+                    da[u] = __builtin_fmaf(nq.y, (float)((ww[q] >> 8) & 0xffu), da[u]);
+                    da[u] = __builtin_fmaf(nq.z, (float)((ww[q] >> 16) & 0xffu), da[u]);
+                    da[u] = __builtin_fmaf(nq.w, (float)((ww[q] >> 24) & 0xffu), da[u]);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            float d = da[u];
+            d += dpp_f<kDppXor1>(d); d += dpp_f<kDppXor2>(d); d += dpp_f<kDppHalfMirror>(d);
+            const float lo = __uint_as_float(head[u].y), scale = __uint_as_float(head[u].z), e1 = __uint_as_float(head[u].w);
+            const float approx = __builtin_fmaf(scale, d, lo * hp2[u]);
+            const bool certain = fabsf(approx - b[u]) > e1 * hp1[u];       // false if anything is NaN
+            right[u] = approx < b[u];
+            redo[u] = valid[u] && !certain;
+        }
+        return;
+    }
     // hyperplane of point u of this group: normal nvec0 + j[u] * nstride, offset b[u] (groups may differ)
     const int lane = lane_id();
     const int sub = lane & 7;
 #pragma unroll
     for (int u = 0; u < NB; ++u) { right[u] = false; redo[u] = valid[u]; }
+    (void)hp1;
+    (void)hp2;
     if (pb16 != nullptr) {
         const int Dv = bf16_valid(D);
         const size_t pitch = (size_t)bf16_pitch(D);
@@ -324,14 +375,16 @@ __global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, i
 
 // Side test of one chunk of one node: sets bit 31 of the permutation entry of
 // every member on the right side and counts the members on the left.
+template <bool Q8>
 __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ points,
-                                                 const uint16_t* __restrict__ pb16, TreeParams P,
+                                                 const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8,
+                                                 TreeParams P,
                                                  int* __restrict__ perm0, int* __restrict__ perm1,
                                                  const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
                                                  const int* __restrict__ chunk2node, int* __restrict__ chunk_left)
 {
-    extern __shared__ __align__(16) float nvec[];          // bf16_valid(D) floats
-    __shared__ float b_s;
+    extern __shared__ __align__(16) float nvec[];          // nvec_len(D) floats
+    __shared__ float hp_s[3];                               // offset, bound of the 1-norm, sum of the components
     __shared__ int left_s, n_def_s;
     __shared__ int deferred[1024];                          // points of the chunk left to the exact test (chunk <= 1024)
     const int c = blockIdx.x;
@@ -346,9 +399,9 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     if (threadIdx.x == 0) { left_s = 0; n_def_s = 0; }
     // p1/p2 must be read by every workgroup of the node before any of them sets
     // side bits; masking with kIdMask makes the read independent of that order.
-    make_hyperplane(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, &b_s);
+    if (threadIdx.x < 64) make_hyperplane_wave(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, hp_s);
     __syncthreads();
-    const float b = b_s;
+    const float b = hp_s[0], n1 = hp_s[1], sn = hp_s[2];
     const int pos0 = nd.start + k * P.chunk;
     const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
     const int grp = threadIdx.x >> 3, sub8 = threadIdx.x & 7;      // 32 groups of 8 lanes, one point each
@@ -356,7 +409,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     int lefts = 0;
     for (int it = 0; it < iters; it += kSideBatch) {
         int id[kSideBatch], jz[kSideBatch], pos[kSideBatch];
-        float bb[kSideBatch];
+        float bb[kSideBatch], h1[kSideBatch], h2[kSideBatch];
         bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
@@ -365,8 +418,10 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
             id[u] = valid[u] ? (perm[pos[u]] & kIdMask) : 0;
             jz[u] = 0;
             bb[u] = b;
+            h1[u] = n1;
+            h2[u] = sn;
         }
-        side_screen8<kSideBatch>(nvec, 0, jz, bb, pb16, id, P.D, P.band, valid, right, redo);
+        side_screen8<kSideBatch, Q8>(nvec, 0, jz, bb, h1, h2, pb16, q8, id, P.D, P.band, valid, right, redo);
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
             if (valid[u] && sub8 == 0) {
@@ -380,7 +435,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
         }
     }
     __syncthreads();
-    resolve_exact(deferred, n_def_s, nvec, 0, &b_s, points, P.D,
+    resolve_exact(deferred, n_def_s, nvec, 0, hp_s, points, P.D,
                   [&](int local) { return perm[pos0 + local] & kIdMask; },
                   [&](int local, bool right) {
                       const int id = perm[pos0 + local] & kIdMask;
@@ -517,9 +572,9 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr)
 {
-    // dynamic LDS: seg[small] | tmp[small] | nvec[G][bf16_valid(D)] | lrec[node_cap] | level lists 2 x node_cap | fmap[small]
+    // dynamic LDS: seg[small] | tmp[small] | nvec[G][nvec_len(D)] | lrec[node_cap] | level lists 2 x node_cap | fmap[small]
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    const int Dv = bf16_valid(P.D);
+    const int Dv = nvec_len(P.D);
     int* seg = reinterpret_cast<int*>(lds_raw);
     int* tmp = seg + P.small;
     float* nvec = reinterpret_cast<float*>(tmp + P.small);
@@ -529,7 +584,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     SmallNode* cur = reinterpret_cast<SmallNode*>(lrec + node_cap);
     SmallNode* nxt = cur + node_cap;
     unsigned char* fmap = reinterpret_cast<unsigned char*>(nxt + node_cap);
-    __shared__ float b_s[kMaxGroup];
+    __shared__ float b_s[kMaxGroup], hp_s[kMaxGroup][3];
     __shared__ int left_s[kMaxGroup], pre_s[kMaxGroup + 1], start_s[kMaxGroup], pair_s[kMaxGroup][2];
     __shared__ int n_cur_s, n_nxt_s, nrec_s, kind_s[2], base_s[2], lev_s, mx_s, mn_s, n_def_s;
 
@@ -589,9 +644,11 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                 pre_s[nb] = run;
             }
             __syncthreads();
-            for (int j = wave; j < nb; j += kBlock / 64)
+            for (int j = wave; j < nb; j += kBlock / 64) {
                 make_hyperplane_wave(points + (size_t)pair_s[j][0] * P.D, points + (size_t)pair_s[j][1] * P.D, P.D,
-                                     nvec + (size_t)j * Dv, &b_s[j]);
+                                     nvec + (size_t)j * Dv, hp_s[j]);
+                if (lane == 0) b_s[j] = hp_s[j][0];       // written by this lane just above
+            }
             for (int j = 0; j < nb; ++j) {
                 const int c = pre_s[j + 1] - pre_s[j];
                 for (int t = tid; t < c; t += kBlock) fmap[pre_s[j] + t] = (unsigned char)j;
@@ -602,7 +659,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
             const int iters = (total + kGroups - 1) / kGroups;
             for (int it = 0; it < iters; it += kSideBatch) {
                 int id[kSideBatch], jj[kSideBatch], pos[kSideBatch];
-                float bb[kSideBatch];
+                float bb[kSideBatch], h1[kSideBatch], h2[kSideBatch];
                 bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
 #pragma unroll
                 for (int u = 0; u < kSideBatch; ++u) {
@@ -612,8 +669,10 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                     pos[u] = valid[u] ? start_s[jj[u]] + f - pre_s[jj[u]] : 0;
                     id[u] = valid[u] ? seg[pos[u]] : 0;
                     bb[u] = b_s[jj[u]];
+                    h1[u] = hp_s[jj[u]][1];
+                    h2[u] = hp_s[jj[u]][2];
                 }
-                side_screen8<kSideBatch>(nvec, Dv, jj, bb, pb16, id, P.D, P.band, valid, right, redo);
+                side_screen8<kSideBatch, false>(nvec, Dv, jj, bb, h1, h2, pb16, nullptr, id, P.D, P.band, valid, right, redo);
 #pragma unroll
                 for (int u = 0; u < kSideBatch; ++u) {
                     if (valid[u] && sub8 == 0) {
@@ -788,7 +847,7 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
 // the buckets, in no particular order: those of at most kBucketSplit points in entries [0, n_small), the
 // larger ones in entries [leaf_cap - n_big, leaf_cap).  host_stats receives 5 ints per tree: number of
 // buckets, number of levels, largest and smallest bucket, number of large buckets.
-int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, int N, int D, int MIN, int MAX,
+int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, const uint8_t* q8, int N, int D, int MIN, int MAX,
                      int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream)
 {
     RSFK_CHECK(nb >= 1 && nb <= w->B && N == w->N && D == w->D, "tree batch: workspace does not match the request");
@@ -816,7 +875,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_HIP(hipGetLastError());
 
     int cur = 0;
-    const size_t side_lds = (size_t)bf16_valid(D) * sizeof(float);
+    const size_t side_lds = (size_t)nvec_len(D) * sizeof(float);
     // wide levels
     while (true) {
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
@@ -833,8 +892,12 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         // n_next := 0 for the level being produced
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
-        hipLaunchKernelGGL(k_side, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, P, w->perm[0], w->perm[1],
-                           w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
+        if (q8)
+            hipLaunchKernelGGL(k_side<true>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
+                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
+        else
+            hipLaunchKernelGGL(k_side<false>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
+                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr);
         RSFK_HIP(hipGetLastError());
@@ -844,11 +907,12 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     const int n_tail = w->h_ctr->n_tail;
     RSFK_CHECK(n_tail <= w->tail_cap, "tree batch: tail queue overflow");
     if (n_tail > 0) {
+        // (the tail kernel keeps the bfloat16 screen: measured, it is not faster with the 8-bit one)
         // nodes of a level of a subtree (and its buckets): at most small / MIN + 1; hyperplanes kept together:
         // as many as 24 KB hold, at most kMaxGroup
         const int node_cap = P.small / std::max(MIN, 1) + 4;
-        const int G = std::max(1, std::min(kMaxGroup, (int)(24 * 1024 / ((size_t)bf16_valid(D) * 4))));
-        const size_t lds = (size_t)(2 * P.small) * 4 + (size_t)G * bf16_valid(D) * 4 + (size_t)node_cap * sizeof(int2) +
+        const int G = std::max(1, std::min(kMaxGroup, (int)(24 * 1024 / ((size_t)nvec_len(D) * 4))));
+        const size_t lds = (size_t)(2 * P.small) * 4 + (size_t)G * nvec_len(D) * 4 + (size_t)node_cap * sizeof(int2) +
                            2 * (size_t)node_cap * sizeof(SmallNode) + (size_t)P.small;
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

@@ -30,7 +30,12 @@ def _say(*a):
     (5000, 32, 33, 66, "u"), (30000, 100, 33, 66, "u"), (60000, 3, 64, 256, "n"),      # wide phase, several levels
     (20000, 33, 17, 34, "n"), (8000, 784, 91, 182, "sparse"),
 ])
-def test_tree_partition_is_identical(gpu, orc, rng, N, D, MIN, MAX, dist):
+@pytest.mark.parametrize("screen", ["auto", "q8", "bf16"])
+def test_tree_partition_is_identical(gpu, orc, rng, monkeypatch, N, D, MIN, MAX, dist, screen):
+    """screen: which low-precision copy the side tests are screened on (RSFK_TREE_SCREEN; "auto" chooses from the
+    data).  The partition must be the one of the fp32 arithmetic whatever the screen."""
+    if screen != "auto":
+        monkeypatch.setenv("RSFK_TREE_SCREEN", screen)
     if dist == "u":
         X = rng.random((N, D), dtype=np.float32)
     elif dist == "n":
@@ -346,10 +351,13 @@ def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant
         monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
     N, D, K = 6000, 24, 10
     X = _hard_inputs(rng, kind, N, D)
-    _say("hard tree", kind)
     perm, ls, lz, st = orc.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
-    gperm, gls, glz, gst = gpu.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
-    assert np.array_equal(gperm, perm) and np.array_equal(glz, lz)
+    for screen in ("q8", "bf16"):
+        _say("hard tree", kind, screen)
+        monkeypatch.setenv("RSFK_TREE_SCREEN", screen)
+        gperm, gls, glz, gst = gpu.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
+        assert np.array_equal(gperm, perm) and np.array_equal(glz, lz)
+    monkeypatch.delenv("RSFK_TREE_SCREEN")
     _say("hard forest", kind)
     r = gpu_rsfk.RSFK(random_state=2)
     gi, gd = r.find_nearest_neighbors(X, K, n_trees=3, max_tree_depth=300, nn_exploring_factor=2)
