@@ -99,15 +99,15 @@ __global__ __launch_bounds__(256) void k_to_q8(const float* __restrict__ points,
 
 int q8_copy_alloc(Q8Copy* c, int N, int D)
 {
-    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * q8_pitch(D), 64)));
-    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->rho_sum), 16));
+    if (ws_alloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * q8_pitch(D), 64))) return 1;
+    if (ws_alloc(reinterpret_cast<void**>(&c->rho_sum), 16)) return 1;
     return 0;
 }
 
 void q8_copy_free(Q8Copy* c)
 {
-    if (c->rows) (void)hipFree(c->rows);
-    if (c->rho_sum) (void)hipFree(c->rho_sum);
+    ws_free(c->rows);
+    ws_free(c->rho_sum);
     c->rows = nullptr;
     c->rho_sum = nullptr;
 }
@@ -136,15 +136,15 @@ size_t bf16_copy_bytes(int N, int D) { return (size_t)N * ((size_t)bf16_pitch(D)
 
 int bf16_copy_alloc(Bf16Copy* c, int N, int D)
 {
-    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * bf16_pitch(D) * 2, 16)));
-    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(&c->norms), std::max<size_t>((size_t)N * 4, 16)));
+    if (ws_alloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * bf16_pitch(D) * 2, 16))) return 1;
+    if (ws_alloc(reinterpret_cast<void**>(&c->norms), std::max<size_t>((size_t)N * 4, 16))) return 1;
     return 0;
 }
 
 void bf16_copy_free(Bf16Copy* c)
 {
-    if (c->rows) (void)hipFree(c->rows);
-    if (c->norms) (void)hipFree(c->norms);
+    ws_free(c->rows);
+    ws_free(c->norms);
     c->rows = nullptr;
     c->norms = nullptr;
 }

@@ -20,8 +20,8 @@ namespace {
 
 struct DevMem {
     void* p = nullptr;
-    ~DevMem() { if (p) (void)hipFree(p); }
-    int alloc(size_t bytes) { RSFK_HIP(hipMalloc(&p, bytes ? bytes : 1)); return 0; }
+    ~DevMem() { ws_free(p); }
+    int alloc(size_t bytes) { return ws_alloc(&p, bytes); }
 };
 
 }  // namespace
@@ -220,6 +220,8 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
 }
 
 RSFK_API const char* rsfk_last_error(void) { return last_error(); }
+
+RSFK_API void rsfk_release_workspace(void) { ws_release_all(); }
 
 RSFK_API int rsfk_device_count(void)
 {

@@ -246,7 +246,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
     w->K = K;
     w->MW = (K + 31) / 32;
     w->n_blocks = (N + kScanBlock - 1) / kScanBlock;
-    auto dm = [](void* p, size_t n) { return hipMalloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)); };
+    auto dm = [](void* p, size_t n) { return ws_alloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)) ? hipErrorOutOfMemory : hipSuccess; };
     if (dm(&w->rev, (size_t)N * K) != hipSuccess || dm(&w->fwd2rev, (size_t)N * K) != hipSuccess ||
         dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->deg, (size_t)N) != hipSuccess ||
         dm(&w->totals, (size_t)w->n_blocks + 1) != hipSuccess || dm(&w->pass, (size_t)N * K * w->MW) != hipSuccess ||
@@ -265,7 +265,7 @@ void explore_ws_free(ExploreWorkspace* w)
     if (!w) return;
     void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass, w->todo};
     for (void* b : bufs)
-        if (b) (void)hipFree(b);
+        ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
     delete w;
 }

@@ -58,7 +58,7 @@ struct WsGuard {
 };
 struct DevBuf {
     void* p = nullptr;
-    ~DevBuf() { if (p) (void)hipFree(p); }
+    ~DevBuf() { ws_free(p); }
 };
 struct Bf16Guard {
     Bf16Copy c;
@@ -172,7 +172,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     const double t_exp0 = now_s();
     if (nnef > 0) {
         DevBuf old;
-        RSFK_HIP(hipMalloc(&old.p, sizeof(int) * (size_t)N * (size_t)K));
+        if (ws_alloc(&old.p, sizeof(int) * (size_t)N * (size_t)K)) return 1;
         ExploreWsGuard ews;      // without a workspace every point enumerates its own candidates
         if (explore_join_enabled(N, K) && explore_ws_alloc(&ews.w, N, K)) return 1;
         for (int it = 0; it < nnef; ++it) {
@@ -195,9 +195,9 @@ int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_
     RSFK_CHECK(N >= 1 && D >= 1 && K >= 1, "forest: N, D and K must be positive");
     DevBuf dp, di, dd;
     const size_t nd = (size_t)N * (size_t)D, nk = (size_t)N * (size_t)K;
-    RSFK_HIP(hipMalloc(&dp.p, nd * sizeof(float)));
-    RSFK_HIP(hipMalloc(&di.p, nk * sizeof(int)));
-    RSFK_HIP(hipMalloc(&dd.p, nk * sizeof(float)));
+    if (ws_alloc(&dp.p, nd * sizeof(float))) return 1;
+    if (ws_alloc(&di.p, nk * sizeof(int))) return 1;
+    if (ws_alloc(&dd.p, nk * sizeof(float))) return 1;
     RSFK_HIP(hipMemcpy(dp.p, points, nd * sizeof(float), hipMemcpyHostToDevice));
     RSFK_HIP(hipMemcpy(di.p, knn_idx, nk * sizeof(int), hipMemcpyHostToDevice));
     RSFK_HIP(hipMemcpy(dd.p, knn_dist, nk * sizeof(float), hipMemcpyHostToDevice));

@@ -15,12 +15,20 @@ namespace rsfk {
 void set_last_error(const std::string& msg);
 const char* last_error();
 
+// workspace.hip: device memory for working buffers, kept for the next call after use
+int ws_alloc(void** out, size_t bytes);
+void ws_free(void* p);
+void ws_release_all();
+
+// Both macros leave the function on failure.  Work that was queued before may still be running and the
+// callers' guards hand their buffers back for reuse on the way out, so the device is drained first.
 #define RSFK_HIP(call)                                                                   \
     do {                                                                                 \
         hipError_t e_ = (call);                                                          \
         if (e_ != hipSuccess) {                                                          \
             ::rsfk::set_last_error(std::string(#call) + ": " + hipGetErrorString(e_) +   \
                                    " (" __FILE__ ":" + std::to_string(__LINE__) + ")");  \
+            (void)hipDeviceSynchronize();                                                \
             return 1;                                                                    \
         }                                                                                \
     } while (0)
@@ -29,6 +37,7 @@ const char* last_error();
     do {                                           \
         if (!(cond)) {                             \
             ::rsfk::set_last_error(msg);           \
+            (void)hipDeviceSynchronize();          \
             return 2;                              \
         }                                          \
     } while (0)

@@ -756,8 +756,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
 template <typename T>
 int dmalloc(T** p, size_t n)
 {
-    RSFK_HIP(hipMalloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(T)));
-    return 0;
+    return ws_alloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(T));
 }
 
 }  // namespace
@@ -787,7 +786,7 @@ static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
                    w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr};
-    for (void* p : dev) if (p) (void)hipFree(p);
+    for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
     w = TreeBatchWorkspace();

@@ -1,0 +1,109 @@
+// Device memory for the working buffers of a call (permutations, screening copies, exploration workspace).
+//
+// hipMalloc / hipFree of a few hundred megabytes cost tens to hundreds of microseconds each and a call needs
+// about thirty of them, so blocks are kept after use and handed out again to the next call that asks for the
+// same size on the same device (a build repeated with the same shapes allocates nothing).  Idle blocks are
+// capped at a quarter of the device memory; rsfk_release_workspace() returns all of them to the driver.
+// The reference allocates and frees inside every tree level (src/rsfk.cu:640-1180).
+#include "rsfk_common.hpp"
+#include <map>
+#include <mutex>
+#include <vector>
+
+namespace rsfk {
+
+namespace {
+
+struct Pool {
+    std::mutex mu;
+    std::multimap<std::pair<int, size_t>, void*> idle;     // (device, bytes) -> block
+    std::map<void*, std::pair<int, size_t>> live;           // blocks handed out
+    size_t idle_bytes = 0;
+};
+
+Pool& pool()
+{
+    static Pool p;
+    return p;
+}
+
+}  // namespace
+
+int ws_alloc(void** out, size_t bytes)
+{
+    *out = nullptr;
+    if (bytes == 0) bytes = 1;
+    bytes = (bytes + 255) & ~(size_t)255;
+    int dev = 0;
+    RSFK_HIP(hipGetDevice(&dev));
+    Pool& P = pool();
+    {
+        std::lock_guard<std::mutex> lock(P.mu);
+        auto it = P.idle.find({dev, bytes});
+        if (it != P.idle.end()) {
+            *out = it->second;
+            P.idle.erase(it);
+            P.idle_bytes -= bytes;
+            P.live[*out] = {dev, bytes};
+            return 0;
+        }
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) {
+        // give the idle blocks back and try once more
+        (void)hipGetLastError();
+        ws_release_all();
+        e = hipMalloc(&p, bytes);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        set_last_error(std::string("out of device memory (") + std::to_string(bytes) + " bytes): " + hipGetErrorString(e));
+        return 1;
+    }
+    std::lock_guard<std::mutex> lock(P.mu);
+    P.live[p] = {dev, bytes};
+    *out = p;
+    return 0;
+}
+
+// The caller has made sure that no work that uses the block is still running.
+void ws_free(void* p)
+{
+    if (!p) return;
+    Pool& P = pool();
+    std::pair<int, size_t> key;
+    {
+        std::lock_guard<std::mutex> lock(P.mu);
+        auto it = P.live.find(p);
+        if (it == P.live.end()) {           // not ours
+            (void)hipFree(p);
+            return;
+        }
+        key = it->second;
+        P.live.erase(it);
+        size_t free_b = 0, total_b = 0;
+        const bool known = hipMemGetInfo(&free_b, &total_b) == hipSuccess;
+        if (!known || P.idle_bytes + key.second <= total_b / 4) {
+            P.idle.insert({key, p});
+            P.idle_bytes += key.second;
+            return;
+        }
+    }
+    (void)hipFree(p);
+}
+
+void ws_release_all()
+{
+    Pool& P = pool();
+    std::vector<void*> blocks;
+    {
+        std::lock_guard<std::mutex> lock(P.mu);
+        for (auto& kv : P.idle) blocks.push_back(kv.second);
+        P.idle.clear();
+        P.idle_bytes = 0;
+    }
+    for (void* b : blocks) (void)hipFree(b);
+}
+
+}  // namespace rsfk

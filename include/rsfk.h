@@ -118,6 +118,11 @@ int rsfk_explore_host(const float* points, int N, int D, int num_neighbors,
 /* text of the last error of a call that returned non-zero */
 const char* rsfk_last_error(void);
 
+/* The library keeps the device buffers of a call (permutations, screening copies, exploration workspace) for the
+ * next call instead of returning them to the driver; this returns all idle ones.  No counterpart in the
+ * reference, which allocates and frees inside every tree level (src/rsfk.cu:640-1180). */
+void rsfk_release_workspace(void);
+
 /* number of HIP devices visible to the library (0 when there is none) */
 int rsfk_device_count(void);
 

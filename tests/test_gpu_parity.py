@@ -375,6 +375,19 @@ def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant
         assert_knn_equal(gi, gd, oi, od)
 
 
+def test_workspace_is_reused_and_can_be_released(gpu, rng):
+    """Device buffers are kept between calls; releasing them changes nothing but the next call's allocations."""
+    import gpu_rsfk
+    from gpu_rsfk import capi
+    X = rng.random((5000, 20), dtype=np.float32)
+    a = gpu_rsfk.RSFK(random_state=4).find_nearest_neighbors(X, 12, n_trees=3)
+    b = gpu_rsfk.RSFK(random_state=4).find_nearest_neighbors(X, 12, n_trees=3)      # served from the kept buffers
+    capi.lib().rsfk_release_workspace()
+    c = gpu_rsfk.RSFK(random_state=4).find_nearest_neighbors(X, 12, n_trees=3)
+    for r in (b, c):
+        assert_knn_equal(r[0], r[1], a[0], a[1])
+
+
 def test_rows_come_back_sorted_and_unsorted_input_is_accepted(gpu, orc, rng):
     """Rows handed in unsorted (the reference keeps them unordered) are merged correctly; rows come back ascending."""
     N, D, K = 3000, 12, 16
