@@ -203,7 +203,7 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
     int skip_upto = 0;
     if (K <= 64) {
         // buckets of up to 64 points go to the specialised kernel; the general one skips them
-        if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, knn_idx, knn_dist, stream))
+        if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
             return 1;
         if (max_bucket >= 0 && max_bucket <= small_bucket_cap()) return 0;
         skip_upto = small_bucket_cap();
@@ -212,19 +212,20 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 }
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
-// (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  bf: bfloat16 copy of the
-// points if the rows are known to be sorted by distance (then the small buckets take the screened kernel), else null.
-int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, int D, int K, const int* ids, const int* starts,
-                           const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx, float* knn_dist,
-                           hipStream_t stream)
+// (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  rows_sorted: every K-NN row is
+// known to be sorted by distance.  bf: bfloat16 copy of the points to send the small buckets to the screened kernel
+// (needs sorted rows), else null.
+int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
+                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx,
+                           float* knn_dist, hipStream_t stream)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
     if (n_small > 0) {
-        if (K <= 64 && bf != nullptr) {
+        if (K <= 64 && bf != nullptr && rows_sorted) {
             if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
-            if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
+            if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream)) {
             return 1;
         }

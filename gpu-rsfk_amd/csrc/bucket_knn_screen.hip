@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                                                                    int ksteps, float kappa, float inv_one_minus_gamma)
 {
     // dynamic LDS: [rows | triangular distance matrix] (region_floats) | ids[64] | tau[64] | taup[64] | nrm[64] |
-    //              n_pairs, active[2] | list
+    //              n_pairs | flag[64] | list
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
     float* tri = lds_f;                      // same storage, used after the last read of rows
@@ -103,8 +103,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     float* taup = tau + kCap;
     float* nrm = taup + kCap;
     int* n_pairs = reinterpret_cast<int*>(nrm + kCap);
-    uint32_t* active_s = reinterpret_cast<uint32_t*>(n_pairs + 1);      // per wavefront: members with a candidate
-    uint16_t* list = reinterpret_cast<uint16_t*>(n_pairs + 4);
+    int* flag = n_pairs + 4;                 // member has a candidate below its last slot
+    uint16_t* list = reinterpret_cast<uint16_t*>(flag + kCap);
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
@@ -121,26 +121,23 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         taup[tid] = (t + 1e-30f) * inv_one_minus_gamma;
         nrm[tid] = id >= 0 ? bnorms[id] : 0.0f;
     }
-    if (tid < 4) n_pairs[tid] = 0;           // n_pairs, active[0], active[1]
+    if (tid < kCap) flag[tid] = 0;
+    if (tid == 0) *n_pairs = 0;
     __syncthreads();
 
     // fp32 rows of a slice: lane pc of a group of 16 loads piece pc of rows rg, rg + 8, ...; requested early,
     // written to LDS when the previous slice has been consumed
     const int pc = tid & (kLanesPerRow - 1), rg = tid / kLanesPerRow;
-    const float* rowp[kLoads];
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-        const int m = rg + kRowsPerStep * i;
-        rowp[i] = points + (size_t)lids[m < s ? m : 0] * (size_t)D + 4 * pc;
-    }
-    float4 pre[kLoads];
-    auto request = [&](int d0) {
-        const int np = min(chunk, (D - d0 + 3) & ~3) >> 2;      // 16-byte pieces per row in this slice
+    // two slices are in flight: A holds slices 0, 2, ..., B slices 1, 3, ...
+    float4 preA[kLoads], preB[kLoads];
+    auto request = [&](float4 (&pre)[kLoads], int d0) {
+        const int np = d0 < D ? min(chunk, (D - d0 + 3) & ~3) >> 2 : 0;      // 16-byte pieces per row in this slice
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
             pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (pc < np && rg + kRowsPerStep * i < s) {
-                const float* src = rowp[i] + d0;
+            const int m = rg + kRowsPerStep * i;
+            if (pc < np && m < s) {
+                const float* src = points + (size_t)lids[m] * (size_t)D + 4 * pc + d0;
                 if (vec_ok) {
                     pre[i] = *reinterpret_cast<const float4*>(src);
                 } else {
@@ -154,7 +151,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         }
         return np;
     };
-    int np = request(0);
+    int npA = 0, npB = 0;
 
     // ---- 1. screen: wavefront 0 takes the tiles (half 0 x half 0) and (half 0 x half 1), wavefront 1 the
     //         tile (half 1 x half 1); members beyond s read the row of member 0 and are ignored
@@ -169,10 +166,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             f32x16 gxx, gxy;
 #pragma unroll
             for (int i = 0; i < 16; ++i) { gxx[i] = 0.0f; gxy[i] = 0.0f; }
-            for (int k0 = 0; k0 < ksteps; k0 += 4) {
-                bf16x8 x[4], y[4];
+            for (int k0 = 0; k0 < ksteps; k0 += 8) {           // operands of eight steps (128 dimensions) in flight
+                bf16x8 x[8], y[8];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < 8; ++u) {
                     if (k0 + u < ksteps) {
                         x[u] = *reinterpret_cast<const bf16x8*>(rx + 16 * (k0 + u));
                         if (second) y[u] = *reinterpret_cast<const bf16x8*>(ry + 16 * (k0 + u));
@@ -180,13 +177,16 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < 8; ++u) {
                     if (k0 + u < ksteps) {
                         gxx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], x[u], gxx, 0, 0, 0);
                         if (second) gxy = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], y[u], gxy, 0, 0, 0);
                     }
                 }
             }
+            // the fp32 rows of the first two slices travel while the tiles are screened
+            npA = request(preA, 0);
+            npB = request(preB, chunk);
             const int mbase = 32 * hx + 4 * (lane >> 5);
             for (int t = 0; t < (second ? 2 : 1); ++t) {
                 const int n = t == 0 ? mx : my;
@@ -200,6 +200,9 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                     list[at++] = (uint16_t)(m | (n << 6));
                 }
             }
+        } else {
+            npA = request(preA, 0);
+            npB = request(preB, chunk);
         }
     }
     __syncthreads();
@@ -207,32 +210,26 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     const int rounds = (n_list + kThreads - 1) / kThreads;      // pairs per thread, at most kPairsPerThread
 
     // ---- 2. exact distances of the listed pairs
-    uint32_t where[kPairsPerThread];          // LDS offsets of the two rows of a pair, 16 bits each
     float acc[kPairsPerThread];
 #pragma unroll
-    for (int k = 0; k < kPairsPerThread; ++k) {
-        const int p = tid + k * kThreads;
-        const uint32_t e = p < n_list ? list[p] : 0u;
-        where[k] = ((e & 63u) * (uint32_t)pitch) | (((e >> 6) * (uint32_t)pitch) << 16);
-        acc[k] = 0.0f;
-    }
-    for (int d0 = 0; d0 < D; d0 += chunk) {
-        if (d0 > 0) __syncthreads();                 // the previous slice has been consumed
-        if (pc < np) {
+    for (int k = 0; k < kPairsPerThread; ++k) acc[k] = 0.0f;
+    auto consume = [&](float4 (&pre)[kLoads], int np_now, bool first) {
+        if (!first) __syncthreads();                 // the previous slice has been consumed
+        if (pc < np_now) {
 #pragma unroll
             for (int i = 0; i < kLoads; ++i) {
                 const int m = rg + kRowsPerStep * i;
                 if (m < s) *reinterpret_cast<float4*>(&rows[m * pitch + 4 * pc]) = pre[i];
             }
         }
-        const int np_now = np;
-        if (d0 + chunk < D) np = request(d0 + chunk);
         __syncthreads();
 #pragma unroll
         for (int k = 0; k < kPairsPerThread; ++k) {
             if (k < rounds) {
-                const float* ra = rows + (where[k] & 0xffffu);
-                const float* rb = rows + (where[k] >> 16);
+                const int p = tid + k * kThreads;
+                const uint32_t e = p < n_list ? list[p] : 0u;      // idle threads compute pair (0, 0)
+                const float* ra = rows + (e & 63u) * (uint32_t)pitch;
+                const float* rb = rows + (e >> 6) * (uint32_t)pitch;
                 float a = acc[k];
                 for (int q = 0; q < np_now; ++q) {
                     const float4 x = *reinterpret_cast<const float4*>(ra + 4 * q);
@@ -245,6 +242,14 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                 }
                 acc[k] = a;
             }
+        }
+    };
+    for (int d0 = 0; d0 < D; d0 += 2 * chunk) {
+        consume(preA, npA, d0 == 0);
+        if (d0 + 2 * chunk < D) npA = request(preA, d0 + 2 * chunk);
+        if (d0 + chunk < D) {
+            consume(preB, npB, false);
+            if (d0 + 3 * chunk < D) npB = request(preB, d0 + 3 * chunk);
         }
     }
     __syncthreads();                           // rows no longer needed: the region becomes the distance matrix
@@ -259,9 +264,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             const int r = (int)(e & 63u), c = (int)(e >> 6);
             const float d = acc[k];
             tri[tri_at(r, c)] = d;
-            // member i belongs to wavefront i % 2 and is its bit i / 2
-            if (d < tau[r]) atomicOr(&active_s[r & 1], 1u << (r >> 1));
-            if (d < tau[c]) atomicOr(&active_s[c & 1], 1u << (c >> 1));
+            if (d < tau[r]) flag[r] = 1;             // plain stores of the same value: no ordering needed
+            if (d < tau[c]) flag[c] = 1;
         }
     }
     __syncthreads();
@@ -269,7 +273,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     // ---- 3. top-K update.  A wavefront owns every second member and walks those that have a candidate below
     //         their last slot, with the rows of the next two in flight.
     const int my_id = lids[lane];
-    uint32_t active = active_s[wave];
+    // bit u: member wave + 2 u has a candidate
+    uint32_t active = (uint32_t)ballot64(lane < 32 && flag[(wave + kWaves * lane) & (kCap - 1)] != 0);
     auto candidate = [&](int i) {
         const int a = min(i, lane), b = max(i, lane);
         return (lane < s && lane != i) ? tri[tri_at(a, b)] : INFINITY;
@@ -289,26 +294,37 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             rd = knn_dist[at];
         }
     };
-    int i0 = next_member(), i1 = next_member();
-    int ri0, ri1, ri2;
-    float rd0, rd1, rd2;
-    load_row(i0, ri0, rd0);
-    load_row(i1, ri1, rd1);
-    while (i0 >= 0) {
-        const int i2 = next_member();
-        load_row(i2, ri2, rd2);
-        const float d = candidate(i0);
-        KnnRow<1> row;
-        row.idx[0] = ri0;
-        row.dist[0] = rd0;
-        row.init_sorted(K);
-        row.offer_lanes<true>(lane < s && lane != i0, my_id, d);
-        if (row.changed) {
-            const size_t at = (size_t)lids[i0] * (size_t)K;
-            row.store(knn_idx + at, knn_dist + at);
+    constexpr int kAhead = 4;
+    int cur_i[kAhead], cur_ri[kAhead], nxt_i[kAhead], nxt_ri[kAhead];
+    float cur_rd[kAhead], nxt_rd[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+        cur_i[u] = next_member();
+        load_row(cur_i[u], cur_ri[u], cur_rd[u]);
+    }
+    while (cur_i[0] >= 0) {
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            nxt_i[u] = next_member();
+            load_row(nxt_i[u], nxt_ri[u], nxt_rd[u]);
         }
-        i0 = i1; ri0 = ri1; rd0 = rd1;
-        i1 = i2; ri1 = ri2; rd1 = rd2;
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int i = cur_i[u];
+            if (i < 0) break;
+            const float d = candidate(i);
+            KnnRow<1> row;
+            row.idx[0] = cur_ri[u];
+            row.dist[0] = cur_rd[u];
+            row.init_sorted(K);
+            row.offer_lanes<true>(lane < s && lane != i, my_id, d);
+            if (row.changed) {
+                const size_t at = (size_t)lids[i] * (size_t)K;
+                row.store(knn_idx + at, knn_dist + at);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }
     }
 }
 
@@ -353,7 +369,7 @@ int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int
     RSFK_CHECK(kCap * pitch < 65536, "screened small-bucket kernel: LDS offsets must fit 16 bits");
     const int region = std::max(kCap * pitch, kMaxPairs);
     const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)(4 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(5 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
     const int ksteps = (bf16_valid(D) + 15) / 16;
     RSFK_CHECK(ksteps * 16 <= bf16_pitch(D), "screened small-bucket kernel: bfloat16 rows too short");
     const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21

@@ -46,13 +46,17 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
                                                                   const int* __restrict__ starts,
                                                                   const int* __restrict__ sizes, int stride,
                                                                   int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                                  int chunk, int pitch, int region_floats)
+                                                                  int chunk, int pitch, int region_floats, int rows_sorted)
 {
-    // dynamic LDS: [rows | dist] (region_floats) | ids[64]
+    // dynamic LDS: [rows | dist] (region_floats) | ids[64] | tau[64] | flag[64]
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
     float* dist = lds_f;                     // same storage, used after the last read of rows
     int* lids = reinterpret_cast<int*>(lds_f + region_floats);
+    // last slot of each member's row when the rows are known to be sorted (else +inf): a member none of whose
+    // candidates is below it is left alone -- its row is neither read nor written
+    float* tau = reinterpret_cast<float*>(lids + kCap);
+    int* flag = reinterpret_cast<int*>(tau + kCap);                    // member has such a candidate
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
@@ -61,7 +65,12 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
-    if (tid < kCap) lids[tid] = tid < s ? bid[tid] : -1;
+    if (tid < kCap) {
+        const int id = tid < s ? bid[tid] : -1;
+        lids[tid] = id;
+        tau[tid] = (rows_sorted && id >= 0) ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : INFINITY;
+        flag[tid] = 0;
+    }
     __syncthreads();
 
     // work assignment: off-diagonal 4x4 blocks (ti < tj) one per thread, then the 6 pairs of each diagonal block
@@ -155,59 +164,79 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
         }
     }
     __syncthreads();                           // rows no longer needed: the region becomes the distance matrix
+    auto put = [&](int i, int j, float d) {
+        dist[i * kDistPitch + j] = d;
+        dist[j * kDistPitch + i] = d;
+        if (d < tau[i]) flag[i] = 1;             // plain stores of the same value: no ordering needed
+        if (d < tau[j]) flag[j] = 1;
+    };
     if (has_tile) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int i = 4 * ti + r, j = 4 * tj + c;
-                if (i < s && j < s) {
-                    dist[i * kDistPitch + j] = acc[r][c];
-                    dist[j * kDistPitch + i] = acc[r][c];
-                }
+                if (i < s && j < s) put(i, j, acc[r][c]);
             }
     }
     if (has_diag) {
         const int i = 4 * dt + dr, j = 4 * dt + dc;
-        if (j < s) {
-            dist[i * kDistPitch + j] = dacc;
-            dist[j * kDistPitch + i] = dacc;
-        }
+        if (j < s) put(i, j, dacc);
     }
 
     __syncthreads();                           // distance matrix complete
 
-    // top-K update, one member at a time per wavefront; the LDS reads of the next member are
-    // issued before the current one is merged
+    // top-K update: a wavefront walks its members that have a candidate, four at a time, with the rows of the
+    // next four in flight (the loop is bound by the latency of these row reads otherwise)
     const int my_id = lids[lane];
-    float d_next = dist[wave * kDistPitch + lane];
+    // bit u: member wave + 2 u has a candidate
+    uint32_t active = (uint32_t)ballot64(lane < 32 && flag[(wave + kWaves * lane) & (kCap - 1)] != 0);
+    auto next_member = [&]() {
+        if (active == 0) return -1;
+        const int u = __ffs(active) - 1;
+        active &= active - 1;
+        return wave + kWaves * u;
+    };
     auto load_row = [&](int i, int& ri, float& rd) {
         ri = -2;
         rd = INFINITY;
-        if (i < s && lane < K) {
+        if (i >= 0 && lane < K) {
             const size_t at = (size_t)lids[i] * (size_t)K + lane;
             ri = knn_idx[at];
             rd = knn_dist[at];
         }
     };
-    int ri0, ri1, ri2;
-    float rd0, rd1, rd2;
-    load_row(wave, ri0, rd0);
-    load_row(wave + kWaves, ri1, rd1);
-    for (int i = wave; i < s; i += kWaves) {
-        load_row(i + 2 * kWaves, ri2, rd2);
-        const float d = d_next;
-        if (i + kWaves < s) d_next = dist[(i + kWaves) * kDistPitch + lane];
-        KnnRow<1> row;
-        row.idx[0] = ri0;
-        row.dist[0] = rd0;
-        ri0 = ri1; rd0 = rd1; ri1 = ri2; rd1 = rd2;
-        row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
-        row.offer_lanes<true>(lane < s && lane != i, my_id, d);
-        if (row.changed) {
-            const size_t at = (size_t)lids[i] * (size_t)K;
-            row.store(knn_idx + at, knn_dist + at);
+    constexpr int kAhead = 4;
+    int cur_i[kAhead], cur_ri[kAhead], nxt_i[kAhead], nxt_ri[kAhead];
+    float cur_rd[kAhead], nxt_rd[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+        cur_i[u] = next_member();
+        load_row(cur_i[u], cur_ri[u], cur_rd[u]);
+    }
+    while (cur_i[0] >= 0) {
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            nxt_i[u] = next_member();
+            load_row(nxt_i[u], nxt_ri[u], nxt_rd[u]);
         }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) {
+            const int i = cur_i[u];
+            if (i < 0) break;
+            const float d = dist[i * kDistPitch + lane];
+            KnnRow<1> row;
+            row.idx[0] = cur_ri[u];
+            row.dist[0] = cur_rd[u];
+            row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
+            row.offer_lanes<true>(lane < s && lane != i, my_id, d);
+            if (row.changed) {
+                const size_t at = (size_t)lids[i] * (size_t)K;
+                row.store(knn_idx + at, knn_dist + at);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }
     }
 }
 
@@ -215,8 +244,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
 
 int small_bucket_cap() { return kCap; }
 
+// rows_sorted: every K-NN row is known to be sorted by distance (then members without a candidate below their
+// last slot are skipped)
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
-                            int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream)
+                            int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream)
 {
     if (n_buckets <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
@@ -226,11 +257,11 @@ int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, c
     if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units
     const int region = std::max(kLdsRows * pitch, kCap * kDistPitch);
     const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)kCap * 4;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(3 * kCap) * 4;
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_small),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(k_bucket_knn_small, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, D, K, ids,
-                       starts, sizes, stride, knn_idx, knn_dist, chunk, pitch, region_floats);
+                       starts, sizes, stride, knn_idx, knn_dist, chunk, pitch, region_floats, rows_sorted ? 1 : 0);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

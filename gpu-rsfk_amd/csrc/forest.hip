@@ -121,9 +121,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (n_trees > 0 && make_tree_screen(q8, d_points, N, D, verbose, stream, &q8_rows)) return 1;
 
     if (n_trees > 0) {
-        // the screened kernel reads a row's maximum from its last slot: rows the caller passed in unsorted are
-        // put in order once
-        if (screen && launch_sort_rows(d_idx, d_dist, N, K, stream)) return 1;
+        // the bucket kernels read a row's maximum from its last slot: rows the caller passed in unsorted are put
+        // in order once
+        if (launch_sort_rows(d_idx, d_dist, N, K, stream)) return 1;
         const int B = choose_batch(n_trees, N, D, MIN);
         WsGuard ws;
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
@@ -139,7 +139,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             const double tb = now_s() - tb0;
             for (int j = 0; j < nb && rc == 0; ++j) {
                 (void)hipEventRecord(ev[j].a, stream);
-                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w),
                                             stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], d_idx, d_dist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
