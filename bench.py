@@ -143,7 +143,7 @@ def main():
     # default workload
     default_workload = (args.workload == "uniform" and (N, D, K) == (1000000, 100, 32) and (mn, mx) == (33, 66))
     traffic = 1.05e9 if default_workload else None
-    roofline = {"kernel": "k_bucket_knn_small + k_bucket_knn", "bound": "hbm", "achieved": round(achieved, 1),
+    roofline = {"kernel": "k_bucket_knn_small (buckets <= 64 and 65..72)", "bound": "hbm", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4),
                 "launches_per_step": T}

@@ -202,11 +202,14 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
     int skip_upto = 0;
     if (K <= 64) {
-        // buckets of up to 64 points go to the specialised kernel; the general one skips them
+        // buckets of up to 72 points go to the specialised kernels; the general one skips them
         if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
             return 1;
         if (max_bucket >= 0 && max_bucket <= small_bucket_cap()) return 0;
-        skip_upto = small_bucket_cap();
+        if (launch_bucket_knn_medium(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
+            return 1;
+        if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
+        skip_upto = medium_bucket_cap();
     }
     return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream);
 }
@@ -216,8 +219,8 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // known to be sorted by distance.  bf: bfloat16 copy of the points to send the small buckets to the screened kernel
 // (needs sorted rows), else null.
 int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
-                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx,
-                           float* knn_dist, hipStream_t stream)
+                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
+                           int* knn_idx, float* knn_dist, hipStream_t stream)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
@@ -230,8 +233,17 @@ int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_so
             return 1;
         }
     }
+    // the large ones: 65..72 points to the three-wavefront variant of the small kernel, the rest to the general one
+    if (n_big <= 0) return 0;
     const int off = leaf_cap - n_big;
-    return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, 0, knn_idx, knn_dist, stream);
+    int skip_upto = 0;
+    if (K <= 64) {
+        if (launch_bucket_knn_medium(points, D, K, ids, starts + off, sizes + off, n_big, 0, rows_sorted, knn_idx, knn_dist, stream))
+            return 1;
+        if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
+        skip_upto = medium_bucket_cap();
+    }
+    return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream);
 }
 
 }  // namespace rsfk

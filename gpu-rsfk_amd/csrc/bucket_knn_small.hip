@@ -1,7 +1,7 @@
-// Bucket K-NN for buckets of at most 64 points and K <= 64: the shape the
-// default parameters (bucket size K+1 .. 2(K+1), K <= 32) produce.  Same function
-// as the general kernel in bucket_knn.hip (see there for the reference kernels it
-// replaces); two wavefronts per bucket.
+// Bucket K-NN for buckets of at most 64 points (two wavefronts per bucket) or of
+// 65..72 points (three) and K <= 64: the shapes the default parameters (bucket size
+// K+1 .. 2(K+1), K <= 32) produce.  Same function as the general kernel in
+// bucket_knn.hip (see there for the reference kernels it replaces).
 //
 //   1. the rows of the bucket, 64 dimensions at a time, are requested from HBM at
 //      once and written to LDS; a row is read by consecutive lanes, 16 bytes each
@@ -11,9 +11,11 @@
 //      (arithmetic of euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
 //      the 6 pairs inside each diagonal block are done one per thread;
 //   3. the distance matrix replaces the rows in LDS; a wavefront owns every second
-//      point: per point, the candidates that are closer than the row's last slot
-//      are inserted into the sorted row unless the row holds them already
-//      (knn_list.hpp); the rows of the next two points are in flight meanwhile.
+//      (third) point: per point, the candidates that are closer than the row's last
+//      slot are inserted into the sorted row unless the row holds them already
+//      (knn_list.hpp); the rows of the next four points are in flight meanwhile, and
+//      points without any such candidate are skipped when the rows are known to be
+//      sorted.
 // Registers are kept near 100 and LDS near 20 KB per workgroup so that four
 // wavefronts per SIMD are resident: the kernel alternates between an arithmetic
 // phase and a latency-bound merge phase, and only other resident workgroups can
@@ -26,28 +28,38 @@ namespace rsfk {
 
 namespace {
 
-constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
-static_assert(kCap == 64, "lane-per-candidate merge and 64-bit presence masks assume 64");
-constexpr int kThreads = 128;
-constexpr int kWaves = kThreads / 64;
-constexpr int kSpacing = 17;                // LDS rows between members 4t, 4t+1, 4t+2, 4t+3
-constexpr int kLdsRows = 15 + 3 * kSpacing + 1;
-constexpr int kDistPitch = kCap + 1;
 constexpr int kMaxChunk = 64;               // dimensions staged at once
-constexpr int kMaxLoads = kCap * (kMaxChunk / 4) / kThreads;   // 16-byte loads per thread and chunk
 
-// LDS row of bucket member m: the 4x4 block of thread t reads rows t, t+17, t+34,
-// t+51 -- consecutive t give conflict-free 16-byte reads (the pitch is an odd
-// number of 16-byte units) and the four rows of one block fall in different banks.
-__device__ __forceinline__ int phys_row(int m) { return (m >> 2) + kSpacing * (m & 3); }
+// CAP = largest bucket, THREADS = workgroup size (one 4x4 block of the pair matrix per thread must do),
+// SPACING = LDS rows between members 4t, 4t+1, 4t+2, 4t+3: the 4x4 block of thread t reads rows t, t+SPACING,
+// t+2 SPACING, t+3 SPACING -- consecutive t give conflict-free 16-byte reads (the pitch is an odd number of
+// 16-byte units) and the four rows of one block fall in different banks.
+template <int CAP, int THREADS, int SPACING>
+struct SmallCfg {
+    static constexpr int kWaves = THREADS / 64;
+    static constexpr int kBlocks = CAP / 4;
+    static constexpr int kLdsRows = (kBlocks - 1) + 3 * SPACING + 1;
+    static constexpr int kDistPitch = CAP + 1;
+    static constexpr int kMaxLoads = (CAP * (kMaxChunk / 4) + THREADS - 1) / THREADS;   // 16-byte loads per thread and chunk
+    static_assert(CAP % 4 == 0 && CAP <= 128 && THREADS % 64 == 0 && THREADS >= CAP, "shape");
+    static_assert(kBlocks * (kBlocks - 1) / 2 <= THREADS && 6 * kBlocks <= THREADS, "one block of the pair matrix per thread");
+    static_assert(SPACING >= kBlocks, "LDS rows of different members must not collide");
+    static_assert((CAP + kWaves - 1) / kWaves <= 32, "members of a wavefront must fit a 32-bit mask");
+};
 
-__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* __restrict__ points, int D, int K,
-                                                                  const int* __restrict__ ids,
-                                                                  const int* __restrict__ starts,
-                                                                  const int* __restrict__ sizes, int stride,
-                                                                  int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                                  int chunk, int pitch, int region_floats, int rows_sorted)
+// min_size: smaller buckets are left to another launch
+template <int CAP, int THREADS, int SPACING>
+__global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __restrict__ points, int D, int K,
+                                                                 const int* __restrict__ ids,
+                                                                 const int* __restrict__ starts,
+                                                                 const int* __restrict__ sizes, int stride, int min_size,
+                                                                 int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                                 int chunk, int pitch, int region_floats, int rows_sorted)
 {
+    using Cfg = SmallCfg<CAP, THREADS, SPACING>;
+    constexpr int kCap = CAP, kThreads = THREADS, kWaves = Cfg::kWaves, kSpacing = SPACING;
+    constexpr int kDistPitch = Cfg::kDistPitch, kMaxLoads = Cfg::kMaxLoads;
+    auto phys_row = [](int m) { return (m >> 2) + kSpacing * (m & 3); };     // LDS row of bucket member m
     // dynamic LDS: [rows | dist] (region_floats) | ids[64] | tau[64] | flag[64]
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
@@ -60,7 +72,7 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
-    if (s < 2 || s > kCap) return;
+    if (s < min_size || s > kCap) return;
     const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
@@ -189,8 +201,10 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
     // top-K update: a wavefront walks its members that have a candidate, four at a time, with the rows of the
     // next four in flight (the loop is bound by the latency of these row reads otherwise)
     const int my_id = lids[lane];
-    // bit u: member wave + 2 u has a candidate
-    uint32_t active = (uint32_t)ballot64(lane < 32 && flag[(wave + kWaves * lane) & (kCap - 1)] != 0);
+    const int my_id2 = (kCap > 64 && 64 + lane < kCap) ? lids[64 + lane] : -1;      // second round of candidates
+    // bit u: member wave + kWaves u has a candidate
+    const int fm = wave + kWaves * lane;
+    uint32_t active = (uint32_t)ballot64(lane < 32 && fm < kCap && flag[fm < kCap ? fm : 0] != 0);
     auto next_member = [&]() {
         if (active == 0) return -1;
         const int u = __ffs(active) - 1;
@@ -230,6 +244,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
             row.dist[0] = cur_rd[u];
             row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
             row.offer_lanes<true>(lane < s && lane != i, my_id, d);
+            if (kCap > 64) {
+                const int j2 = 64 + lane;
+                const float d2 = j2 < s ? dist[i * kDistPitch + j2] : INFINITY;
+                row.offer_lanes<true>(j2 < s && j2 != i, my_id2, d2);
+            }
             if (row.changed) {
                 const size_t at = (size_t)lids[i] * (size_t)K;
                 row.store(knn_idx + at, knn_dist + at);
@@ -242,28 +261,52 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_small(const float* _
 
 }  // namespace
 
-int small_bucket_cap() { return kCap; }
+int small_bucket_cap() { return kBucketSplit; }
+int medium_bucket_cap() { return 72; }
 
-// rows_sorted: every K-NN row is known to be sorted by distance (then members without a candidate below their
-// last slot are skipped)
+namespace {
+
+template <int CAP, int THREADS, int SPACING>
+int launch_cfg(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
+               int stride, int min_size, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream)
+{
+    using Cfg = SmallCfg<CAP, THREADS, SPACING>;
+    const int dpad = (D + 3) & ~3;
+    const int chunk = dpad < kMaxChunk ? dpad : kMaxChunk;
+    int pitch = chunk;
+    if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units
+    const int region = std::max(Cfg::kLdsRows * pitch, CAP * Cfg::kDistPitch);
+    const int region_floats = (region + 3) & ~3;
+    const size_t lds = (size_t)region_floats * 4 + (size_t)(3 * CAP) * 4;
+    auto kern = k_bucket_knn_small<CAP, THREADS, SPACING>;
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned)n_buckets), dim3(THREADS), lds, stream, points, D, K, ids, starts, sizes, stride,
+                       min_size, knn_idx, knn_dist, chunk, pitch, region_floats, rows_sorted ? 1 : 0);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+}  // namespace
+
+// Buckets of 2..64 points.  rows_sorted: every K-NN row is known to be sorted by distance (then members without
+// a candidate below their last slot are skipped).
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
                             int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream)
 {
     if (n_buckets <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
-    const int dpad = (D + 3) & ~3;
-    const int chunk = dpad < kMaxChunk ? dpad : kMaxChunk;
-    int pitch = chunk;
-    if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units
-    const int region = std::max(kLdsRows * pitch, kCap * kDistPitch);
-    const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)(3 * kCap) * 4;
-    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_small),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k_bucket_knn_small, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, D, K, ids,
-                       starts, sizes, stride, knn_idx, knn_dist, chunk, pitch, region_floats, rows_sorted ? 1 : 0);
-    RSFK_HIP(hipGetLastError());
-    return 0;
+    return launch_cfg<64, 128, 17>(points, D, K, ids, starts, sizes, n_buckets, stride, 2, rows_sorted, knn_idx, knn_dist,
+                                   stream);
+}
+
+// Buckets of 65..72 points (what a leaf limit of 2 (K + 1) with K = 32 leaves just above 64); other sizes are skipped.
+int launch_bucket_knn_medium(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                             int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream)
+{
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
+    return launch_cfg<72, 192, 19>(points, D, K, ids, starts, sizes, n_buckets, stride, 65, rows_sorted, knn_idx, knn_dist,
+                                   stream);
 }
 
 }  // namespace rsfk

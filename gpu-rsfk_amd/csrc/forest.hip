@@ -141,7 +141,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 (void)hipEventRecord(ev[j].a, stream);
                 rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w),
-                                            stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], d_idx, d_dist, stream);
+                                            stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], stats[5 * j + 2], d_idx, d_dist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
             }
             if (rc) break;

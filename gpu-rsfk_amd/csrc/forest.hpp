@@ -27,8 +27,8 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       hipStream_t stream);
 
 int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
-                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int* knn_idx,
-                           float* knn_dist, hipStream_t stream);
+                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
+                           int* knn_idx, float* knn_dist, hipStream_t stream);
 
 // bucket_knn_screen.hip
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);
@@ -37,6 +37,9 @@ int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int
 
 // bucket_knn_small.hip
 int small_bucket_cap();
+int medium_bucket_cap();
+int launch_bucket_knn_medium(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                             int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream);
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
                             int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream);
 
