@@ -258,7 +258,8 @@ __device__ __forceinline__ void resolve_exact(const int* list, int n, const floa
     }
 }
 
-constexpr int kSideBatch = 4;        // points per group and call of side_right8
+constexpr int kSideBatch = 4;        // points per group and call of the screen in the wide phase
+constexpr int kTailBatch = 2;        // ... in the tail kernel
 
 // Append a child node either to the next wide level or to the tail queue.
 __device__ __forceinline__ void emit_node(const TreeNode& c, const TreeParams& P, TreeNode* next, int next_cap,
@@ -657,12 +658,12 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
             // side of every point of the group's nodes
             const int total = pre_s[nb];
             const int iters = (total + kGroups - 1) / kGroups;
-            for (int it = 0; it < iters; it += kSideBatch) {
-                int id[kSideBatch], jj[kSideBatch], pos[kSideBatch];
-                float bb[kSideBatch], h1[kSideBatch], h2[kSideBatch];
-                bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
+            for (int it = 0; it < iters; it += kTailBatch) {
+                int id[kTailBatch], jj[kTailBatch], pos[kTailBatch];
+                float bb[kTailBatch], h1[kTailBatch], h2[kTailBatch];
+                bool valid[kTailBatch], right[kTailBatch], redo[kTailBatch];
 #pragma unroll
-                for (int u = 0; u < kSideBatch; ++u) {
+                for (int u = 0; u < kTailBatch; ++u) {
                     const int f = (it + u) * kGroups + grp;
                     valid[u] = f < total;
                     jj[u] = valid[u] ? fmap[f] : 0;
@@ -672,9 +673,9 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                     h1[u] = hp_s[jj[u]][1];
                     h2[u] = hp_s[jj[u]][2];
                 }
-                side_screen8<kSideBatch, false>(nvec, Dv, jj, bb, h1, h2, pb16, nullptr, id, P.D, P.band, valid, right, redo);
+                side_screen8<kTailBatch, false>(nvec, Dv, jj, bb, h1, h2, pb16, nullptr, id, P.D, P.band, valid, right, redo);
 #pragma unroll
-                for (int u = 0; u < kSideBatch; ++u) {
+                for (int u = 0; u < kTailBatch; ++u) {
                     if (valid[u] && sub8 == 0) {
                         if (redo[u]) tmp[atomicAdd(&n_def_s, 1)] = pos[u] | (jj[u] << 16);      // tmp is free until the partition
                         else if (right[u]) seg[pos[u]] = id[u] | (int)0x80000000;
