@@ -8,7 +8,8 @@ namespace {
 
 // one wavefront per row: convert, pad, and sum the squares of the rounded values
 __global__ __launch_bounds__(256) void k_to_bf16(const float* __restrict__ points, uint16_t* __restrict__ out,
-                                                 float* __restrict__ norms, int N, int D, int Db)
+                                                 float* __restrict__ norms, const float* __restrict__ mu, int N, int D,
+                                                 int Db)
 {
     const int lane = threadIdx.x & 63;
     const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(256) void k_to_bf16(const float* __restrict__ point
         uint16_t* dst = out + (size_t)r * (size_t)Db;
         float q = 0.0f;
         for (int d = lane; d < Db; d += 64) {
-            uint32_t u = d < D ? __float_as_uint(src[d]) : 0u;
+            uint32_t u = d < D ? __float_as_uint(mu ? src[d] - mu[d] : src[d]) : 0u;
             if ((u & 0x7f800000u) != 0x7f800000u) u += 0x7fffu + ((u >> 16) & 1u);      // finite: round to nearest even
             else if (u & 0x007fffffu) u |= 0x00400000u;                                  // NaN stays NaN
             u &= 0xffff0000u;
@@ -30,6 +31,28 @@ __global__ __launch_bounds__(256) void k_to_bf16(const float* __restrict__ point
         q += __shfl_xor(q, 1, 64); q += __shfl_xor(q, 2, 64); q += __shfl_xor(q, 4, 64);
         q += __shfl_xor(q, 8, 64); q += __shfl_xor(q, 16, 64); q += __shfl_xor(q, 32, 64);
         if (lane == 0) norms[r] = q;
+    }
+}
+
+// column sums: a workgroup adds up its share of the rows, 256 columns at a time, and adds the result to sum[]
+__global__ __launch_bounds__(256) void k_col_sum(const float* __restrict__ points, int N, int D, float* __restrict__ sum)
+{
+    const int rows_per = (N + gridDim.x - 1) / gridDim.x;
+    const int r0 = blockIdx.x * rows_per, r1 = min(N, r0 + rows_per);
+    for (int d = threadIdx.x; d < D; d += 256) {
+        float acc = 0.0f;
+        for (int r = r0; r < r1; ++r) acc += points[(size_t)r * (size_t)D + d];
+        atomicAdd(&sum[d], acc);
+    }
+}
+
+// sums -> means; a mean that is not finite is replaced by 0 (any shift is a valid one)
+__global__ void k_col_mean(float* __restrict__ mu, int D, float inv_n)
+{
+    const int d = blockIdx.x * blockDim.x + threadIdx.x;
+    if (d < D) {
+        const float m = mu[d] * inv_n;
+        mu[d] = fabsf(m) <= 3.0e38f ? m : 0.0f;
     }
 }
 
@@ -146,8 +169,9 @@ int q8_copy_mean_rho(const Q8Copy& c, int N, float* mean_rho, hipStream_t stream
 
 size_t bf16_copy_bytes(int N, int D) { return (size_t)N * ((size_t)bf16_pitch(D) * 2 + 4); }
 
-int bf16_copy_alloc(Bf16Copy* c, int N, int D)
+int bf16_copy_alloc(Bf16Copy* c, int N, int D, bool centred)
 {
+    if (centred && ws_alloc(reinterpret_cast<void**>(&c->mu), std::max<size_t>((size_t)D * 4, 16))) return 1;
     if (ws_alloc(reinterpret_cast<void**>(&c->rows), std::max<size_t>((size_t)N * bf16_pitch(D) * 2, 16))) return 1;
     if (ws_alloc(reinterpret_cast<void**>(&c->norms), std::max<size_t>((size_t)N * 4, 16))) return 1;
     return 0;
@@ -157,14 +181,22 @@ void bf16_copy_free(Bf16Copy* c)
 {
     ws_free(c->rows);
     ws_free(c->norms);
+    ws_free(c->mu);
+    c->mu = nullptr;
     c->rows = nullptr;
     c->norms = nullptr;
 }
 
 int bf16_copy_fill(const Bf16Copy& c, const float* points, int N, int D, hipStream_t stream)
 {
+    if (c.mu) {
+        RSFK_HIP(hipMemsetAsync(c.mu, 0, sizeof(float) * (size_t)D, stream));
+        const int g = std::max(1, std::min(N / 64, 2048));
+        hipLaunchKernelGGL(k_col_sum, dim3(g), dim3(256), 0, stream, points, N, D, c.mu);
+        hipLaunchKernelGGL(k_col_mean, dim3((D + 255) / 256), dim3(256), 0, stream, c.mu, D, 1.0f / (float)N);
+    }
     const int grid = std::min((N + 3) / 4, 65536);
-    hipLaunchKernelGGL(k_to_bf16, dim3(grid), dim3(256), 0, stream, points, c.rows, c.norms, N, D, bf16_pitch(D));
+    hipLaunchKernelGGL(k_to_bf16, dim3(grid), dim3(256), 0, stream, points, c.rows, c.norms, c.mu, N, D, bf16_pitch(D));
     RSFK_HIP(hipGetLastError());
     return 0;
 }

@@ -19,9 +19,16 @@ namespace rsfk {
 __host__ __device__ inline int bf16_pitch(int D) { return (D + 31) & ~31; }
 __host__ __device__ inline int bf16_valid(int D) { return (D + 7) & ~7; }
 
+//
+// A copy can be centred: the rows then hold x - mu rounded (first to fp32, then to bfloat16) with mu the
+// column means.  Distances do not change under a common shift, and the rounding errors -- proportional to the
+// magnitude of what is rounded -- shrink with the norms, so distance screens pass fewer candidates on data that
+// sits away from the origin.  fl(x - mu) adds a relative 2^-24 to the 2^-8 of the bfloat16 rounding; the bounds
+// of the consumers carry one per cent of slack for such terms.  Only screens of distances may use a centred copy.
 struct Bf16Copy {
     uint16_t* rows = nullptr;     // N x bf16_pitch(D)
     float* norms = nullptr;       // N
+    float* mu = nullptr;          // D column means the rows were shifted by, or null
 };
 
 // 8-bit screening copy of the points, used by the side test of the tree build when the rows have a narrow
@@ -48,7 +55,7 @@ int q8_copy_fill(const Q8Copy& c, const float* points, int N, int D, hipStream_t
 int q8_copy_mean_rho(const Q8Copy& c, int N, float* mean_rho, hipStream_t stream);     // synchronises the stream
 
 size_t bf16_copy_bytes(int N, int D);
-int bf16_copy_alloc(Bf16Copy* c, int N, int D);
+int bf16_copy_alloc(Bf16Copy* c, int N, int D, bool centred = false);
 void bf16_copy_free(Bf16Copy* c);
 int bf16_copy_fill(const Bf16Copy& c, const float* points, int N, int D, hipStream_t stream);
 

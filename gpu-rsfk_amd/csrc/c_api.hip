@@ -121,10 +121,16 @@ RSFK_API int rsfk_explore_device(const float* d_points, int N, int D, int num_ne
     int rc = bf16_copy_alloc(&bf, N, D);
     if (!rc) rc = bf16_copy_fill(bf, d_points, N, D, s);
     ExploreWorkspace* ws = nullptr;
-    if (!rc && explore_join_enabled(N, num_neighbors)) rc = explore_ws_alloc(&ws, N, num_neighbors);
-    if (!rc) rc = launch_explore(d_points, &bf, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, ws, s);
+    Bf16Copy bfc;            // centred copy for the join
+    if (!rc && explore_join_enabled(N, num_neighbors)) {
+        rc = explore_ws_alloc(&ws, N, num_neighbors);
+        if (!rc) rc = bf16_copy_alloc(&bfc, N, D, true);
+        if (!rc) rc = bf16_copy_fill(bfc, d_points, N, D, s);
+    }
+    if (!rc) rc = launch_explore(d_points, &bf, &bfc, N, D, num_neighbors, d_knn_indices, d_knn_sqr_distances, d_scratch, ws, s);
     if (!rc && hipStreamSynchronize(s) != hipSuccess) { set_last_error("hipStreamSynchronize failed"); rc = 1; }
     explore_ws_free(ws);
+    bf16_copy_free(&bfc);
     bf16_copy_free(&bf);
     return rc;
 }
@@ -205,12 +211,18 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
     int rc = bf16_copy_alloc(&bf, N, D);
     if (!rc) rc = bf16_copy_fill(bf, static_cast<const float*>(dp.p), N, D, nullptr);
     ExploreWorkspace* ws = nullptr;
-    if (!rc && explore_join_enabled(N, num_neighbors)) rc = explore_ws_alloc(&ws, N, num_neighbors);
+    Bf16Copy bfc;            // centred copy for the join
+    if (!rc && explore_join_enabled(N, num_neighbors)) {
+        rc = explore_ws_alloc(&ws, N, num_neighbors);
+        if (!rc) rc = bf16_copy_alloc(&bfc, N, D, true);
+        if (!rc) rc = bf16_copy_fill(bfc, static_cast<const float*>(dp.p), N, D, nullptr);
+    }
     for (int it = 0; it < passes && !rc; ++it)
-        rc = launch_explore(static_cast<const float*>(dp.p), &bf, N, D, num_neighbors, static_cast<int*>(dki.p),
+        rc = launch_explore(static_cast<const float*>(dp.p), &bf, &bfc, N, D, num_neighbors, static_cast<int*>(dki.p),
                             static_cast<float*>(dkd.p), static_cast<int*>(dold.p), ws, nullptr);
     if (!rc && hipDeviceSynchronize() != hipSuccess) { set_last_error("hipDeviceSynchronize failed"); rc = 1; }
     explore_ws_free(ws);
+    bf16_copy_free(&bfc);
     bf16_copy_free(&bf);
     if (rc) return rc;
     RSFK_HIP(hipDeviceSynchronize());

@@ -557,14 +557,16 @@ int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, cons
 
 // One exploration pass.  old_idx is scratch of N*K ints (receives the snapshot).
 // bf may be null (or hold null rows): every candidate then gets the exact distance.
-// ws may be null; with a workspace and a bfloat16 copy the candidates come from the join over the
-// reversed graph (explore_join.hip), which needs rows sorted by distance.
-int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K, int* knn_idx, float* knn_dist,
-                   int* old_idx, ExploreWorkspace* ws, hipStream_t stream)
+// ws may be null; with a workspace and a bfloat16 copy for the join (bf_join, may be centred; bf must not be)
+// the candidates come from the join over the reversed graph (explore_join.hip), which needs rows sorted by
+// distance.
+int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream)
 {
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
-    const bool join = ws != nullptr && bf != nullptr && bf->rows != nullptr;
+    RSFK_CHECK(bf == nullptr || bf->mu == nullptr, "exploration: the general kernel needs an uncentred copy");
+    const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr;
     if (join && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
     const int dpad = bf16_valid(D);
@@ -594,7 +596,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K,
         // Marks from the join, then the merge kernel with a small set (little LDS, many wavefronts per CU).
         // The points it cannot take come back in a list and get a second launch with the largest set that
         // fits; what is left after that goes to the general kernel below.
-        if (launch_explore_join(ws, b, N, D, K, old_idx, knn_dist, stream)) return 1;
+        if (launch_explore_join(ws, *bf_join, N, D, K, old_idx, knn_dist, stream)) return 1;
         const int* f2r = explore_ws_fwd2rev(ws);
         const uint32_t* pass = explore_ws_pass(ws);
         int* listA = explore_ws_todo(ws, 0);

@@ -174,9 +174,14 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         DevBuf old;
         if (ws_alloc(&old.p, sizeof(int) * (size_t)N * (size_t)K)) return 1;
         ExploreWsGuard ews;      // without a workspace every point enumerates its own candidates
-        if (explore_join_enabled(N, K) && explore_ws_alloc(&ews.w, N, K)) return 1;
+        Bf16Guard bfc;           // centred copy for the join
+        if (explore_join_enabled(N, K)) {
+            if (explore_ws_alloc(&ews.w, N, K)) return 1;
+            if (bf16_copy_alloc(&bfc.c, N, D, true) || bf16_copy_fill(bfc.c, d_points, N, D, stream)) return 1;
+        }
         for (int it = 0; it < nnef; ++it) {
-            if (launch_explore(d_points, &bf.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream)) return 1;
+            if (launch_explore(d_points, &bf.c, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream))
+                return 1;
         }
         RSFK_HIP(hipStreamSynchronize(stream));
     }

@@ -57,8 +57,8 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
                         const float* knn_dist, hipStream_t stream);
 
 // explore.hip
-int launch_explore(const float* points, const Bf16Copy* bf, int N, int D, int K, int* knn_idx, float* knn_dist,
-                   int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
+int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
 // forest.hip
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
