@@ -14,6 +14,8 @@
  *   - bucket K-NN update, diagonal schedule           src/kernels/compute_knn_from_buckets.cu:998-1378
  *   - neighbours-of-neighbours exploration            src/kernels/nearest_neighbors_exploring.cu:41-146
  *   - forest loop, seed increment, exploration loop   src/rsfk.cu:2033-2183
+ *   - query-set search: routing and bucket update     src/rsfk.cu:98-498,
+ *                                                     src/kernels/build_tree_update_parents_ann.cu:77-517
  *
  * Deliberate differences from the reference (none of them is pinned by any
  * fixture in the reference, see the parity notes at the end of this header):
@@ -42,6 +44,9 @@
  *                               graphs and by invariants
  *   tree build rules          : pinned by invariants, hand-traceable cases and
  *                               a pure-Python restatement of the same rules
+ *   query-set search          : routing pinned by a pure-Python restatement and by
+ *                               "a base point used as a query lands in its own leaf";
+ *                               the update by brute force inside the reached leaves
  *   random draw sequence      : parity unpinned (cuRAND is not available and
  *                               no reference fixture holds a partition)
  */
@@ -173,6 +178,7 @@ typedef struct {
     int depth;             /* level of the node, root = 0                        */
     int leaf;
     uint64_t key;
+    int qstart, qcount;    /* query points that reached the node = qperm[qstart .. +qcount) */
 } or_node;
 
 /*
@@ -181,12 +187,24 @@ typedef struct {
  * start order.  Returns the number of leaves, or -1 if leaf_cap is too small.
  * stats[0] = number of levels, stats[1] = max leaf size, stats[2] = min leaf size.
  */
-RSFK_OR_EXPORT int rsfk_or_build_tree(const float* points, int N, int D,
-                                      int MIN, int MAX, int MAX_DEPTH, int seed,
-                                      int* perm, int* leaf_start, int* leaf_size,
-                                      int leaf_cap, int* stats)
+/*
+ * The same with NQ query points routed down the tree while it is built (the routing of
+ * RSFK::knn_gpu_rsfk_forest_ann_tree, src/rsfk.cu:262-356: the side test of
+ * build_tree_check_points_side.cu on the query, then the child on that side, or the only child where the
+ * node has one -- src/kernels/build_tree_update_parents_ann.cu:141-151).  q_leaf_start/q_leaf_size
+ * (NQ ints each) receive the leaf each query ends in, as a segment of perm.  queries may be NULL.
+ */
+static int build_tree_ex(const float* points, int N, int D,
+                         int MIN, int MAX, int MAX_DEPTH, int seed,
+                         int* perm, int* leaf_start, int* leaf_size,
+                         int leaf_cap, int* stats,
+                         const float* queries, int NQ, int* q_leaf_start, int* q_leaf_size)
 {
     if (N <= 0) { if (stats) { stats[0] = 0; stats[1] = 0; stats[2] = 0; } return 0; }
+    if (!queries) NQ = 0;
+    int* qperm = (int*)malloc(sizeof(int) * (size_t)(NQ > 0 ? NQ : 1));
+    int* qtmp = (int*)malloc(sizeof(int) * (size_t)(NQ > 0 ? NQ : 1));
+    for (int i = 0; i < NQ; ++i) qperm[i] = i;
     int* tmp = (int*)malloc(sizeof(int) * (size_t)N);
     unsigned char* side = (unsigned char*)malloc((size_t)N);
     float* nvec = (float*)malloc(sizeof(float) * (size_t)(D > 0 ? D : 1));
@@ -195,15 +213,21 @@ RSFK_OR_EXPORT int rsfk_or_build_tree(const float* points, int N, int D,
     for (int i = 0; i < N; ++i) perm[i] = i;
 
     int n_leaves = 0, levels = 1, maxleaf = 0, minleaf = 0x7fffffff, overflow = 0;
-    or_node root = {0, N, 0, N, 0, 0, rsfk_or_root_key(seed)};   /* never a leaf: build_tree_init.cu:79 */
+    or_node root = {0, N, 0, N, 0, 0, rsfk_or_root_key(seed), 0, NQ};   /* never a leaf: build_tree_init.cu:79 */
     stack[top++] = root;
 
     while (top > 0) {
         or_node nd = stack[--top];
         if (nd.depth + 1 > levels) levels = nd.depth + 1;
         if (nd.leaf || nd.depth >= MAX_DEPTH - 1) {
-            if (n_leaves < leaf_cap) { leaf_start[n_leaves] = nd.start; leaf_size[n_leaves] = nd.count; }
-            else overflow = 1;
+            if (leaf_start) {
+                if (n_leaves < leaf_cap) { leaf_start[n_leaves] = nd.start; leaf_size[n_leaves] = nd.count; }
+                else overflow = 1;
+            }
+            for (int i = 0; i < nd.qcount; ++i) {
+                q_leaf_start[qperm[nd.qstart + i]] = nd.start;
+                q_leaf_size[qperm[nd.qstart + i]] = nd.count;
+            }
             ++n_leaves;
             if (nd.count > maxleaf) maxleaf = nd.count;
             if (nd.count < minleaf) minleaf = nd.count;
@@ -232,6 +256,18 @@ RSFK_OR_EXPORT int rsfk_or_build_tree(const float* points, int N, int D,
             }
             memcpy(perm + nd.start, tmp, sizeof(int) * (size_t)nd.count);
         }
+        /* the queries in the node take the same test; where the node gets one child they all follow it */
+        int qa = nd.qcount;
+        if (a != 0 && r != 0 && (a < r ? a : r) >= MIN) {
+            int il = 0, ir = 0;
+            for (int i = 0; i < nd.qcount; ++i) {
+                int q = qperm[nd.qstart + i];
+                int right = rsfk_or_dot32(nvec, queries + (size_t)q * D, D) < b;
+                if (right) qtmp[nd.qcount - 1 - ir++] = q; else qperm[nd.qstart + il++] = q;
+            }
+            qa = il;
+            for (int i = 0; i < ir; ++i) qperm[nd.qstart + il + i] = qtmp[nd.qcount - 1 - i];
+        }
         uint64_t kl = rsfk_or_child_key(nd.key, 0), kr = rsfk_or_child_key(nd.key, 1);
         or_node c0, c1; int nchild;
         if (a == 0 || r == 0) {
@@ -256,14 +292,35 @@ RSFK_OR_EXPORT int rsfk_or_build_tree(const float* points, int N, int D,
             c1.depth = nd.depth + 1; c1.key = kr; c1.leaf = r <= MAX - 2;
             nchild = 2;
         }
+        c0.qstart = nd.qstart; c0.qcount = nchild == 2 ? qa : nd.qcount;
+        c1.qstart = nd.qstart + qa; c1.qcount = nd.qcount - qa;
         if (top + 2 > cap) { cap *= 2; stack = (or_node*)realloc(stack, sizeof(or_node) * cap); }
         /* push right first so that leaves come out in ascending start order */
         if (nchild == 2) stack[top++] = c1;
         stack[top++] = c0;
     }
-    free(tmp); free(side); free(nvec); free(stack);
+    free(tmp); free(side); free(nvec); free(stack); free(qperm); free(qtmp);
     if (stats) { stats[0] = levels; stats[1] = maxleaf; stats[2] = n_leaves ? minleaf : 0; }
     return overflow ? -1 : n_leaves;
+}
+
+RSFK_OR_EXPORT int rsfk_or_build_tree(const float* points, int N, int D,
+                                      int MIN, int MAX, int MAX_DEPTH, int seed,
+                                      int* perm, int* leaf_start, int* leaf_size,
+                                      int leaf_cap, int* stats)
+{
+    return build_tree_ex(points, N, D, MIN, MAX, MAX_DEPTH, seed, perm, leaf_start, leaf_size, leaf_cap, stats,
+                         NULL, 0, NULL, NULL);
+}
+
+/* One tree on the points, the queries routed to their leaves: see build_tree_ex.  Returns the number of leaves. */
+RSFK_OR_EXPORT int rsfk_or_route_queries(const float* points, int N, int D,
+                                         int MIN, int MAX, int MAX_DEPTH, int seed,
+                                         const float* queries, int NQ,
+                                         int* perm, int* q_leaf_start, int* q_leaf_size)
+{
+    return build_tree_ex(points, N, D, MIN, MAX, MAX_DEPTH, seed, perm, NULL, NULL, 0, NULL,
+                         queries, NQ, q_leaf_start, q_leaf_size);
 }
 
 /* ------------------------------------------------------------------ */
@@ -463,6 +520,42 @@ RSFK_OR_EXPORT int rsfk_or_forest(int n_trees, int K, int N, int D,
 
 /* For each query row id in queries[0..nq): the K nearest points (the query
  * itself included), fp64 distances, ties broken by smaller index; sorted. */
+/*
+ * Query-set search (RSFK::knn_gpu_rsfk_forest_ann, src/rsfk.cu:98-155): for every tree (seed + tree index, as in
+ * the forest above) the queries are routed to a leaf and every point of that leaf is offered to the query's
+ * row (compute_knn_from_buckets_perwarp_coalesced_ann, src/kernels/build_tree_update_parents_ann.cu:239-517,
+ * update rule as everywhere).  Indices in q_idx refer to `points`.  No exploration pass (the reference accepts
+ * the parameter and ignores it).  Distances use the sequential chain of rsfk_or_sqdist like every other
+ * stage here; the reference's kernel uses its 32-lane form for this one.
+ */
+RSFK_OR_EXPORT int rsfk_or_ann_forest(int n_trees, int K, int N, int NQ, int D,
+                                      int MIN, int MAX, int MAX_DEPTH, int seed,
+                                      const float* points, const float* queries,
+                                      int* q_idx, float* q_dist)
+{
+    int* perm = (int*)malloc(sizeof(int) * (size_t)(N > 0 ? N : 1));
+    int* qs = (int*)malloc(sizeof(int) * (size_t)(NQ > 0 ? NQ : 1));
+    int* qz = (int*)malloc(sizeof(int) * (size_t)(NQ > 0 ? NQ : 1));
+    for (int t = 0; t < n_trees; ++t) {
+        rsfk_or_route_queries(points, N, D, MIN, MAX, MAX_DEPTH, seed + t, queries, NQ, perm, qs, qz);
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic, 64)
+#endif
+        for (int q = 0; q < NQ; ++q) {
+            int* idx = q_idx + (size_t)q * K;
+            float* dist = q_dist + (size_t)q * K;
+            int maxpos = first_max(dist, K);
+            for (int i = 0; i < qz[q]; ++i) {
+                int c = perm[qs[q] + i];
+                float d = rsfk_or_sqdist(queries + (size_t)q * D, points + (size_t)c * D, D);
+                try_insert(idx, dist, K, &maxpos, c, d);
+            }
+        }
+    }
+    free(perm); free(qs); free(qz);
+    return 0;
+}
+
 RSFK_OR_EXPORT void rsfk_or_bruteforce(const float* points, int N, int D, int K,
                                        const int* queries, int nq,
                                        int* out_idx, double* out_dist)

@@ -59,6 +59,11 @@ def lib():
         L.rsfk_or_explore.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _i32p, _f32p]
         L.rsfk_or_forest.restype = ctypes.c_int
         L.rsfk_or_forest.argtypes = [ctypes.c_int] * 9 + [_f32p, _i32p, _f32p, ctypes.c_void_p]
+        L.rsfk_or_route_queries.restype = ctypes.c_int
+        L.rsfk_or_route_queries.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            ctypes.c_int, ctypes.c_int, _f32p, ctypes.c_int, _i32p, _i32p, _i32p]
+        L.rsfk_or_ann_forest.restype = ctypes.c_int
+        L.rsfk_or_ann_forest.argtypes = [ctypes.c_int] * 9 + [_f32p, _f32p, _i32p, _f32p]
         L.rsfk_or_bruteforce.restype = None
         L.rsfk_or_bruteforce.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                          ctypes.c_int, _i32p, _f64p]
@@ -176,6 +181,38 @@ def forest(points, K, n_trees, min_children=-1, max_children=-1, max_depth=5000,
     if want_log:
         return knn_idx, knn_dist, log
     return knn_idx, knn_dist
+
+
+def route_queries(points, queries, min_children, max_children, max_depth=5000, seed=0):
+    """One tree on the points; -> perm, start and size (segments of perm) of the leaf every query ends in."""
+    points, queries = _pts(points), _pts(queries)
+    N, D = points.shape
+    NQ = queries.shape[0]
+    perm = np.empty(N, np.int32)
+    qs = np.full(NQ, -1, np.int32)
+    qz = np.full(NQ, -1, np.int32)
+    lib().rsfk_or_route_queries(points, N, D, int(min_children), int(max_children), int(max_depth), int(seed),
+                                queries, NQ, perm, qs, qz)
+    return perm, qs, qz
+
+
+def ann_forest(points, queries, K, n_trees, min_children=-1, max_children=-1, max_depth=5000, seed=0,
+               q_idx=None, q_dist=None):
+    """Query-set search; rows start empty (-1, +inf) unless given."""
+    points, queries = _pts(points), _pts(queries)
+    N, D = points.shape
+    NQ = queries.shape[0]
+    if min_children == -1:
+        min_children = K + 1
+    if max_children == -1:
+        max_children = 2 * min_children
+    if q_idx is None:
+        q_idx, q_dist = init_lists(NQ, K, self_in=False)
+    rc = lib().rsfk_or_ann_forest(int(n_trees), int(K), N, NQ, D, int(min_children), int(max_children),
+                                  int(max_depth), int(seed), points, queries, q_idx, q_dist)
+    if rc != 0:
+        raise RuntimeError("oracle query search failed")
+    return q_idx, q_dist
 
 
 def bruteforce(points, K, queries=None):

@@ -7,7 +7,10 @@ inputs.  They are written from the rules, not from the oracle's C code:
             expressed recursively over Python lists;
   insert  : "replace the maximum iff strictly closer and not present"
             (compute_knn_from_buckets.cu:1215-1230);
-  explore : nearest_neighbors_exploring.cu:70-141.
+  explore : nearest_neighbors_exploring.cu:70-141;
+  route   : the descent of a query point through a tree (src/rsfk.cu:262-356,
+            build_tree_update_parents_ann.cu:141-151): side test where the node has
+            two children, the only child otherwise.
 
 The random draws and the fp32 side test are taken from the oracle's exported
 helpers (pick_pair / hyperplane / dot32), which have their own tests.
@@ -53,6 +56,48 @@ def tree(orc, X, MIN, MAX, MAX_DEPTH, seed):
     finally:
         sys.setrecursionlimit(old)
     return buckets, levels[0]
+
+
+def route(orc, X, Q, MIN, MAX, MAX_DEPTH, seed):
+    """-> for every query the bucket (list of ids of X) it ends in.  The tree is the one of `tree` above; a query
+    is carried along the recursion instead of being routed afterwards."""
+    out = [None] * Q.shape[0]
+
+    def rec(members, draw_from, key, depth, leaf, queries):
+        if leaf or depth >= MAX_DEPTH - 1:
+            for q in queries:
+                out[q] = list(members)
+            return
+        r1, r2 = orc.pick_pair(key, len(draw_from))
+        n, b = orc.hyperplane(X[draw_from[r1]], X[draw_from[r2]])
+        left = [p for p in members if not (orc.dot32(n, X[p]) < b)]
+        right = [p for p in members if orc.dot32(n, X[p]) < b]
+        kl, kr = orc.child_key(key, 0), orc.child_key(key, 1)
+        c = len(members)
+        if not left or not right:
+            only = left if left else right
+            rec(only, only, kl if left else kr, depth + 1, c <= MAX - 2, queries)
+        elif min(len(left), len(right)) < MIN:
+            whole = left + right
+            if len(left) >= len(right):
+                rec(whole, left, kl, depth + 1, c <= MAX, queries)
+            else:
+                rec(whole, right, kr, depth + 1, c <= MAX, queries)
+        else:
+            ql = [q for q in queries if not (orc.dot32(n, Q[q]) < b)]
+            qr = [q for q in queries if orc.dot32(n, Q[q]) < b]
+            rec(left, left, kl, depth + 1, len(left) <= MAX - 2, ql)
+            rec(right, right, kr, depth + 1, len(right) <= MAX - 2, qr)
+
+    import sys
+    old = sys.getrecursionlimit()
+    sys.setrecursionlimit(max(old, MAX_DEPTH + 1000))
+    try:
+        ids = list(range(X.shape[0]))
+        rec(ids, ids, orc.root_key(seed), 0, False, list(range(Q.shape[0])))
+    finally:
+        sys.setrecursionlimit(old)
+    return out
 
 
 def insert(idx_row, dist_row, c, d):
