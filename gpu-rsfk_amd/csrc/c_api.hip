@@ -40,12 +40,15 @@ RSFK_API void pymodule_rsfk_knn(int n_trees, int num_neighbors, int N, int D, in
         die("pymodule_rsfk_knn");
 }
 
-RSFK_API void pymodule_rsfk_knn_ann(int, int, int, int, int, int, int, int, int, int, int, float*, float*, int*,
-                                    float*, float*)
+RSFK_API void pymodule_rsfk_knn_ann(int n_trees, int num_neighbors, int N, int NQ, int D, int MIN_TREE_CHILD,
+                                    int MAX_TREE_CHILD, int MAX_DEPTH, int VERBOSE, int RANDOM_STATE,
+                                    int /*nn_exploring_factor: accepted and ignored, as in the reference*/,
+                                    float* points, float* query_points, int* knn_indices, float* knn_sqr_distances,
+                                    float* log_forest)
 {
-    std::fprintf(stderr,
-                 "pymodule_rsfk_knn_ann: the query-set (ANN) path is not implemented in this library; "
-                 "outputs are left untouched\n");
+    if (knn_ann_forest_host(n_trees, num_neighbors, N, NQ, D, MIN_TREE_CHILD, MAX_TREE_CHILD, MAX_DEPTH, VERBOSE,
+                            RANDOM_STATE, points, query_points, knn_indices, knn_sqr_distances, log_forest))
+        die("pymodule_rsfk_knn_ann");
 }
 
 RSFK_API void pymodule_cluster_by_sample_tree(int N, int D, int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
@@ -99,6 +102,16 @@ RSFK_API int rsfk_knn_forest_device(int n_trees, int num_neighbors, int N, int D
     return knn_forest_device(n_trees, num_neighbors, N, D, MIN_TREE_CHILD, MAX_TREE_CHILD, MAX_DEPTH, VERBOSE,
                              RANDOM_STATE, nn_exploring_factor, d_points, d_knn_indices, d_knn_sqr_distances,
                              log_forest, static_cast<hipStream_t>(stream));
+}
+
+RSFK_API int rsfk_knn_ann_device(int n_trees, int num_neighbors, int N, int NQ, int D, int MIN_TREE_CHILD,
+                                 int MAX_TREE_CHILD, int MAX_DEPTH, int VERBOSE, int RANDOM_STATE,
+                                 const float* d_points, const float* d_query_points, int* d_knn_indices,
+                                 float* d_knn_sqr_distances, float* log_forest, void* stream)
+{
+    return knn_ann_forest_device(n_trees, num_neighbors, N, NQ, D, MIN_TREE_CHILD, MAX_TREE_CHILD, MAX_DEPTH, VERBOSE,
+                                 RANDOM_STATE, d_points, d_query_points, d_knn_indices, d_knn_sqr_distances, log_forest,
+                                 static_cast<hipStream_t>(stream));
 }
 
 RSFK_API int rsfk_bucket_knn_device(const float* d_points, int N, int D, int num_neighbors, const int* d_ids,

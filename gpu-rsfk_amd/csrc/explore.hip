@@ -41,13 +41,13 @@
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
 #include "forest.hpp"
+#include "exact_batch.hpp"
 #include <algorithm>
 
 namespace rsfk {
 
 namespace {
 
-constexpr int kChunk = 32;              // fp32 dimensions per staging step (exact path)
 constexpr int kPitch = kChunk + 4;      // 36 words = 9 x 16 B: conflict-free b128 reads down a column of rows
 constexpr int kBlockB = 128;            // bfloat16 dimensions per pipeline stage of the screen (2 x 64)
 constexpr int kQueue2 = 128;            // candidates waiting for the exact distance
@@ -74,85 +74,6 @@ __device__ __forceinline__ bool set_insert(int* table, int mask, int c, bool see
         h = (h + 1) & (uint32_t)mask;
     }
     return false;
-}
-
-struct ExploreLds {          // per wavefront; sizes fixed at launch
-    int* table;              // hash set / candidate list, table_size ints
-    int* srow;               // snapshot of the point's own row, K ints
-    int* queue2;             // candidates that passed the screen, waiting for the exact distance
-    float* xrow;             // the point's coordinates, zero padded to bf16_valid(D)
-    float* tile;             // 64 x (chunk + 4) words
-};
-
-// Load one 16-byte piece (4 dimensions) of a candidate row, zero beyond D.
-__device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int d, int D, bool vec_ok)
-{
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (d < D) {
-        if (vec_ok) {
-            v = *reinterpret_cast<const float4*>(row + d);
-        } else {
-            v.x = row[d];
-            if (d + 1 < D) v.y = row[d + 1];
-            if (d + 2 < D) v.z = row[d + 2];
-            if (d + 3 < D) v.w = row[d + 3];
-        }
-    }
-    return v;
-}
-
-// Exact distances of the first n candidates of `list` to the point, then offer them.  CH = dimensions
-// staged per step (32 or 16): a step moves 64 rows x CH floats through the tile.
-template <int SL, int CH = kChunk>
-__device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
-                                            const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row)
-{
-    constexpr int kPieces = CH / 4;         // 16-byte pieces of a row per step = lanes per row
-    constexpr int kRows = 64 / kPieces;     // rows per load instruction
-    constexpr int kLoads = 64 / kRows;      // load instructions per step
-    constexpr int kP = CH + 4;              // tile pitch: odd number of 16-byte units
-    const int lane = lane_id();
-    const int sub = lane / kPieces;         // which of the rows of a load instruction
-    const int piece = lane % kPieces;       // which 16-byte piece of the segment
-    const int my_c = lane < n ? list[lane] : -1;
-    const float* rp[kLoads];
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-        const int r = i * kRows + sub;
-        rp[i] = points + (size_t)list[r < n ? r : 0] * (size_t)D;      // rows beyond n repeat row 0 (ignored later)
-    }
-    float4 pre[kLoads];
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok);
-    float acc = 0.0f;
-    const float tau0 = row.tau;
-    for (int d0 = 0; d0 < D; d0 += CH) {
-        wave_lds_sync();                 // previous step's tile reads are done
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i)
-            *reinterpret_cast<float4*>(&L.tile[(i * kRows + sub) * kP + piece * 4]) = pre[i];
-        if (d0 + CH < D) {
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], d0 + CH + piece * 4, D, vec_ok);
-        }
-        wave_lds_sync();
-        const int pieces = min(kPieces, (D - d0 + 3) >> 2);
-        const float* mine = &L.tile[lane * kP];
-        const float* xs = &L.xrow[d0];
-        for (int q = 0; q < pieces; ++q) {
-            const float4 a = *reinterpret_cast<const float4*>(mine + 4 * q);
-            const float4 x = *reinterpret_cast<const float4*>(xs + 4 * q);
-            float df;
-            df = a.x - x.x; acc = __builtin_fmaf(df, df, acc);
-            df = a.y - x.y; acc = __builtin_fmaf(df, df, acc);
-            df = a.z - x.z; acc = __builtin_fmaf(df, df, acc);
-            df = a.w - x.w; acc = __builtin_fmaf(df, df, acc);
-        }
-        // partial sums only grow: once all of them reached the row maximum nothing can enter
-        if (ballot64(lane < n && acc < tau0) == 0) break;
-    }
-    wave_lds_sync();
-    row.offer_lanes(lane < n, my_c, acc);
 }
 
 __device__ __forceinline__ void screen_pair(uint32_t w, float x0, float x1, float& da, float& ta)

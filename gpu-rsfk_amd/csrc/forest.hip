@@ -194,6 +194,103 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     return 0;
 }
 
+// Query-set search (RSFK::knn_gpu_rsfk_forest_ann, src/rsfk.cu:98-155): n_trees trees on the base points (seed + tree
+// index, as in the forest above); per tree the queries are routed to a leaf and the base points of that leaf are
+// offered to the query's row.  Rows are merged into, indices refer to the base points.  The log receives the
+// per-tree series of the forest (tree statistics, tree time, update time) and the total time.
+int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                          const float* d_points, const float* d_queries, int* d_qidx, float* d_qdist, float* log_forest,
+                          hipStream_t stream)
+{
+    RSFK_CHECK(N >= 1 && D >= 1 && K >= 1 && NQ >= 0, "query-set search: N, D and K must be positive");
+    RSFK_CHECK(n_trees >= 0, "query-set search: n_trees must not be negative");
+    RSFK_CHECK(K <= 256, "query-set search: K above 256 is not supported");
+    if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
+    const double t0 = now_s();
+    if (n_trees > 0 && NQ > 0) {
+        Bf16Guard bf;
+        if (bf16_copy_alloc(&bf.c, N, D)) return 1;
+        if (bf16_copy_fill(bf.c, d_points, N, D, stream)) return 1;
+        Q8Guard q8;
+        const uint8_t* q8_rows = nullptr;
+        if (make_tree_screen(q8, d_points, N, D, verbose, stream, &q8_rows)) return 1;
+        const int B = choose_batch(n_trees, N, D, MIN);
+        WsGuard ws;
+        if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
+        if (tree_ws_enable_index(ws.w, MIN, MAX_DEPTH)) return 1;
+        DevBuf qs, qz;
+        if (ws_alloc(&qs.p, sizeof(int) * (size_t)NQ) || ws_alloc(&qz.p, sizeof(int) * (size_t)NQ)) return 1;
+        std::vector<int> stats((size_t)5 * B);
+        std::vector<EventPair> ev((size_t)B);
+        for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        int rc = 0;
+        for (int tb0 = 0; tb0 < n_trees && rc == 0; tb0 += B) {
+            const int nb = std::min(B, n_trees - tb0);
+            const double tt0 = now_s();
+            rc = build_tree_batch(ws.w, d_points, bf.c.rows, q8_rows, N, D, MIN, MAX, MAX_DEPTH, seed + tb0, nb, stats.data(),
+                                  stream);
+            if (rc) break;
+            const double tt = now_s() - tt0;
+            for (int j = 0; j < nb && rc == 0; ++j) {
+                (void)hipEventRecord(ev[j].a, stream);
+                rc = launch_route_queries(d_points, d_queries, NQ, D, tree_ws_recs(ws.w, j), tree_ws_rec_cap(ws.w),
+                                          static_cast<int*>(qs.p), static_cast<int*>(qz.p), stream);
+                if (!rc)
+                    rc = launch_ann_knn(d_points, d_queries, NQ, D, K, tree_ws_perm(ws.w, j), static_cast<int*>(qs.p),
+                                        static_cast<int*>(qz.p), d_qidx, d_qdist, stream);
+                (void)hipEventRecord(ev[j].b, stream);
+            }
+            if (rc) break;
+            RSFK_HIP(hipStreamSynchronize(stream));
+            for (int j = 0; j < nb; ++j) {
+                float ms = 0.0f;
+                (void)hipEventElapsedTime(&ms, ev[j].a, ev[j].b);
+                const int t = tb0 + j;
+                if (log_forest) {
+                    log_forest[(size_t)0 * n_trees + t] = (float)stats[5 * j + 1];   // Tree Depth
+                    log_forest[(size_t)1 * n_trees + t] = (float)stats[5 * j + 2];   // Max Leaf Size
+                    log_forest[(size_t)2 * n_trees + t] = (float)stats[5 * j + 3];   // Min Leaf Size
+                    log_forest[(size_t)3 * n_trees + t] = (float)stats[5 * j + 0];   // Total Leaves
+                    log_forest[(size_t)5 * n_trees + t] = (float)(tt / nb);          // Total Tree Building Time
+                    log_forest[(size_t)15 * n_trees + t] = ms * 1e-3f;               // KNN Sets Updates
+                }
+                if (verbose >= 2)
+                    std::printf("tree %d: depth %d, leaves %d, leaf size %d..%d, query update %.6f s\n", t, stats[5 * j + 1],
+                                stats[5 * j + 0], stats[5 * j + 3], stats[5 * j + 2], ms * 1e-3);
+            }
+        }
+        for (auto& e : ev) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+        if (rc) return rc;
+    }
+    const double t_total = now_s() - t0;
+    if (verbose >= 1) std::printf("Query-set search over %d trees takes %lf seconds\n", n_trees, t_total);
+    if (log_forest) log_forest[(size_t)16 * n_trees] = (float)t_total;
+    return 0;
+}
+
+int knn_ann_forest_host(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                        const float* points, const float* queries, int* q_idx, float* q_dist, float* log_forest)
+{
+    RSFK_CHECK(N >= 1 && D >= 1 && K >= 1 && NQ >= 0, "query-set search: N, D and K must be positive");
+    if (NQ == 0) return 0;
+    DevBuf dp, dq, di, dd;
+    const size_t nd = (size_t)N * (size_t)D, qd = (size_t)NQ * (size_t)D, nk = (size_t)NQ * (size_t)K;
+    if (ws_alloc(&dp.p, nd * sizeof(float)) || ws_alloc(&dq.p, qd * sizeof(float)) || ws_alloc(&di.p, nk * sizeof(int)) ||
+        ws_alloc(&dd.p, nk * sizeof(float)))
+        return 1;
+    RSFK_HIP(hipMemcpy(dp.p, points, nd * sizeof(float), hipMemcpyHostToDevice));
+    RSFK_HIP(hipMemcpy(dq.p, queries, qd * sizeof(float), hipMemcpyHostToDevice));
+    RSFK_HIP(hipMemcpy(di.p, q_idx, nk * sizeof(int), hipMemcpyHostToDevice));
+    RSFK_HIP(hipMemcpy(dd.p, q_dist, nk * sizeof(float), hipMemcpyHostToDevice));
+    const int rc = knn_ann_forest_device(n_trees, K, N, NQ, D, MIN, MAX, MAX_DEPTH, verbose, seed,
+                                         static_cast<const float*>(dp.p), static_cast<const float*>(dq.p),
+                                         static_cast<int*>(di.p), static_cast<float*>(dd.p), log_forest, nullptr);
+    if (rc) return rc;
+    RSFK_HIP(hipMemcpy(q_idx, di.p, nk * sizeof(int), hipMemcpyDeviceToHost));
+    RSFK_HIP(hipMemcpy(q_dist, dd.p, nk * sizeof(float), hipMemcpyDeviceToHost));
+    return 0;
+}
+
 int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                     int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest)
 {

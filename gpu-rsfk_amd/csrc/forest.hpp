@@ -12,6 +12,8 @@ struct TreeBatchWorkspace;
 size_t tree_ws_bytes(int N, int D, int MIN, int B);
 int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B);
 void tree_ws_free(TreeBatchWorkspace* w);
+int tree_ws_enable_index(TreeBatchWorkspace* w, int MIN, int MAX_DEPTH);
+const TreeRec* tree_ws_recs(const TreeBatchWorkspace* w, int t);
 int tree_ws_leaf_cap(const TreeBatchWorkspace* w);
 const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
@@ -60,7 +62,19 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
+// ann.hip
+int launch_route_queries(const float* points, const float* queries, int NQ, int D, const TreeRec* recs, int n_rec,
+                         int* q_start, int* q_size, hipStream_t stream);
+int launch_ann_knn(const float* points, const float* queries, int NQ, int D, int K, const int* perm, const int* q_start,
+                   const int* q_size, int* q_idx, float* q_dist, hipStream_t stream);
+
 // forest.hip
+int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                          const float* d_points, const float* d_queries, int* d_qidx, float* d_qdist, float* log_forest,
+                          hipStream_t stream);
+int knn_ann_forest_host(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
+                        const float* points, const float* queries, int* q_idx, float* q_dist, float* log_forest);
+int tree_ws_rec_cap(const TreeBatchWorkspace* w);
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                       int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
                       hipStream_t stream);

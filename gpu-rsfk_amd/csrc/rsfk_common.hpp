@@ -96,7 +96,17 @@ struct TreeNode {
     int depth;        // level of the node, root = 0
     int buf;          // which of the two permutation buffers holds the members
     int leaf;         // 1 = already decided to be a bucket
+    int rec;          // where the node is written in the index of the tree (only when an index is recorded)
+    int pad_;
     uint64_t key;
+};
+
+// Index of a tree for routing query points (recorded only on request).  Internal node with two children: a, b =
+// the drawn pair of points, c0 / c1 = records of the left / right child.  Bucket: a = start of its segment of the
+// tree's permutation, b = its size, c0 = c1 = -1.  A node with one child has no record (its child stands in its
+// place).  Record 0 is the root.
+struct TreeRec {
+    int a, b, c0, c1;
 };
 
 // Buckets of at most this many points are handled by the small-bucket K-NN kernel; the

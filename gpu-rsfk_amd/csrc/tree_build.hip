@@ -288,6 +288,8 @@ __device__ __forceinline__ int split_rules(const TreeNode& nd, int a, int MIN, i
     c0.tree = c1.tree = nd.tree;
     c0.depth = c1.depth = nd.depth + 1;
     c0.buf = c1.buf = child_buf;
+    c0.rec = c1.rec = 0;
+    c0.pad_ = c1.pad_ = 0;
     if (a == 0 || r == 0) {
         c0.start = nd.start; c0.count = nd.count; c0.dstart = nd.start; c0.dcount = nd.count;
         c0.key = a ? kl : kr; c0.leaf = nd.count <= MAX - 2;
@@ -308,6 +310,40 @@ __device__ __forceinline__ int split_rules(const TreeNode& nd, int a, int MIN, i
     return 2;
 }
 
+// Index of the tree (TreeRec): reserve the records of the children of node nd and write nd's own record.
+// recs / n_rec belong to the tree of nd.  p1, p2: the drawn pair.  A node with one child (an empty side, or the
+// min-size merge) routes every query the same way: it leaves no record and its child takes over its place, so a
+// tree has fewer than twice as many records as buckets whatever its depth.
+__device__ __forceinline__ void index_split(TreeRec* recs, int* n_rec, int rec_cap, int my_rec, int p1, int p2, int nc,
+                                            int& rec0, int& rec1, LevelCounters* ctr)
+{
+    if (nc != 2) {
+        rec0 = rec1 = my_rec;
+        return;
+    }
+    const int base = atomicAdd(n_rec, 2);
+    rec0 = base;
+    rec1 = base + 1;
+    if (base + 2 <= rec_cap && my_rec < rec_cap) {
+        TreeRec r;
+        r.a = p1; r.b = p2; r.c0 = rec0; r.c1 = rec1;
+        recs[my_rec] = r;
+    } else {
+        ctr->overflow = 1;
+    }
+}
+
+__device__ __forceinline__ void index_bucket(TreeRec* recs, int rec_cap, int my_rec, int start, int count, LevelCounters* ctr)
+{
+    if (my_rec < rec_cap) {
+        TreeRec r;
+        r.a = start; r.b = count; r.c0 = -1; r.c1 = -1;
+        recs[my_rec] = r;
+    } else {
+        ctr->overflow = 1;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // wide phase kernels
 // ---------------------------------------------------------------------------
@@ -319,12 +355,15 @@ __global__ void k_init_perm(int* __restrict__ perm, int N, int B)
         perm[i] = (int)(i % (size_t)N);
 }
 
-__global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr, TreeParams P, int B, int seed0)
+__global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr, TreeParams P, int B, int seed0,
+                             int* n_rec)
 {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= B) return;
+    if (n_rec) n_rec[t] = 1;               // record 0 is the root
     TreeNode r;
     r.tree = t; r.start = 0; r.count = P.N; r.dstart = 0; r.dcount = P.N; r.depth = 0; r.buf = 0; r.leaf = 0;
+    r.rec = 0; r.pad_ = 0;
     r.key = root_key(seed0 + t);
     // the root is never a leaf (src/kernels/build_tree_init.cu:79) unless the depth limit forces it
     emit_node(r, P, nodes, B, tail, B, ctr);
@@ -454,7 +493,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
                                                     const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
                                                     const int* __restrict__ chunk2node, const int* __restrict__ chunk_left,
                                                     TreeNode* __restrict__ next, int next_cap,
-                                                    TreeNode* __restrict__ tail, int tail_cap, LevelCounters* ctr)
+                                                    TreeNode* __restrict__ tail, int tail_cap, LevelCounters* ctr,
+                                                    TreeRec* __restrict__ recs, int* __restrict__ n_rec, int rec_cap)
 {
     __shared__ int red[2][kBlock / 64];
     __shared__ int wcnt[kBlock / 64];
@@ -510,6 +550,12 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
     if (k == 0 && tid == 0) {
         TreeNode c0, c1;
         const int nc = split_rules(nd, all, P.MIN, P.MAX, nd.buf ^ 1, c0, c1);
+        if (recs) {
+            int r1, r2;
+            pick_pair(nd.key, nd.dcount, r1, r2);
+            index_split(recs + (size_t)nd.tree * rec_cap, n_rec + nd.tree, rec_cap, nd.rec, src[nd.dstart + r1] & kIdMask,
+                        src[nd.dstart + r2] & kIdMask, nc, c0.rec, c1.rec, ctr);
+        }
         emit_node(c0, P, next, next_cap, tail, tail_cap, ctr);
         if (nc == 2) emit_node(c1, P, next, next_cap, tail, tail_cap, ctr);
     }
@@ -521,6 +567,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
 struct SmallNode {
     int start, count, dstart, dcount;     // offsets inside the task's segment
     int depth, leaf;
+    int rec, pad_;                        // record of the node in the index of the tree, if one is written
     uint64_t key;
 };
 
@@ -571,7 +618,8 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                                                  int* __restrict__ perm_out,
                                                  const TreeNode* __restrict__ tasks, int n_tasks, int node_cap, int G,
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
-                                                 TreeStats* stats, LevelCounters* ctr)
+                                                 TreeStats* stats, LevelCounters* ctr,
+                                                 TreeRec* __restrict__ recs_all, int* __restrict__ n_rec_all, int rec_cap)
 {
     // dynamic LDS: seg[small] | tmp[small] | nvec[G][nvec_len(D)] | lrec[node_cap] | level lists 2 x node_cap | fmap[small]
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -601,20 +649,26 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         // already a bucket (any size): move it to the output buffer and record it
         if (src != dst)
             for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = src[tk.start + i] & kIdMask;
-        if (tid == 0) emit_leaf(tk.tree, tk.start, tk.count, tk.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
+        if (tid == 0) {
+            emit_leaf(tk.tree, tk.start, tk.count, tk.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
+            if (recs_all) index_bucket(recs_all + (size_t)tk.tree * rec_cap, rec_cap, tk.rec, tk.start, tk.count, ctr);
+        }
         return;
     }
+    TreeRec* recs = recs_all ? recs_all + (size_t)tk.tree * rec_cap : nullptr;
+    int* n_rec = recs_all ? n_rec_all + tk.tree : nullptr;
     for (int i = tid; i < tk.count; i += kBlock) seg[i] = src[tk.start + i] & kIdMask;
     if (tid == 0) {
         SmallNode r;
         r.start = 0; r.count = tk.count; r.dstart = tk.dstart - tk.start; r.dcount = tk.dcount;
-        r.depth = tk.depth; r.leaf = 0; r.key = tk.key;
+        r.depth = tk.depth; r.leaf = 0; r.key = tk.key; r.rec = tk.rec; r.pad_ = 0;
         cur[0] = r;
         n_cur_s = 1; n_nxt_s = 0; nrec_s = 0; kind_s[0] = 0; kind_s[1] = 0; lev_s = 0; mx_s = 0; mn_s = 0x7fffffff;
     }
     __syncthreads();
 
-    auto record_leaf = [&](int start, int count, int depth) {
+    auto record_leaf = [&](int start, int count, int depth, int rec) {
+        if (recs) index_bucket(recs, rec_cap, rec, tk.start + start, count, ctr);
         const int at = atomicAdd(&nrec_s, 1);
         const int rank = atomicAdd(&kind_s[count > kBucketSplit ? 1 : 0], 1);
         if (at < node_cap) lrec[at] = make_int2(tk.start + start, count | (rank << 16)); else ctr->overflow = 1;
@@ -714,15 +768,16 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                 full.tree = tk.tree; full.start = nd.start; full.count = nd.count; full.dstart = nd.dstart;
                 full.dcount = nd.dcount; full.depth = nd.depth; full.buf = 0; full.leaf = 0; full.key = nd.key;
                 const int nc = split_rules(full, left_s[tid], P.MIN, P.MAX, 0, c[0], c[1]);
+                if (recs) index_split(recs, n_rec, rec_cap, nd.rec, pair_s[tid][0], pair_s[tid][1], nc, c[0].rec, c[1].rec, ctr);
                 for (int q = 0; q < nc; ++q) {
                     if (c[q].leaf || c[q].depth >= P.MAX_DEPTH - 1) {
-                        record_leaf(c[q].start, c[q].count, c[q].depth);
+                        record_leaf(c[q].start, c[q].count, c[q].depth, c[q].rec);
                     } else {
                         const int at = atomicAdd(&n_nxt_s, 1);
                         if (at < node_cap) {
                             SmallNode sn;
                             sn.start = c[q].start; sn.count = c[q].count; sn.dstart = c[q].dstart; sn.dcount = c[q].dcount;
-                            sn.depth = c[q].depth; sn.leaf = 0; sn.key = c[q].key;
+                            sn.depth = c[q].depth; sn.leaf = 0; sn.key = c[q].key; sn.rec = c[q].rec; sn.pad_ = 0;
                             nxt[at] = sn;
                         } else {
                             ctr->overflow = 1;
@@ -781,12 +836,16 @@ struct TreeBatchWorkspace {
     int D = 0;
     LevelCounters* h_ctr = nullptr;      // pinned
     TreeStats* h_stats = nullptr;        // pinned
+    // index of the trees for routing query points (allocated by tree_ws_enable_index)
+    TreeRec* recs = nullptr;             // B x rec_cap
+    int* n_rec = nullptr;                // B
+    int rec_cap = 0;
 };
 
 static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
-                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr};
+                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec};
     for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
@@ -813,6 +872,21 @@ size_t tree_ws_bytes(int N, int D, int MIN, int B)
     const size_t lc = (size_t)N / (size_t)std::max(MIN, 1) + 2;
     return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24));
 }
+
+// From now on every build with this workspace also writes the index of each tree (TreeRec records).
+int tree_ws_enable_index(TreeBatchWorkspace* w, int MIN, int MAX_DEPTH)
+{
+    if (w->recs) return 0;
+    // buckets <= N / MIN + 1, two-child nodes fewer than buckets, plus the one-child nodes of re-draws
+    const size_t cap = (size_t)8 * ((size_t)w->N / (size_t)std::max(MIN, 1) + 2) + 2 * (size_t)std::max(MAX_DEPTH, 0) + 64;
+    RSFK_CHECK(cap < ((size_t)1 << 30), "tree index: too many nodes");
+    w->rec_cap = (int)cap;
+    if (dmalloc(&w->recs, (size_t)w->B * cap)) return 1;
+    if (dmalloc(&w->n_rec, (size_t)w->B)) return 1;
+    return 0;
+}
+const TreeRec* tree_ws_recs(const TreeBatchWorkspace* w, int t) { return w->recs + (size_t)t * w->rec_cap; }
+int tree_ws_rec_cap(const TreeBatchWorkspace* w) { return w->rec_cap; }
 
 int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
 {
@@ -871,7 +945,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     std::memcpy(w->h_stats, init.data(), sizeof(TreeStats) * (size_t)nb);
     RSFK_HIP(hipMemcpyAsync(w->stats, w->h_stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyHostToDevice, stream));
     RSFK_HIP(hipMemsetAsync(w->ctr, 0, sizeof(LevelCounters), stream));
-    hipLaunchKernelGGL(k_init_roots, dim3((nb + 63) / 64), dim3(64), 0, stream, w->nodes[0], w->tail, w->ctr, P, nb, seed0);
+    hipLaunchKernelGGL(k_init_roots, dim3((nb + 63) / 64), dim3(64), 0, stream, w->nodes[0], w->tail, w->ctr, P, nb, seed0,
+                       w->n_rec);
     RSFK_HIP(hipGetLastError());
 
     int cur = 0;
@@ -899,7 +974,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
             hipLaunchKernelGGL(k_side<false>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
                                w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
-                           w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr);
+                           w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
+                           w->recs, w->n_rec, w->rec_cap);
         RSFK_HIP(hipGetLastError());
         cur ^= 1;
     }
@@ -917,7 +993,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
-                           w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr);
+                           w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr, w->recs, w->n_rec,
+                           w->rec_cap);
         RSFK_HIP(hipGetLastError());
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));

@@ -189,10 +189,84 @@ class RSFK(object):
         self._last_search_time = time.time() - t_init
         return knn_indices, knn_squared_dist
 
-    def find_nearest_neighbors_ann(self, *args, **kwargs):
-        """The query-set search of the reference (RSFK.py:371-539) is not part of
-        this library."""
-        raise NotImplementedError("find_nearest_neighbors_ann is not implemented by the MI355X library")
+    def find_nearest_neighbors_ann(self, points, query_points, num_nearest_neighbors,
+                                   n_trees=-1, max_tree_depth=5000,
+                                   verbose=0, min_tree_children=-1,
+                                   max_tree_children=-1,
+                                   ensure_valid_indices=True,
+                                   add_bit_random_motion=False,
+                                   random_motion_force=1.0,
+                                   nn_exploring_factor=-1):
+        """Neighbours of ``query_points`` among ``points`` (reference RSFK.py:371-539).
+
+        Every tree is built on ``points``; a query is routed to one bucket per tree
+        and the points of that bucket are merged into its row.  Parameters and
+        defaults as in ``find_nearest_neighbors``; ``nn_exploring_factor`` is passed
+        on and ignored by the library, as in the reference.
+
+        Returns
+        -------
+        knn_indices : int32 ndarray (NQ, K), indices into ``points``, -1 = empty slot
+        knn_squared_dist : float32 ndarray (NQ, K)
+        """
+        points = np.require(points, np.float32, ['CONTIGUOUS', 'ALIGNED'])
+
+        max_tree_depth = int(max_tree_depth)
+        verbose = int(verbose)
+        max_tree_children = int(max_tree_children)
+        min_tree_children = int(min_tree_children)
+        N = points.shape[0]
+        NQ = query_points.shape[0]
+        D = points.shape[1]
+        K = int(num_nearest_neighbors)
+        n_trees = int(n_trees)
+
+        if nn_exploring_factor == -1:
+            nn_exploring_factor = 1 if K <= 32 else 0
+
+        if min_tree_children == -1:
+            min_tree_children = K + 1
+        if min_tree_children < 0:
+            raise Exception('min_tree_children = {} \t => min_tree_children must be at least 1'.format(min_tree_children))
+        if max_tree_children == -1:
+            max_tree_children = 2 * min_tree_children
+        if max_tree_children < 2 * min_tree_children:
+            raise Exception('min_tree_children = {}, max_tree_children = {} \t => max_tree_children must be at least 2*min_tree_children'.format(min_tree_children, max_tree_children))
+
+        if n_trees == -1:
+            avg_bucket_size = (min_tree_children + max_tree_children) / 2
+            n_trees = (N * D) / (avg_bucket_size * 24913)
+            n_trees = max(np.ceil(n_trees), 50)
+            if verbose > 0:
+                print("Automatically setting n_trees to {}".format(n_trees))
+        n_trees = int(n_trees)
+
+        if add_bit_random_motion:
+            random_motion(points, random_motion_force)
+            random_motion(query_points, random_motion_force)
+        points = np.require(points, np.float32, ['CONTIGUOUS', 'ALIGNED'])
+        query_points = np.require(query_points, np.float32, ['CONTIGUOUS', 'ALIGNED'])
+
+        knn_indices = np.full((NQ, K), -1, dtype=np.int32)
+        knn_squared_dist = np.full((NQ, K), np.inf, dtype=np.float32)
+
+        t_init = time.time()
+
+        log_forest = np.zeros(n_trees * 16 + 2, dtype=np.float32)
+        self._lib.pymodule_rsfk_knn_ann(
+            n_trees, K, N, NQ, D, min_tree_children, max_tree_children, max_tree_depth,
+            verbose, self.random_state, int(nn_exploring_factor),
+            points, query_points, knn_indices, knn_squared_dist, log_forest)
+
+        if ensure_valid_indices and min_tree_children < K + 1:
+            log_extra = np.zeros(1 * 16 + 2, dtype=np.float32)
+            self._lib.pymodule_rsfk_knn_ann(
+                1, K, N, NQ, D, K + 1, 3 * (K + 1), max_tree_depth,
+                verbose, self.random_state, int(nn_exploring_factor),
+                points, query_points, knn_indices, knn_squared_dist, log_extra)
+
+        self._last_search_time = time.time() - t_init
+        return knn_indices, knn_squared_dist
 
     def cluster_by_sample_tree(self, points, max_tree_depth=5000,
                                verbose=1, min_tree_children=32,

@@ -19,6 +19,7 @@ SYMBOLS = {
     "pymodule_rsfk_knn_ann": (None, [_ci] * 11 + [_vp, _vp, _vp, _vp, _vp]),
     "pymodule_cluster_by_sample_tree": (None, [_ci] * 7 + [_vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_forest_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp]),
+    "rsfk_knn_ann_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp, _vp]),
     "rsfk_bucket_knn_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _ci, _ci, _vp, _vp, _vp]),
     "rsfk_explore_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
     "rsfk_build_tree_host": (_ci, [_f32, _ci, _ci, _ci, _ci, _ci, _ci, _i32, _i32, _i32, _ci, _i32]),
@@ -101,6 +102,15 @@ def knn_forest_device(n_trees, K, N, D, min_children, max_children, max_depth, v
     _check(lib().rsfk_knn_forest_device(int(n_trees), int(K), int(N), int(D), int(min_children), int(max_children),
                                         int(max_depth), int(verbose), int(seed), int(nnef),
                                         _vp(d_points), _vp(d_idx), _vp(d_dist), lp, _vp(stream)))
+
+
+def knn_ann_device(n_trees, K, N, NQ, D, min_children, max_children, max_depth, verbose, seed,
+                   d_points, d_queries, d_idx, d_dist, log=None, stream=0):
+    """Query-set search on device-resident buffers (integer addresses); rows NQ x K are merged into."""
+    lp = None if log is None else log.ctypes.data_as(_vp)
+    _check(lib().rsfk_knn_ann_device(int(n_trees), int(K), int(N), int(NQ), int(D), int(min_children),
+                                     int(max_children), int(max_depth), int(verbose), int(seed),
+                                     _vp(d_points), _vp(d_queries), _vp(d_idx), _vp(d_dist), lp, _vp(stream)))
 
 
 def bucket_knn_device(d_points, N, D, K, d_ids, d_starts, d_sizes, n_buckets, stride, d_idx, d_dist, stream=0):

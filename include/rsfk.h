@@ -38,10 +38,14 @@ void pymodule_rsfk_knn(int n_trees, int num_neighbors, int N, int D,
                        float* points, int* knn_indices, float* knn_sqr_distances,
                        float* log_forest);
 
-/* Query-set variant of the reference (src/python/pymodule_ext.cu:149-181).  Not
- * implemented: the symbol exists because the Python layer binds it on
- * construction (python/gpu_rsfk/RSFK.py:134); a call prints a message to stderr
- * and leaves the outputs untouched. */
+/* Query-set search.  Replaces pymodule_rsfk_knn_ann (src/python/pymodule_ext.cu:149-181 ->
+ * RSFK::knn_gpu_rsfk_forest_ann, src/rsfk.cu:98-498): n_trees trees are built on `points`
+ * (tree t with seed RANDOM_STATE + t); per tree every query point is routed to a leaf and
+ * the points of that leaf are merged into the query's row.  knn_indices / knn_sqr_distances
+ * are NQ x num_neighbors, in/out (merged into, -1 / +inf = empty), indices refer to
+ * `points`.  nn_exploring_factor is accepted and ignored, as in the reference.
+ * log_forest: 16*n_trees+2 floats (series of pymodule_rsfk_knn; entry 16*n_trees = total
+ * seconds).  Errors: message on stderr, exit(1). */
 void pymodule_rsfk_knn_ann(int n_trees, int num_neighbors, int N, int NQ, int D,
                            int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
                            int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
@@ -74,6 +78,17 @@ int rsfk_knn_forest_device(int n_trees, int num_neighbors, int N, int D,
                            int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
                            const float* d_points, int* d_knn_indices, float* d_knn_sqr_distances,
                            float* log_forest, void* stream);
+
+/* pymodule_rsfk_knn_ann with device-resident buffers (points N x D, queries NQ x D, rows
+ * NQ x num_neighbors); log_forest is host memory or NULL.  Replaces the body of
+ * RSFK::knn_gpu_rsfk_forest_ann between its copies (src/rsfk.cu:117-128).  Returns 0, or
+ * nonzero with the reason in rsfk_last_error(). */
+int rsfk_knn_ann_device(int n_trees, int num_neighbors, int N, int NQ, int D,
+                        int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                        int VERBOSE, int RANDOM_STATE,
+                        const float* d_points, const float* d_query_points,
+                        int* d_knn_indices, float* d_knn_sqr_distances,
+                        float* log_forest, void* stream);
 
 /* Bucket K-NN over a given partition, device pointers.  Bucket b holds
  * d_ids[start_b .. start_b + d_sizes[b]) with start_b = d_starts ? d_starts[b]

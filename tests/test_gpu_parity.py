@@ -405,3 +405,112 @@ def test_rows_come_back_sorted_and_unsorted_input_is_accepted(gpu, orc, rng):
     gi2, gd2 = gi.copy(), gd.copy()
     gpu.explore(X, K, gi2, gd2, 1)
     assert (np.diff(gd2, axis=1) >= 0).all()                       # every row ascending after a full pass
+
+
+# ---------------------------------------------------------------------------
+# query-set search
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("N,NQ,D,MIN,MAX,dist", [
+    (6000, 2500, 24, 9, 18, "normal"),
+    (5000, 1, 130, 33, 66, "normal"),
+    (3000, 777, 3, 5, 11, "grid"),           # many points on a hyperplane and duplicated points
+    (20000, 4000, 64, 33, 66, "uniform"),
+])
+def test_queries_reach_the_leaf_the_oracle_routes_them_to(gpu, orc, rng, N, NQ, D, MIN, MAX, dist):
+    """One tree and a row longer than any bucket: the row of a query is then exactly the bucket it was routed to."""
+    import gpu_rsfk
+    if dist == "grid":
+        X = rng.integers(0, 6, (N, D)).astype(np.float32)
+        Q = rng.integers(0, 6, (NQ, D)).astype(np.float32)
+    elif dist == "uniform":
+        X = rng.random((N, D), dtype=np.float32)
+        Q = X[rng.permutation(N)[:NQ]].copy()           # queries that are base points: always on their own side
+        Q[::2] += rng.standard_normal((len(Q[::2]), D)).astype(np.float32) * 0.01
+    else:
+        X = rng.standard_normal((N, D)).astype(np.float32)
+        Q = rng.standard_normal((NQ, D)).astype(np.float32)
+    perm, qs, qz = orc.route_queries(X, Q, MIN, MAX, 5000, 5)
+    K = max(MAX, int(qz.max()))              # identical points cannot be split: such buckets stay above MAX
+    assert (qz >= 1).all() and K <= 256
+    r = gpu_rsfk.RSFK(random_state=5)
+    _say("route", N, NQ, D, MIN, MAX, dist, K)
+    gi, gd = r.find_nearest_neighbors_ann(X, Q, K, n_trees=1, min_tree_children=MIN, max_tree_children=MAX,
+                                          ensure_valid_indices=False)
+    for q in range(NQ):
+        want = np.sort(perm[qs[q]:qs[q] + qz[q]])
+        got = np.sort(gi[q][gi[q] >= 0])
+        assert np.array_equal(got, want), (q, got, want)
+    fin = gi >= 0
+    assert np.isinf(gd[~fin]).all()
+    d64 = ((X[gi[fin]].astype(np.float64) - np.repeat(Q, fin.sum(1), axis=0)) ** 2).sum(1)
+    assert np.allclose(gd[fin], d64, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("N,NQ,D,K,T,kw", [
+    (20000, 3000, 100, 32, 5, {}),
+    (8000, 1500, 18, 8, 3, dict(min_tree_children=4, max_tree_children=9)),    # second call with K+1 .. 3(K+1)
+    (9000, 500, 50, 100, 3, {}),
+    (7000, 2000, 33, 200, 2, dict(min_tree_children=40, max_tree_children=90, ensure_valid_indices=False)),
+    (300, 50, 7, 5, 4, {}),
+])
+def test_find_nearest_neighbors_ann_matches_oracle(gpu, orc, rng, N, NQ, D, K, T, kw):
+    import gpu_rsfk
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    Q = rng.standard_normal((NQ, D)).astype(np.float32)
+    r = gpu_rsfk.RSFK(random_state=23)
+    _say("ann", N, NQ, D, K, T, kw)
+    gi, gd = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T, **kw)
+    mn = kw.get("min_tree_children", K + 1)
+    mx = kw.get("max_tree_children", 2 * mn)
+    oi, od = orc.ann_forest(X, Q, K, T, mn, mx, 5000, 23)
+    if kw.get("ensure_valid_indices", True) and mn < K + 1:
+        orc.ann_forest(X, Q, K, 1, K + 1, 3 * (K + 1), 5000, 23, q_idx=oi, q_dist=od)
+    assert gi.shape == (NQ, K) and gi.dtype == np.int32 and gd.dtype == np.float32
+    assert_knn_equal(gi, gd, oi, od)
+    assert rows_have_no_duplicates(gi)
+    assert r._last_search_time > 0
+
+
+def test_ann_device_entry_point_merges_into_given_rows(gpu, capi, orc, rng):
+    """Device-resident call, twice with different seeds on the same rows == the oracle doing the same."""
+    import torch
+    N, NQ, D, K = 12000, 2048, 40, 16
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    Q = rng.standard_normal((NQ, D)).astype(np.float32)
+    dX, dQ = torch.from_numpy(X).cuda(), torch.from_numpy(Q).cuda()
+    idx = torch.full((NQ, K), -1, dtype=torch.int32, device="cuda")
+    dist = torch.full((NQ, K), float("inf"), dtype=torch.float32, device="cuda")
+    log = np.zeros(16 * 3 + 2, np.float32)
+    _say("ann device", N, NQ, D, K)
+    capi.knn_ann_device(3, K, N, NQ, D, K + 1, 2 * K + 2, 5000, 0, 7, dX.data_ptr(), dQ.data_ptr(),
+                        idx.data_ptr(), dist.data_ptr(), log)
+    capi.knn_ann_device(2, K, N, NQ, D, K + 1, 2 * K + 2, 5000, 0, 100, dX.data_ptr(), dQ.data_ptr(),
+                        idx.data_ptr(), dist.data_ptr())
+    torch.cuda.synchronize()
+    oi, od = orc.ann_forest(X, Q, K, 3, K + 1, 2 * K + 2, 5000, 7)
+    orc.ann_forest(X, Q, K, 2, K + 1, 2 * K + 2, 5000, 100, q_idx=oi, q_dist=od)
+    assert_knn_equal(idx.cpu().numpy(), dist.cpu().numpy(), oi, od)
+    assert (log[9:12] > 0).all() and log[48] > 0          # Total Leaves per tree, total seconds
+    # the recorded index must not change the partition a plain tree build gives
+    perm, ls, lz, st = capi.build_tree(X, K + 1, 2 * K + 2, 5000, 7)
+    operm, ostarts, osizes, ost = orc.build_tree(X, K + 1, 2 * K + 2, 5000, 7)
+    assert np.array_equal(perm, operm) and np.array_equal(lz, osizes) and int(log[9]) == len(osizes)
+    # no queries: nothing to do, nothing touched
+    capi.knn_ann_device(2, K, N, 0, D, K + 1, 2 * K + 2, 5000, 0, 1, dX.data_ptr(), dQ.data_ptr(),
+                        idx.data_ptr(), dist.data_ptr())
+
+
+def test_ann_recall_rises_with_the_number_of_trees(gpu, rng):
+    import gpu_rsfk
+    N, NQ, D, K = 30000, 2000, 16, 10
+    X = rng.random((N, D), dtype=np.float32)
+    Q = rng.random((NQ, D), dtype=np.float32)
+    d2 = (Q ** 2).sum(1)[:, None] - 2.0 * Q @ X.T + (X ** 2).sum(1)[None, :]
+    true = np.argsort(d2, axis=1)[:, :K]
+    r = gpu_rsfk.RSFK(random_state=1)
+    rec = []
+    for T in (1, 8, 40):
+        gi, _ = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T)
+        rec.append(np.mean([len(set(gi[q]) & set(true[q])) / K for q in range(NQ)]))
+    _say("ann recall", rec)
+    assert rec[0] < rec[1] < rec[2] and rec[2] > 0.5

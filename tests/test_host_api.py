@@ -39,6 +39,13 @@ def test_python_layer_signatures_match_the_reference():
     assert (d["n_trees"], d["max_tree_depth"], d["verbose"], d["min_tree_children"], d["max_tree_children"]) == (-1, 5000, 0, -1, -1)
     assert (d["ensure_valid_indices"], d["add_bit_random_motion"], d["random_motion_force"]) == (True, False, 1.0)
     assert (d["nn_exploring_factor"], d["point_in_self_neigh"]) == (-1, True)
+    sig = inspect.signature(gpu_rsfk.RSFK.find_nearest_neighbors_ann)      # reference RSFK.py:371-378
+    assert list(sig.parameters)[1:] == [
+        "points", "query_points", "num_nearest_neighbors", "n_trees", "max_tree_depth", "verbose",
+        "min_tree_children", "max_tree_children", "ensure_valid_indices", "add_bit_random_motion",
+        "random_motion_force", "nn_exploring_factor"]
+    d = {k: v.default for k, v in sig.parameters.items()}
+    assert (d["n_trees"], d["max_tree_depth"], d["verbose"], d["min_tree_children"], d["max_tree_children"]) == (-1, 5000, 0, -1, -1)
     sig = inspect.signature(gpu_rsfk.RSFK.cluster_by_sample_tree)
     assert list(sig.parameters)[1:] == ["points", "max_tree_depth", "verbose", "min_tree_children",
                                         "max_tree_children", "add_bit_random_motion", "random_motion_force",
@@ -63,8 +70,8 @@ def test_argument_errors_are_raised_before_the_library_is_called():
         r.cluster_by_sample_tree(X, min_tree_children=32, max_tree_children=63)
     with pytest.raises(Exception, match="min_tree_children must be at least 1"):
         r.cluster_by_sample_tree(X, min_tree_children=-1, max_tree_children=10)
-    with pytest.raises(NotImplementedError):
-        r.find_nearest_neighbors_ann(X, X, 4)
+    with pytest.raises(Exception, match="max_tree_children must be at least 2\\*min_tree_children"):
+        r.find_nearest_neighbors_ann(X, X, 4, min_tree_children=8, max_tree_children=15)
 
 
 def test_forest_log_decoding():
