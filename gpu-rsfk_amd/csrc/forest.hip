@@ -218,8 +218,12 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
         WsGuard ws;
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
         if (tree_ws_enable_index(ws.w, MIN, MAX_DEPTH)) return 1;
-        DevBuf qs, qz;
-        if (ws_alloc(&qs.p, sizeof(int) * (size_t)NQ) || ws_alloc(&qz.p, sizeof(int) * (size_t)NQ)) return 1;
+        const int rec_cap = tree_ws_rec_cap(ws.w);
+        DevBuf aws;
+        if (ws_alloc(&aws.p, sizeof(int) * ann_ws_ints(NQ, rec_cap))) return 1;
+        if (launch_ann_ws_init(static_cast<int*>(aws.p), NQ, rec_cap, stream)) return 1;
+        DevBuf planes;
+        if (ws_alloc(&planes.p, sizeof(float) * (size_t)rec_cap * (size_t)ann_plane_pitch(D))) return 1;
         std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
         for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
@@ -233,11 +237,9 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
             const double tt = now_s() - tt0;
             for (int j = 0; j < nb && rc == 0; ++j) {
                 (void)hipEventRecord(ev[j].a, stream);
-                rc = launch_route_queries(d_points, d_queries, NQ, D, tree_ws_recs(ws.w, j), tree_ws_rec_cap(ws.w),
-                                          static_cast<int*>(qs.p), static_cast<int*>(qz.p), stream);
-                if (!rc)
-                    rc = launch_ann_knn(d_points, d_queries, NQ, D, K, tree_ws_perm(ws.w, j), static_cast<int*>(qs.p),
-                                        static_cast<int*>(qz.p), d_qidx, d_qdist, stream);
+                rc = launch_ann_tree(d_points, d_queries, NQ, D, K, tree_ws_perm(ws.w, j), tree_ws_recs(ws.w, j),
+                                     tree_ws_n_rec(ws.w, j), rec_cap, stats[5 * j + 0], static_cast<int*>(aws.p),
+                                     static_cast<float*>(planes.p), d_qidx, d_qdist, stream);
                 (void)hipEventRecord(ev[j].b, stream);
             }
             if (rc) break;

@@ -63,18 +63,19 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
 // ann.hip
-int launch_route_queries(const float* points, const float* queries, int NQ, int D, const TreeRec* recs, int n_rec,
-                         int* q_start, int* q_size, hipStream_t stream);
-int launch_ann_knn(const float* points, const float* queries, int NQ, int D, int K, const int* perm, const int* q_start,
-                   const int* q_size, int* q_idx, float* q_dist, hipStream_t stream);
-
-// forest.hip
+size_t ann_ws_ints(int NQ, int rec_cap);
+int ann_plane_pitch(int D);
+int launch_ann_ws_init(int* ws, int NQ, int rec_cap, hipStream_t stream);
+int launch_ann_tree(const float* points, const float* queries, int NQ, int D, int K, const int* perm, const TreeRec* recs,
+                    const int* n_rec_dev, int rec_cap, int n_leaves, int* ws, float* planes, int* q_idx, float* q_dist,
+                    hipStream_t stream);
 int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                           const float* d_points, const float* d_queries, int* d_qidx, float* d_qdist, float* log_forest,
                           hipStream_t stream);
 int knn_ann_forest_host(int n_trees, int K, int N, int NQ, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                         const float* points, const float* queries, int* q_idx, float* q_dist, float* log_forest);
 int tree_ws_rec_cap(const TreeBatchWorkspace* w);
+const int* tree_ws_n_rec(const TreeBatchWorkspace* w, int t);     // device address of the number of records of tree t
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                       int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
                       hipStream_t stream);

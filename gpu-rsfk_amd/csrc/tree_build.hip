@@ -877,8 +877,9 @@ size_t tree_ws_bytes(int N, int D, int MIN, int B)
 int tree_ws_enable_index(TreeBatchWorkspace* w, int MIN, int MAX_DEPTH)
 {
     if (w->recs) return 0;
-    // buckets <= N / MIN + 1, two-child nodes fewer than buckets, plus the one-child nodes of re-draws
-    const size_t cap = (size_t)8 * ((size_t)w->N / (size_t)std::max(MIN, 1) + 2) + 2 * (size_t)std::max(MAX_DEPTH, 0) + 64;
+    // buckets <= N / MIN + 1 and two-child nodes fewer than buckets (one-child nodes leave no record)
+    (void)MAX_DEPTH;
+    const size_t cap = (size_t)2 * ((size_t)w->N / (size_t)std::max(MIN, 1) + 2) + 64;
     RSFK_CHECK(cap < ((size_t)1 << 30), "tree index: too many nodes");
     w->rec_cap = (int)cap;
     if (dmalloc(&w->recs, (size_t)w->B * cap)) return 1;
@@ -887,6 +888,7 @@ int tree_ws_enable_index(TreeBatchWorkspace* w, int MIN, int MAX_DEPTH)
 }
 const TreeRec* tree_ws_recs(const TreeBatchWorkspace* w, int t) { return w->recs + (size_t)t * w->rec_cap; }
 int tree_ws_rec_cap(const TreeBatchWorkspace* w) { return w->rec_cap; }
+const int* tree_ws_n_rec(const TreeBatchWorkspace* w, int t) { return w->n_rec + t; }
 
 int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
 {
