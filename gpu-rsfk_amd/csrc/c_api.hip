@@ -114,6 +114,20 @@ RSFK_API int rsfk_knn_ann_device(int n_trees, int num_neighbors, int N, int NQ, 
                                  static_cast<hipStream_t>(stream));
 }
 
+RSFK_API int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn_sqr_distances, int N, int num_neighbors,
+                                    int drop_self, int* d_indptr, int* d_indices, float* d_data, long long capacity,
+                                    long long* nnz, void* stream)
+{
+    return symmetrize_device(d_knn_indices, d_knn_sqr_distances, N, num_neighbors, drop_self, d_indptr, d_indices, d_data,
+                             capacity, nnz, static_cast<hipStream_t>(stream));
+}
+
+RSFK_API int rsfk_symmetrize_host(const int* knn_indices, const float* knn_sqr_distances, int N, int num_neighbors,
+                                  int drop_self, int* indptr, int* indices, float* data, long long capacity, long long* nnz)
+{
+    return symmetrize_host(knn_indices, knn_sqr_distances, N, num_neighbors, drop_self, indptr, indices, data, capacity, nnz);
+}
+
 RSFK_API int rsfk_bucket_knn_device(const float* d_points, int N, int D, int num_neighbors, const int* d_ids,
                                     const int* d_starts, const int* d_sizes, int n_buckets, int stride,
                                     int* d_knn_indices, float* d_knn_sqr_distances, void* stream)

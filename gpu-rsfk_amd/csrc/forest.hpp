@@ -62,6 +62,12 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
+// graph_export.hip
+int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int drop_self, int* d_indptr, int* d_cols,
+                      float* d_vals, long long cap, long long* nnz, hipStream_t stream);
+int symmetrize_host(const int* idx, const float* dist, int N, int K, int drop_self, int* indptr, int* cols, float* vals,
+                    long long cap, long long* nnz);
+
 // ann.hip
 size_t ann_ws_ints(int NQ, int rec_cap);
 int ann_plane_pitch(int D);

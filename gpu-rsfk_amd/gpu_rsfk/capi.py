@@ -20,6 +20,8 @@ SYMBOLS = {
     "pymodule_cluster_by_sample_tree": (None, [_ci] * 7 + [_vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_forest_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_ann_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp, _vp]),
+    "rsfk_symmetrize_device": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp, _vp]),
+    "rsfk_symmetrize_host": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp]),
     "rsfk_bucket_knn_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _ci, _ci, _vp, _vp, _vp]),
     "rsfk_explore_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
     "rsfk_build_tree_host": (_ci, [_f32, _ci, _ci, _ci, _ci, _ci, _ci, _i32, _i32, _i32, _ci, _i32]),
@@ -111,6 +113,39 @@ def knn_ann_device(n_trees, K, N, NQ, D, min_children, max_children, max_depth, 
     _check(lib().rsfk_knn_ann_device(int(n_trees), int(K), int(N), int(NQ), int(D), int(min_children),
                                      int(max_children), int(max_depth), int(verbose), int(seed),
                                      _vp(d_points), _vp(d_queries), _vp(d_idx), _vp(d_dist), lp, _vp(stream)))
+
+
+def symmetrize(knn_idx, knn_dist=None, drop_self=False):
+    """Symmetrised K-NN graph in CSR form -> indptr (N+1), indices, data; columns ascend inside a row."""
+    knn_idx = np.ascontiguousarray(knn_idx, np.int32)
+    N, K = knn_idx.shape
+    dp = None
+    if knn_dist is not None:
+        knn_dist = np.ascontiguousarray(knn_dist, np.float32)
+        if knn_dist.shape != knn_idx.shape:
+            raise ValueError("knn_dist must have the shape of knn_idx")
+        dp = knn_dist.ctypes.data_as(_vp)
+    indptr = np.empty(N + 1, np.int32)
+    nnz = ctypes.c_longlong(0)
+    _check(lib().rsfk_symmetrize_host(knn_idx.ctypes.data_as(_vp), dp, N, K, int(bool(drop_self)),
+                                      indptr.ctypes.data_as(_vp), None, None, 0, ctypes.byref(nnz)))
+    n = int(nnz.value)
+    cols = np.empty(n, np.int32)
+    vals = np.empty(n, np.float32)
+    if n:
+        _check(lib().rsfk_symmetrize_host(knn_idx.ctypes.data_as(_vp), dp, N, K, int(bool(drop_self)),
+                                          indptr.ctypes.data_as(_vp), cols.ctypes.data_as(_vp),
+                                          vals.ctypes.data_as(_vp), n, ctypes.byref(nnz)))
+    return indptr, cols, vals
+
+
+def symmetrize_device(d_idx, d_dist, N, K, drop_self, d_indptr, d_cols, d_vals, capacity, stream=0):
+    """Device-resident form (integer addresses; d_cols = d_vals = 0 for the count only) -> number of entries."""
+    nnz = ctypes.c_longlong(0)
+    _check(lib().rsfk_symmetrize_device(_vp(d_idx), _vp(d_dist) if d_dist else None, int(N), int(K), int(bool(drop_self)),
+                                        _vp(d_indptr), _vp(d_cols) if d_cols else None, _vp(d_vals) if d_vals else None,
+                                        int(capacity), ctypes.byref(nnz), _vp(stream)))
+    return int(nnz.value)
 
 
 def bucket_knn_device(d_points, N, D, K, d_ids, d_starts, d_sizes, n_buckets, stride, d_idx, d_dist, stream=0):

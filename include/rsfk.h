@@ -107,6 +107,17 @@ int rsfk_bucket_knn_device(const float* d_points, int N, int D, int num_neighbor
 int rsfk_explore_device(const float* d_points, int N, int D, int num_neighbors,
                         int* d_knn_indices, float* d_knn_sqr_distances, int* d_scratch, void* stream);
 
+/* Symmetrised K-NN graph in compressed-row (CSR) form, device pointers: row p holds every neighbour stored for p and
+ * every point that stores p, each once, with the squared distance of the pair; columns ascend inside a row.
+ * d_indptr: N + 1 ints.  d_indices / d_data: room for `capacity` entries (2 * N * num_neighbors always suffices), or both
+ * NULL to obtain d_indptr and *nnz only.  Slots that are negative or >= N are no edges; drop_self != 0 removes p from
+ * its own row; d_knn_sqr_distances may be NULL (data is then zero).  A row must not hold a point twice.  Replaces the
+ * kernels the reference keeps commented out beside its spectral experiment (symmetric_knn_graph_edge_count,
+ * symmetric_knn_graph_offset, symmetric_knn_graph_add_edges, src/rsfk.cu:1229-1299). */
+int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn_sqr_distances, int N, int num_neighbors,
+                           int drop_self, int* d_indptr, int* d_indices, float* d_data, long long capacity,
+                           long long* nnz, void* stream);
+
 /* ---- stage-level calls with host buffers (copies in and out) ------------ */
 
 /* One tree (RSFK::create_bucket_from_sample_tree, src/rsfk.cu:500-1207).
@@ -123,6 +134,10 @@ int rsfk_bucket_knn_host(const float* points, int N, int D, int num_neighbors,
                          const int* ids, int n_ids, const int* starts, const int* sizes,
                          int n_buckets, int stride,
                          int* knn_indices, float* knn_sqr_distances);
+
+/* rsfk_symmetrize_device with host buffers. */
+int rsfk_symmetrize_host(const int* knn_indices, const float* knn_sqr_distances, int N, int num_neighbors,
+                         int drop_self, int* indptr, int* indices, float* data, long long capacity, long long* nnz);
 
 /* `passes` exploration passes with host buffers. */
 int rsfk_explore_host(const float* points, int N, int D, int num_neighbors,

@@ -16,6 +16,7 @@
  *   - forest loop, seed increment, exploration loop   src/rsfk.cu:2033-2183
  *   - query-set search: routing and bucket update     src/rsfk.cu:98-498,
  *                                                     src/kernels/build_tree_update_parents_ann.cu:77-517
+ *   - symmetrised graph in compressed-row form        src/rsfk.cu:1229-1299 (commented out there)
  *
  * Deliberate differences from the reference (none of them is pinned by any
  * fixture in the reference, see the parity notes at the end of this header):
@@ -47,6 +48,8 @@
  *   query-set search          : routing pinned by a pure-Python restatement and by
  *                               "a base point used as a query lands in its own leaf";
  *                               the update by brute force inside the reached leaves
+ *   symmetrised graph         : pinned by scipy.sparse (A.maximum(A.T) of the directed graph) and by a
+ *                               hand-written 5-point case (tests/test_oracle_graph.py)
  *   random draw sequence      : parity unpinned (cuRAND is not available and
  *                               no reference fixture holds a partition)
  */
@@ -554,6 +557,64 @@ RSFK_OR_EXPORT int rsfk_or_ann_forest(int n_trees, int K, int N, int NQ, int D,
     }
     free(perm); free(qs); free(qz);
     return 0;
+}
+
+/*
+ * Symmetrised K-NN graph in compressed-row form (the commented-out kernels symmetric_knn_graph_edge_count /
+ * _offset / _add_edges, src/rsfk.cu:1229-1299): every stored edge p -> c goes into row p; if row c does not store p
+ * the reverse edge goes into row c (line 1243-1249 / 1287-1296: "force the bidirectional edge if it doesn't exist").
+ * Differences: slots that are negative or >= N are skipped (the reference would read out of range), drop_self
+ * removes p from its own row, and the columns of a row are sorted ascending (the reference leaves the arrival order
+ * of atomics).  indptr: N + 1; cols / vals: capacity cap or NULL (count only).  Returns the number of entries, or
+ * -1 when cap is too small.
+ */
+typedef struct { int col; float val; } or_edge;
+static int or_edge_cmp(const void* a, const void* b)
+{
+    int ca = ((const or_edge*)a)->col, cb = ((const or_edge*)b)->col;
+    return (ca > cb) - (ca < cb);
+}
+
+RSFK_OR_EXPORT long long rsfk_or_symmetrize(const int* idx, const float* dist, int N, int K, int drop_self,
+                                            int* indptr, int* cols, float* vals, long long cap)
+{
+    long long* len = (long long*)calloc((size_t)N + 1, sizeof(long long));
+    for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+            long long run = 0;
+            for (int p = 0; p <= N; ++p) { long long l = len[p]; indptr[p] = (int)run; len[p] = run; run += l; }
+            if (!cols) { free(len); return run; }
+            if (run > cap) { free(len); return -1; }
+        }
+        for (int p = 0; p < N; ++p) {
+            for (int k = 0; k < K; ++k) {
+                int c = idx[(size_t)p * K + k];
+                if (c < 0 || c >= N || (drop_self && c == p)) continue;
+                float d = dist ? dist[(size_t)p * K + k] : 0.0f;
+                int mutual = 0;
+                for (int j = 0; j < K; ++j) mutual |= idx[(size_t)c * K + j] == p;
+                if (pass == 0) {
+                    len[p]++;
+                    if (!mutual) len[c]++;
+                } else {
+                    cols[len[p]] = c; vals[len[p]] = d; len[p]++;
+                    if (!mutual) { cols[len[c]] = p; vals[len[c]] = d; len[c]++; }
+                }
+            }
+        }
+    }
+    long long total = indptr[N];
+    or_edge* tmp = (or_edge*)malloc(sizeof(or_edge) * (size_t)(2 * K + 1));
+    size_t tmp_cap = (size_t)(2 * K + 1);
+    for (int p = 0; p < N; ++p) {
+        size_t n = (size_t)(indptr[p + 1] - indptr[p]);
+        if (n > tmp_cap) { tmp_cap = n; tmp = (or_edge*)realloc(tmp, sizeof(or_edge) * tmp_cap); }
+        for (size_t i = 0; i < n; ++i) { tmp[i].col = cols[indptr[p] + i]; tmp[i].val = vals[indptr[p] + i]; }
+        qsort(tmp, n, sizeof(or_edge), or_edge_cmp);
+        for (size_t i = 0; i < n; ++i) { cols[indptr[p] + i] = tmp[i].col; vals[indptr[p] + i] = tmp[i].val; }
+    }
+    free(tmp); free(len);
+    return total;
 }
 
 RSFK_OR_EXPORT void rsfk_or_bruteforce(const float* points, int N, int D, int K,

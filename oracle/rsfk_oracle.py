@@ -19,7 +19,9 @@ _f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
 
 def build(force=False):
     """Compile the oracle with the Makefile next to this file."""
-    if force or not os.path.exists(_SO):
+    src = os.path.join(_HERE, "rsfk_oracle.c")
+    stale = os.path.exists(_SO) and os.path.exists(src) and os.path.getmtime(src) > os.path.getmtime(_SO)
+    if force or stale or not os.path.exists(_SO):
         subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "librsfk_oracle.so"])
     return _SO
 
@@ -64,6 +66,9 @@ def lib():
                                             ctypes.c_int, ctypes.c_int, _f32p, ctypes.c_int, _i32p, _i32p, _i32p]
         L.rsfk_or_ann_forest.restype = ctypes.c_int
         L.rsfk_or_ann_forest.argtypes = [ctypes.c_int] * 9 + [_f32p, _f32p, _i32p, _f32p]
+        L.rsfk_or_symmetrize.restype = ctypes.c_longlong
+        L.rsfk_or_symmetrize.argtypes = [_i32p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, _i32p,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong]
         L.rsfk_or_bruteforce.restype = None
         L.rsfk_or_bruteforce.argtypes = [_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                          ctypes.c_int, _i32p, _f64p]
@@ -213,6 +218,25 @@ def ann_forest(points, queries, K, n_trees, min_children=-1, max_children=-1, ma
     if rc != 0:
         raise RuntimeError("oracle query search failed")
     return q_idx, q_dist
+
+
+def symmetrize(knn_idx, knn_dist=None, drop_self=False):
+    """Symmetrised graph in CSR form -> indptr (N+1), indices, data (columns ascending inside a row)."""
+    knn_idx = np.ascontiguousarray(knn_idx, np.int32)
+    N, K = knn_idx.shape
+    dp = None
+    if knn_dist is not None:
+        knn_dist = np.ascontiguousarray(knn_dist, np.float32)
+        dp = knn_dist.ctypes.data_as(ctypes.c_void_p)
+    indptr = np.empty(N + 1, np.int32)
+    nnz = lib().rsfk_or_symmetrize(knn_idx, dp, N, K, int(bool(drop_self)), indptr, None, None, 0)
+    cols = np.empty(max(nnz, 1), np.int32)
+    vals = np.empty(max(nnz, 1), np.float32)
+    got = lib().rsfk_or_symmetrize(knn_idx, dp, N, K, int(bool(drop_self)), indptr,
+                                   cols.ctypes.data_as(ctypes.c_void_p), vals.ctypes.data_as(ctypes.c_void_p), nnz)
+    if got != nnz:
+        raise RuntimeError("oracle symmetrize failed")
+    return indptr, cols[:nnz], vals[:nnz]
 
 
 def bruteforce(points, K, queries=None):

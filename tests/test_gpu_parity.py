@@ -514,3 +514,55 @@ def test_ann_recall_rises_with_the_number_of_trees(gpu, rng):
         rec.append(np.mean([len(set(gi[q]) & set(true[q])) / K for q in range(NQ)]))
     _say("ann recall", rec)
     assert rec[0] < rec[1] < rec[2] and rec[2] > 0.5
+
+
+# ---------------------------------------------------------------------------
+# symmetrised graph export
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("N,K,drop_self", [(5000, 16, True), (3000, 100, False), (2000, 200, True), (1, 3, False),
+                                           (700, 1, True)])
+def test_symmetric_graph_matches_oracle(gpu, orc, rng, N, K, drop_self):
+    import gpu_rsfk
+    idx = np.stack([rng.permutation(max(N, K + 1))[:K] for _ in range(N)]).astype(np.int32)
+    idx[idx >= N] = -1                                           # only when N <= K: empty slots
+    idx[:, 0] = np.arange(N)                                     # the point itself first, as the forest stores it
+    for p in range(N):
+        dup = np.flatnonzero(idx[p, 1:] == p) + 1
+        idx[p, dup] = -1
+    idx[rng.random((N, K)) < 0.02] = -1
+    val = rng.random((N, K)).astype(np.float32)
+    _say("symmetrize", N, K, drop_self)
+    gp, gc, gv = gpu_rsfk.symmetric_knn_graph(idx, val, drop_self=drop_self)
+    op, oc, ov = orc.symmetrize(idx, val, drop_self=drop_self)
+    assert np.array_equal(gp, op) and np.array_equal(gc, oc)
+    assert np.array_equal(gv, ov)          # a stored edge keeps its own value, an added one the value of its source
+    gp2, gc2, gv2 = gpu_rsfk.symmetric_knn_graph(idx, None, drop_self=drop_self)
+    assert np.array_equal(gp2, op) and np.array_equal(gc2, oc) and (gv2 == 0).all()
+
+
+def test_symmetric_graph_of_a_built_graph(gpu, capi, orc, rng):
+    """On a graph the library built (one distance value per pair) the export equals the oracle's bit for bit; device
+    entry point with the two-call protocol (count, then fill)."""
+    import torch
+    import gpu_rsfk
+    N, D, K = 30000, 20, 12
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    gi, gd = gpu_rsfk.RSFK(random_state=2).find_nearest_neighbors(X, K, n_trees=6)
+    op, oc, ov = orc.symmetrize(gi, gd, drop_self=True)
+    di, dd = torch.from_numpy(gi).cuda(), torch.from_numpy(gd).cuda()
+    indptr = torch.empty(N + 1, dtype=torch.int32, device="cuda")
+    _say("symmetrize device", N, K)
+    nnz = capi.symmetrize_device(di.data_ptr(), dd.data_ptr(), N, K, True, indptr.data_ptr(), 0, 0, 0)
+    assert nnz == len(oc) and N * (K - 1) <= nnz <= 2 * N * (K - 1)
+    cols = torch.empty(nnz, dtype=torch.int32, device="cuda")
+    vals = torch.empty(nnz, dtype=torch.float32, device="cuda")
+    assert capi.symmetrize_device(di.data_ptr(), dd.data_ptr(), N, K, True, indptr.data_ptr(), cols.data_ptr(),
+                                  vals.data_ptr(), nnz) == nnz
+    torch.cuda.synchronize()
+    assert np.array_equal(indptr.cpu().numpy(), op) and np.array_equal(cols.cpu().numpy(), oc)
+    assert np.array_equal(vals.cpu().numpy(), ov)
+    with pytest.raises(RuntimeError, match="too small"):
+        capi.symmetrize_device(di.data_ptr(), dd.data_ptr(), N, K, True, indptr.data_ptr(), cols.data_ptr(),
+                               vals.data_ptr(), nnz - 1)
+    S = gpu_rsfk.symmetric_knn_graph(gi, gd, as_scipy=True)
+    assert S.shape == (N, N) and (abs(S - S.T)).nnz == 0 and S.diagonal().sum() == 0
