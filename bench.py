@@ -63,6 +63,143 @@ def exact_knn_sample(torch, dX, queries, K, chunk=65536):
     return best_i
 
 
+def _base(metric, value, unit, args, sec_per_step, workload):
+    return {"metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 3), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic", "config": {"workload": workload}}
+
+
+def bench_ann(args):
+    """Query-set search: a step = n_trees trees built on the points, every query routed and merged per tree."""
+    import torch
+    from gpu_rsfk import capi
+    from gpu_rsfk.RSFK import ForestLog
+    if not torch.cuda.is_available() or capi.lib().rsfk_device_count() < 1:
+        raise SystemExit("bench.py: no GPU visible")
+    N, D, K, T = args.n, args.d, args.k, args.trees
+    NQ = N if args.queries < 0 else args.queries
+    mn = K + 1 if args.min_children < 0 else args.min_children
+    mx = 2 * mn if args.max_children < 0 else args.max_children
+    both = make_points(N + NQ, D, args.workload)           # points and queries from one distribution
+    X, Q = np.ascontiguousarray(both[:N]), np.ascontiguousarray(both[N:])
+    del both
+    dX, dQ = torch.from_numpy(X).cuda(), torch.from_numpy(Q).cuda()
+    idx = torch.empty((NQ, K), dtype=torch.int32, device="cuda")
+    dist = torch.empty((NQ, K), dtype=torch.float32, device="cuda")
+    logs = []
+
+    def step(keep):
+        idx.fill_(-1)
+        dist.fill_(float("inf"))
+        log = np.zeros(16 * T + 2, np.float32)
+        capi.knn_ann_device(T, K, N, NQ, D, mn, mx, 5000, 0, 0, dX.data_ptr(), dQ.data_ptr(), idx.data_ptr(),
+                            dist.data_ptr(), log)
+        if keep:
+            logs.append(log)
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / max(args.steps, 1)
+
+    nq = min(args.recall_queries, NQ)
+    sel = torch.from_numpy(np.random.default_rng(1).choice(NQ, nq, replace=False)).cuda()
+    best_d = torch.full((nq, K), float("inf"), device="cuda", dtype=torch.float64)
+    best_i = torch.full((nq, K), -1, device="cuda", dtype=torch.int64)
+    q64 = dQ[sel].double()
+    for a in range(0, N, 65536):
+        xs = dX[a:a + 65536].double()
+        dd = torch.cat([best_d, torch.cdist(q64, xs) ** 2], 1)
+        ii = torch.cat([best_i, torch.arange(a, a + xs.shape[0], device="cuda").expand(nq, -1)], 1)
+        best_d, o = torch.topk(dd, K, dim=1, largest=False)
+        best_i = torch.gather(ii, 1, o)
+    hits = (idx[sel].long()[:, :, None] == best_i[:, None, :]).any(2).sum().item()
+
+    upd_s = float(np.mean([np.mean(ForestLog(l).data["KNN Sets Updates"]) for l in logs])) if logs and T > 0 else 0.0
+    alg_bytes = float(N) * 4 * D + float(NQ) * (4 * D + 16 * K)
+    achieved = alg_bytes / upd_s / 1e9 if upd_s > 0 else 0.0
+    cpu = None
+    if args.cpu_sample > 0:
+        from oracle import rsfk_oracle as orc
+        ns, nqs = min(args.cpu_sample, N), min(args.cpu_sample, NQ)
+        c0 = time.perf_counter()
+        orc.ann_forest(np.ascontiguousarray(X[:ns]), np.ascontiguousarray(Q[:nqs]), K, T, mn, mx, 5000, 0)
+        cs = time.perf_counter() - c0
+        cpu = {"value": round(nqs / cs, 1), "unit": "queries/s", "cores": orc.num_threads(), "kind": "port",
+               "seconds": round(cs, 3),
+               "sample": "first %d points and first %d queries of the same workload, same D, K, %d trees, OpenMP" % (ns, nqs, T)}
+    out = _base("ann_queries_per_sec", NQ / sec, "queries/s", args, sec,
+                "%s N=%d NQ=%d D=%d K=%d n_trees=%d buckets=%d..%d seed=0" % (args.workload, N, NQ, D, K, T, mn, mx))
+    out.update({"recall_at_k": round(hits / float(nq * K), 4), "recall_queries": nq,
+                "roofline": {"kernel": "per-tree query update (k_planes, k_route, scan, k_ann_fill, k_ann_leaf)", "bound": "hbm",
+                             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                             "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(upd_s * 1e3, 4),
+                             "launches_per_step": T},
+                "cpu_baseline": cpu})
+    print(json.dumps(out))
+
+
+def bench_graph(args):
+    """CSR export: a step = one full rsfk_symmetrize_device call on a graph built beforehand."""
+    import torch
+    from gpu_rsfk import capi
+    if not torch.cuda.is_available() or capi.lib().rsfk_device_count() < 1:
+        raise SystemExit("bench.py: no GPU visible")
+    N, D, K, T = args.n, args.d, args.k, args.trees
+    mn = K + 1 if args.min_children < 0 else args.min_children
+    mx = 2 * mn if args.max_children < 0 else args.max_children
+    X = make_points(N, D, args.workload)
+    dX = torch.from_numpy(X).cuda()
+    idx = torch.full((N, K), -1, dtype=torch.int32, device="cuda")
+    idx[:, 0] = torch.arange(N, dtype=torch.int32, device="cuda")
+    dist = torch.full((N, K), float("inf"), dtype=torch.float32, device="cuda")
+    dist[:, 0] = 0.0
+    capi.knn_forest_device(T, K, N, D, mn, mx, 5000, 0, 0, args.explore, dX.data_ptr(), idx.data_ptr(), dist.data_ptr())
+    indptr = torch.empty(N + 1, dtype=torch.int32, device="cuda")
+    nnz = capi.symmetrize_device(idx.data_ptr(), dist.data_ptr(), N, K, True, indptr.data_ptr(), 0, 0, 0)
+    cols = torch.empty(nnz, dtype=torch.int32, device="cuda")
+    vals = torch.empty(nnz, dtype=torch.float32, device="cuda")
+
+    def step():
+        capi.symmetrize_device(idx.data_ptr(), dist.data_ptr(), N, K, True, indptr.data_ptr(), cols.data_ptr(),
+                               vals.data_ptr(), nnz)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / max(args.steps, 1)
+    cpu = None
+    if args.cpu_sample > 0:
+        from oracle import rsfk_oracle as orc
+        hi, hd = idx.cpu().numpy(), dist.cpu().numpy()
+        c0 = time.perf_counter()
+        op, oc, ov = orc.symmetrize(hi, hd, drop_self=True)
+        cs = time.perf_counter() - c0
+        same = bool(np.array_equal(op, indptr.cpu().numpy()) and np.array_equal(oc, cols.cpu().numpy()) and
+                    np.array_equal(ov, vals.cpu().numpy()))
+        cpu = {"value": round(len(oc) / cs, 1), "unit": "edges/s", "cores": 1, "kind": "port", "seconds": round(cs, 3),
+               "sample": "the same graph, whole", "identical_to_gpu_result": same}
+    alg_bytes = float(N) * K * 8 + float(nnz) * 8 + (N + 1) * 4.0
+    out = _base("graph_export_edges_per_sec", nnz / sec, "edges/s", args, sec,
+                "%s N=%d D=%d K=%d n_trees=%d exploration=%d: symmetrised CSR without self edges, %d entries" % (
+                    args.workload, N, D, K, T, args.explore, nnz))
+    out.update({"roofline": {"kernel": "whole export (k_sym_flags, scan, k_sym_fill, segmented sort)", "bound": "hbm",
+                             "achieved": round(alg_bytes / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(alg_bytes / sec / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                             "algorithmic_bytes_per_launch": alg_bytes},
+                "cpu_baseline": cpu})
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -78,9 +215,16 @@ def main():
     ap.add_argument("--workload", default="uniform", choices=["uniform", "normal", "gmm64", "sparse"])
     ap.add_argument("--recall-queries", type=int, default=10000)
     ap.add_argument("--cpu-sample", type=int, default=200000, help="rows of the workload the CPU baseline runs on (0 = skip)")
+    ap.add_argument("--path", default="knng", choices=["knng", "ann", "graph"],
+                    help="knng = K-NN-graph build (the headline metric); ann = query-set search; graph = CSR export")
+    ap.add_argument("--queries", type=int, default=-1, help="query points of --path ann (default: as many as points)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU only (--gpus 1); nothing here uses a second GPU")
+    if args.path == "ann":
+        return bench_ann(args)
+    if args.path == "graph":
+        return bench_graph(args)
 
     import torch
     from gpu_rsfk import capi
