@@ -612,8 +612,9 @@ constexpr int kMaxGroup = 16;        // nodes of one level of a subtree worked o
 // fewer, G) at a time -- their hyperplanes are made together (one wavefront each), all their points are tested in
 // one sweep, and each node is partitioned by one wavefront -- so the number of dependent trips to memory per
 // subtree is a few per level instead of a few per node.
+template <bool Q8>
 __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ points,
-                                                 const uint16_t* __restrict__ pb16, TreeParams P,
+                                                 const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8, TreeParams P,
                                                  const int* __restrict__ perm0, const int* __restrict__ perm1,
                                                  int* __restrict__ perm_out,
                                                  const TreeNode* __restrict__ tasks, int n_tasks, int node_cap, int G,
@@ -727,7 +728,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                     h1[u] = hp_s[jj[u]][1];
                     h2[u] = hp_s[jj[u]][2];
                 }
-                side_screen8<kTailBatch, false>(nvec, Dv, jj, bb, h1, h2, pb16, nullptr, id, P.D, P.band, valid, right, redo);
+                side_screen8<kTailBatch, Q8>(nvec, Dv, jj, bb, h1, h2, pb16, q8, id, P.D, P.band, valid, right, redo);
 #pragma unroll
                 for (int u = 0; u < kTailBatch; ++u) {
                     if (valid[u] && sub8 == 0) {
@@ -993,10 +994,20 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         const size_t lds = (size_t)(2 * P.small) * 4 + (size_t)G * nvec_len(D) * 4 + (size_t)node_cap * sizeof(int2) +
                            2 * (size_t)node_cap * sizeof(SmallNode) + (size_t)P.small;
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
-        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k_tail, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, P, w->perm[0], w->perm[1], w->perm[0],
-                           w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr, w->recs, w->n_rec,
-                           w->rec_cap);
+        const bool tail_q8 = q8 != nullptr && std::getenv("RSFK_TAIL_BF16") == nullptr;
+        if (tail_q8) {
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds));
+            hipLaunchKernelGGL(k_tail<true>, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, q8, P, w->perm[0], w->perm[1],
+                               w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr,
+                               w->recs, w->n_rec, w->rec_cap);
+        } else {
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds));
+            hipLaunchKernelGGL(k_tail<false>, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, q8, P, w->perm[0], w->perm[1],
+                               w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr,
+                               w->recs, w->n_rec, w->rec_cap);
+        }
         RSFK_HIP(hipGetLastError());
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
