@@ -66,22 +66,37 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
 {
     const int lane = lane_id();
     const int Dn = nvec_len(D);
-    for (int d = lane; d < Dn; d += 64) nvec[d] = d < D ? x1[d] - x2[d] : 0.0f;
+    const int hl = lane & 31;
+    const bool lowh = lane < 32;
+    // Both halves of the wavefront walk the dimensions hl, hl + 32, ... (the loads of eight steps are requested
+    // together): the lower half forms the offset with the arithmetic of create_node.cu:122-135 and writes the normal,
+    // the upper half the 1-norm and the sum of the components.
     float s = 0.0f, s2 = 0.0f;
-    if (lane < 32) {
-        for (int d = lane; d < D; d += 32) {
-            const float t1 = x1[d], t2 = x2[d];
-            const float nd = t1 - t2;
-            const float prod = nd * (t1 + t2);
-            s = s + prod * 0.5f;
+    for (int d0 = hl; d0 < D; d0 += 256) {
+        float t1[8], t2[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int d = d0 + 32 * k;
+            t1[k] = d < D ? x1[d] : 0.0f;
+            t2[k] = d < D ? x2[d] : 0.0f;
         }
-    } else {
-        for (int d = lane - 32; d < D; d += 32) {
-            const float nd = x1[d] - x2[d];
-            s += fabsf(nd);
-            s2 += nd;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int d = d0 + 32 * k;
+            if (d < D) {
+                const float nd = t1[k] - t2[k];
+                if (lowh) {
+                    nvec[d] = nd;
+                    const float prod = nd * (t1[k] + t2[k]);
+                    s = s + prod * 0.5f;
+                } else {
+                    s += fabsf(nd);
+                    s2 += nd;
+                }
+            }
         }
     }
+    for (int d = D + lane; d < Dn; d += 64) nvec[d] = 0.0f;
     s = half_butterfly_sum(s);
     s2 = half_butterfly_sum(s2);
     if (lane == 0) hp[0] = s;

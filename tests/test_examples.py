@@ -69,8 +69,8 @@ def test_sweep_quality_rises_with_trees_and_exploration(gpu, tmp_path):
     for r in res:
         q = r["quality_list"]
         assert q[0] < q[1] < q[2] <= 1.0 and all(t > 0 for t in r["time_list"])
-    assert all(a <= b for a, b in zip(res[0]["quality_list"], res[1]["quality_list"]))     # one tree: nothing new to explore
-    assert res[0]["quality_list"][-1] < res[1]["quality_list"][-1]
+    # (with one tree there is nothing new to explore; every call perturbs the data afresh, so that pair is noise)
+    assert all(a < b for a, b in zip(res[0]["quality_list"][1:], res[1]["quality_list"][1:]))
     assert res[1]["quality_list"][-1] > 0.9
     assert json.load(open(tmp_path / "sweep.json"))[0]["parameter_list"] == [1, 4, 12]
     args = knn_experiment1.build_parser().parse_args(
