@@ -428,6 +428,33 @@ __global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, i
     chunk2node[c] = lo;
 }
 
+// Hyperplanes of the nodes of a wide level, one wavefront per node: record ni of the table is
+// [offset, bound of the 1-norm, sum of the components, 0 | normal, nvec_len(D) floats].  The workgroups of a node
+// (one per chunk, up to a thousand at the first levels) fetch the record instead of each making the hyperplane again.
+__global__ __launch_bounds__(256) void k_level_planes(const float* __restrict__ points, TreeParams P,
+                                                      const int* __restrict__ perm0, const int* __restrict__ perm1,
+                                                      const TreeNode* __restrict__ nodes, int n_nodes,
+                                                      float* __restrict__ table)
+{
+    extern __shared__ __align__(16) float lds_p[];          // per wavefront: 4 + nvec_len(D) floats
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int ni = blockIdx.x * 4 + wave;
+    if (ni >= n_nodes) return;
+    const int rec = 4 + nvec_len(P.D);
+    float* mine = lds_p + (size_t)wave * rec;
+    const TreeNode nd = nodes[ni];
+    const int* perm = (nd.buf ? perm1 : perm0) + (size_t)nd.tree * (size_t)P.N;
+    int r1, r2;
+    pick_pair(nd.key, nd.dcount, r1, r2);
+    const int p1 = perm[nd.dstart + r1] & kIdMask;
+    const int p2 = perm[nd.dstart + r2] & kIdMask;
+    if (lane == 0) mine[3] = 0.0f;
+    make_hyperplane_wave(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, mine + 4, mine);
+    wave_lds_sync();
+    float* out = table + (size_t)ni * rec;
+    for (int i = lane; i < rec; i += 64) out[i] = mine[i];
+}
+
 // Side test of one chunk of one node: sets bit 31 of the permutation entry of
 // every member on the right side and counts the members on the left.
 template <bool Q8>
@@ -436,10 +463,12 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
                                                  TreeParams P,
                                                  int* __restrict__ perm0, int* __restrict__ perm1,
                                                  const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
-                                                 const int* __restrict__ chunk2node, int* __restrict__ chunk_left)
+                                                 const int* __restrict__ chunk2node, int* __restrict__ chunk_left,
+                                                 const float* __restrict__ planes)
 {
-    extern __shared__ __align__(16) float nvec[];          // nvec_len(D) floats
-    __shared__ float hp_s[3];                               // offset, bound of the 1-norm, sum of the components
+    extern __shared__ __align__(16) float side_lds[];      // record of the node's hyperplane (k_level_planes)
+    float* hp_s = side_lds;                                 // offset, bound of the 1-norm, sum of the components
+    float* nvec = side_lds + 4;                             // nvec_len(D) floats
     __shared__ int left_s, n_def_s;
     __shared__ int deferred[1024];                          // points of the chunk left to the exact test (chunk <= 1024)
     const int c = blockIdx.x;
@@ -447,14 +476,12 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     const TreeNode nd = nodes[ni];
     const int k = c - chunk_base[ni];
     int* perm = (nd.buf ? perm1 : perm0) + (size_t)nd.tree * (size_t)P.N;
-    int r1, r2;
-    pick_pair(nd.key, nd.dcount, r1, r2);
-    const int p1 = perm[nd.dstart + r1] & kIdMask;
-    const int p2 = perm[nd.dstart + r2] & kIdMask;
     if (threadIdx.x == 0) { left_s = 0; n_def_s = 0; }
-    // p1/p2 must be read by every workgroup of the node before any of them sets
-    // side bits; masking with kIdMask makes the read independent of that order.
-    if (threadIdx.x < 64) make_hyperplane_wave(points + (size_t)p1 * P.D, points + (size_t)p2 * P.D, P.D, nvec, hp_s);
+    {
+        const int rec4 = (4 + nvec_len(P.D)) >> 2;          // 16-byte pieces of the record
+        const float4* src = reinterpret_cast<const float4*>(planes + (size_t)ni * (size_t)(4 * rec4));
+        for (int i = threadIdx.x; i < rec4; i += kBlock) reinterpret_cast<float4*>(side_lds)[i] = src[i];
+    }
     __syncthreads();
     const float b = hp_s[0], n1 = hp_s[1], sn = hp_s[2];
     const int pos0 = nd.start + k * P.chunk;
@@ -845,6 +872,7 @@ struct TreeBatchWorkspace {
     int* chunk_base = nullptr;
     int* chunk2node = nullptr;
     int* chunk_left = nullptr;
+    float* planes = nullptr;             // hyperplanes of the nodes of the current wide level: node_cap x (4 + nvec_len(D))
     int* leaf_start = nullptr;
     int* leaf_size = nullptr;
     TreeStats* stats = nullptr;
@@ -861,7 +889,7 @@ struct TreeBatchWorkspace {
 static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
-                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec};
+                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec, w.planes};
     for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
@@ -886,7 +914,7 @@ int tree_small_threshold() { return 1024; }
 size_t tree_ws_bytes(int N, int D, int MIN, int B)
 {
     const size_t lc = (size_t)N / (size_t)std::max(MIN, 1) + 2;
-    return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24));
+    return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24 + (size_t)(4 + nvec_len(D)) * 4));
 }
 
 // From now on every build with this workspace also writes the index of each tree (TreeRec records).
@@ -924,6 +952,7 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     if (dmalloc(&w->chunk_base, (size_t)w->node_cap + 1)) return 1;
     if (dmalloc(&w->chunk2node, (size_t)w->chunk_cap)) return 1;
     if (dmalloc(&w->chunk_left, (size_t)w->chunk_cap)) return 1;
+    if (dmalloc(&w->planes, (size_t)w->node_cap * (size_t)(4 + nvec_len(D)))) return 1;
     if (dmalloc(&w->leaf_start, (size_t)B * w->leaf_cap)) return 1;
     if (dmalloc(&w->leaf_size, (size_t)B * w->leaf_cap)) return 1;
     if (dmalloc(&w->stats, (size_t)B)) return 1;
@@ -968,7 +997,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_HIP(hipGetLastError());
 
     int cur = 0;
-    const size_t side_lds = (size_t)nvec_len(D) * sizeof(float);
+    const size_t side_lds = (size_t)(4 + nvec_len(D)) * sizeof(float);
     // wide levels
     while (true) {
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
@@ -977,6 +1006,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         const int n_nodes = w->h_ctr->n_next;
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
+        hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + 3) / 4)), dim3(256), 4 * side_lds, stream, points, P,
+                           w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
         hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], n_nodes, P.chunk, w->chunk_base, w->ctr);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
@@ -987,10 +1018,10 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
         if (q8)
             hipLaunchKernelGGL(k_side<true>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
-                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
+                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes);
         else
             hipLaunchKernelGGL(k_side<false>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
-                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left);
+                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes);
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
                            w->recs, w->n_rec, w->rec_cap);
