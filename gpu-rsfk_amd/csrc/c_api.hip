@@ -114,6 +114,16 @@ RSFK_API int rsfk_knn_ann_device(int n_trees, int num_neighbors, int N, int NQ, 
                                  static_cast<hipStream_t>(stream));
 }
 
+RSFK_API int rsfk_knn_forest_fresh_host(int n_trees, int num_neighbors, int N, int D, int MIN_TREE_CHILD, int MAX_TREE_CHILD,
+                                        int MAX_DEPTH, int VERBOSE, int RANDOM_STATE, int nn_exploring_factor,
+                                        int point_in_self_neigh, const float* points, int* knn_indices,
+                                        float* knn_sqr_distances, float* log_forest)
+{
+    return knn_forest_host(n_trees, num_neighbors, N, D, MIN_TREE_CHILD, MAX_TREE_CHILD, MAX_DEPTH, VERBOSE, RANDOM_STATE,
+                           nn_exploring_factor, points, knn_indices, knn_sqr_distances, log_forest,
+                           point_in_self_neigh ? 2 : 1);
+}
+
 RSFK_API int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn_sqr_distances, int N, int num_neighbors,
                                     int drop_self, int* d_indptr, int* d_indices, float* d_data, long long capacity,
                                     long long* nnz, void* stream)

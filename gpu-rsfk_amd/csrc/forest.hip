@@ -293,8 +293,23 @@ int knn_ann_forest_host(int n_trees, int K, int N, int NQ, int D, int MIN, int M
     return 0;
 }
 
+namespace {
+// rows as the Python layer prepares them (RSFK.py:330-335 of the reference): empty, or the point itself in slot 0
+__global__ __launch_bounds__(256) void k_fresh_rows(int* __restrict__ idx, float* __restrict__ dist, size_t total, int K,
+                                                    int self_in)
+{
+    for (size_t e = blockIdx.x * (size_t)256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+        const bool first = self_in && e % (size_t)K == 0;
+        idx[e] = first ? (int)(e / (size_t)K) : -1;
+        dist[e] = first ? 0.0f : INFINITY;
+    }
+}
+}  // namespace
+
+// fresh_rows: 0 = the rows are in/out (copied to the device first), 1 = they start empty, 2 = they start with the
+// point itself (distance 0) in slot 0; with 1 or 2 the host arrays are only written.
 int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
-                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest)
+                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest, int fresh_rows)
 {
     RSFK_CHECK(N >= 1 && D >= 1 && K >= 1, "forest: N, D and K must be positive");
     DevBuf dp, di, dd;
@@ -303,8 +318,15 @@ int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_
     if (ws_alloc(&di.p, nk * sizeof(int))) return 1;
     if (ws_alloc(&dd.p, nk * sizeof(float))) return 1;
     RSFK_HIP(hipMemcpy(dp.p, points, nd * sizeof(float), hipMemcpyHostToDevice));
-    RSFK_HIP(hipMemcpy(di.p, knn_idx, nk * sizeof(int), hipMemcpyHostToDevice));
-    RSFK_HIP(hipMemcpy(dd.p, knn_dist, nk * sizeof(float), hipMemcpyHostToDevice));
+    if (fresh_rows) {
+        const unsigned grid = (unsigned)std::min<size_t>((nk + 255) / 256, 65536);
+        hipLaunchKernelGGL(k_fresh_rows, dim3(grid), dim3(256), 0, nullptr, static_cast<int*>(di.p), static_cast<float*>(dd.p),
+                           nk, K, fresh_rows == 2 ? 1 : 0);
+        RSFK_HIP(hipGetLastError());
+    } else {
+        RSFK_HIP(hipMemcpy(di.p, knn_idx, nk * sizeof(int), hipMemcpyHostToDevice));
+        RSFK_HIP(hipMemcpy(dd.p, knn_dist, nk * sizeof(float), hipMemcpyHostToDevice));
+    }
     const int rc = knn_forest_device(n_trees, K, N, D, MIN, MAX, MAX_DEPTH, verbose, seed, nnef,
                                      static_cast<const float*>(dp.p), static_cast<int*>(di.p),
                                      static_cast<float*>(dd.p), log_forest, nullptr);

@@ -86,7 +86,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                       int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
                       hipStream_t stream);
 int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
-                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest);
+                    int nnef, const float* points, int* knn_idx, float* knn_dist, float* log_forest, int fresh_rows = 0);
 int build_tree_host(const float* d_points, int N, int D, int MIN, int MAX, int MAX_DEPTH, int seed,
                     std::vector<int>& perm, std::vector<int>& leaf_start, std::vector<int>& leaf_size, int stats[5]);
 

@@ -89,6 +89,11 @@ def load_library():
         ctypes.POINTER(ctypes.c_int),
         ctypes.POINTER(ctypes.c_int),
     ]
+    # entry point of this library only: rows that start empty are made on the device instead of being uploaded
+    if hasattr(lib, 'rsfk_knn_forest_fresh_host'):
+        lib.rsfk_knn_forest_fresh_host.restype = ctypes.c_int
+        lib.rsfk_knn_forest_fresh_host.argtypes = [ctypes.c_int] * 11 + [_f32_2d, _i32_2d_w, _f32_2d_w, _f32_1d_w]
+        lib.rsfk_last_error.restype = ctypes.c_char_p
     return lib
 
 
@@ -164,19 +169,33 @@ class RSFK(object):
             random_motion(points, random_motion_force)
         points = np.require(points, np.float32, ['CONTIGUOUS', 'ALIGNED'])
 
-        knn_indices = np.full((N, K), -1, dtype=np.int32)
-        knn_squared_dist = np.full((N, K), np.inf, dtype=np.float32)
-        if point_in_self_neigh:
-            knn_indices[:, 0] = np.arange(N, dtype=np.int32)
-            knn_squared_dist[:, 0] = 0.0
+        fresh = hasattr(self._lib, 'rsfk_knn_forest_fresh_host')
+        if fresh:
+            # the library makes the initial rows (empty, or the point itself in slot 0) on the device
+            knn_indices = np.empty((N, K), dtype=np.int32)
+            knn_squared_dist = np.empty((N, K), dtype=np.float32)
+        else:
+            knn_indices = np.full((N, K), -1, dtype=np.int32)
+            knn_squared_dist = np.full((N, K), np.inf, dtype=np.float32)
+            if point_in_self_neigh:
+                knn_indices[:, 0] = np.arange(N, dtype=np.int32)
+                knn_squared_dist[:, 0] = 0.0
 
         t_init = time.time()
 
         log_forest = np.zeros(n_trees * 16 + 2, dtype=np.float32)
-        self._lib.pymodule_rsfk_knn(
-            n_trees, K, N, D, min_tree_children, max_tree_children, max_tree_depth,
-            verbose, self.random_state, int(nn_exploring_factor),
-            points, knn_indices, knn_squared_dist, log_forest)
+        if fresh:
+            rc = self._lib.rsfk_knn_forest_fresh_host(
+                n_trees, K, N, D, min_tree_children, max_tree_children, max_tree_depth,
+                verbose, self.random_state, int(nn_exploring_factor), int(bool(point_in_self_neigh)),
+                points, knn_indices, knn_squared_dist, log_forest)
+            if rc != 0:
+                raise RuntimeError(self._lib.rsfk_last_error().decode('utf-8', 'replace'))
+        else:
+            self._lib.pymodule_rsfk_knn(
+                n_trees, K, N, D, min_tree_children, max_tree_children, max_tree_depth,
+                verbose, self.random_state, int(nn_exploring_factor),
+                points, knn_indices, knn_squared_dist, log_forest)
         self.log_forest = ForestLog(log_forest)
 
         if ensure_valid_indices and min_tree_children < K + 1:

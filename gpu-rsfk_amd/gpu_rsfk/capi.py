@@ -20,6 +20,7 @@ SYMBOLS = {
     "pymodule_cluster_by_sample_tree": (None, [_ci] * 7 + [_vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_forest_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_ann_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp, _vp]),
+    "rsfk_knn_forest_fresh_host": (_ci, [_ci] * 11 + [_vp, _vp, _vp, _vp]),
     "rsfk_symmetrize_device": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp, _vp]),
     "rsfk_symmetrize_host": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp]),
     "rsfk_bucket_knn_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _ci, _ci, _vp, _vp, _vp]),

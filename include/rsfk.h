@@ -135,6 +135,15 @@ int rsfk_bucket_knn_host(const float* points, int N, int D, int num_neighbors,
                          int n_buckets, int stride,
                          int* knn_indices, float* knn_sqr_distances);
 
+/* pymodule_rsfk_knn for rows that start empty (point_in_self_neigh = 0) or with the point itself at distance 0 in
+ * slot 0 (!= 0), which is how RSFK.find_nearest_neighbors prepares them (python/gpu_rsfk/RSFK.py:330-335): the rows
+ * are made on the device, knn_indices / knn_sqr_distances are only written, and a third of the bytes of the call
+ * stay off the PCIe bus.  Returns 0, or nonzero with the reason in rsfk_last_error(). */
+int rsfk_knn_forest_fresh_host(int n_trees, int num_neighbors, int N, int D,
+                               int MIN_TREE_CHILD, int MAX_TREE_CHILD, int MAX_DEPTH,
+                               int VERBOSE, int RANDOM_STATE, int nn_exploring_factor, int point_in_self_neigh,
+                               const float* points, int* knn_indices, float* knn_sqr_distances, float* log_forest);
+
 /* rsfk_symmetrize_device with host buffers. */
 int rsfk_symmetrize_host(const int* knn_indices, const float* knn_sqr_distances, int N, int num_neighbors,
                          int drop_self, int* indptr, int* indices, float* data, long long capacity, long long* nnz);

@@ -566,3 +566,24 @@ def test_symmetric_graph_of_a_built_graph(gpu, capi, orc, rng):
                                vals.data_ptr(), nnz - 1)
     S = gpu_rsfk.symmetric_knn_graph(gi, gd, as_scipy=True)
     assert S.shape == (N, N) and (abs(S - S.T)).nnz == 0 and S.diagonal().sum() == 0
+
+
+@pytest.mark.parametrize("self_in", [True, False])
+def test_rows_made_on_the_device_equal_uploaded_rows(gpu, rng, self_in):
+    """find_nearest_neighbors lets the library make the initial rows; the reference's entry point with the rows
+    uploaded must give the same arrays."""
+    import gpu_rsfk
+    N, D, K, T = 9000, 20, 12, 3
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    r = gpu_rsfk.RSFK(random_state=4)
+    _say("fresh rows", self_in)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=T, point_in_self_neigh=self_in)
+    hi = np.full((N, K), -1, np.int32)
+    hd = np.full((N, K), np.inf, np.float32)
+    if self_in:
+        hi[:, 0] = np.arange(N, dtype=np.int32)
+        hd[:, 0] = 0.0
+    log = np.zeros(16 * T + 2, np.float32)
+    r._lib.pymodule_rsfk_knn(T, K, N, D, K + 1, 2 * K + 2, 5000, 0, 4, 1, X, hi, hd, log)
+    assert np.array_equal(gd, hd)
+    assert_knn_equal(gi, gd, hi, hd)
