@@ -217,14 +217,15 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
 // (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  rows_sorted: every K-NN row is
 // known to be sorted by distance.  bf: bfloat16 copy of the points to send the small buckets to the screened kernel
-// (needs sorted rows), else null.
+// (needs sorted rows), else null.  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
+// kinds touch different rows, so the two parts of one tree may run side by side).
 int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream)
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
-    if (n_small > 0) {
+    if (n_small > 0 && part != 2) {
         if (K <= 64 && bf != nullptr && rows_sorted) {
             if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
@@ -234,7 +235,7 @@ int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_so
         }
     }
     // the large ones: 65..72 points to the three-wavefront variant of the small kernel, the rest to the general one
-    if (n_big <= 0) return 0;
+    if (n_big <= 0 || part == 1) return 0;
     const int off = leaf_cap - n_big;
     int skip_upto = 0;
     if (K <= 64) {

@@ -60,6 +60,24 @@ struct DevBuf {
     void* p = nullptr;
     ~DevBuf() { ws_free(p); }
 };
+// second stream (default priority) and the two events that order it against the caller's stream
+struct SideStream {
+    hipStream_t side = nullptr;
+    hipEvent_t start = nullptr, big = nullptr;
+    int open()
+    {
+        RSFK_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
+        RSFK_HIP(hipEventCreateWithFlags(&start, hipEventDisableTiming));
+        RSFK_HIP(hipEventCreateWithFlags(&big, hipEventDisableTiming));
+        return 0;
+    }
+    ~SideStream()
+    {
+        if (side) { (void)hipStreamSynchronize(side); (void)hipStreamDestroy(side); }
+        if (start) (void)hipEventDestroy(start);
+        if (big) (void)hipEventDestroy(big);
+    }
+};
 struct Bf16Guard {
     Bf16Copy c;
     ~Bf16Guard() { bf16_copy_free(&c); }
@@ -130,6 +148,8 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
         for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        SideStream sync;
+        if (std::getenv("RSFK_KNN_ONE_STREAM") == nullptr && sync.open()) return 1;
         int rc = 0;
         for (int t0 = 0; t0 < n_trees && rc == 0; t0 += B) {
             const int nb = std::min(B, n_trees - t0);
@@ -137,13 +157,33 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             rc = build_tree_batch(ws.w, d_points, bf.c.rows, q8_rows, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
             if (rc) break;
             const double tb = now_s() - tb0;
+            // The larger buckets of a tree (a few per cent of the points at the default sizes: a grid too small to fill
+            // the device) run on a second stream beside the small ones: different buckets of one tree touch different
+            // rows.  Both parts of tree j wait for both parts of tree j - 1.
+            bool big_pending = false;                    // sync.big holds the larger buckets of the previous tree
             for (int j = 0; j < nb && rc == 0; ++j) {
+                const int n_big = stats[5 * j + 4], n_small = stats[5 * j] - n_big;
+                const bool split = sync.side != nullptr && n_big > 0 && n_small > 0;
+                if (big_pending) (void)hipStreamWaitEvent(stream, sync.big, 0);
+                if (j > 0) (void)hipEventRecord(ev[j - 1].b, stream);          // both parts of the previous tree are done
                 (void)hipEventRecord(ev[j].a, stream);
+                if (split) {
+                    (void)hipEventRecord(sync.start, stream);                    // everything before this tree
+                    (void)hipStreamWaitEvent(sync.side, sync.start, 0);
+                }
                 rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
-                                            tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w),
-                                            stats[5 * j] - stats[5 * j + 4], stats[5 * j + 4], stats[5 * j + 2], d_idx, d_dist, stream);
-                (void)hipEventRecord(ev[j].b, stream);
+                                            tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
+                                            d_idx, d_dist, stream, split ? 1 : 0);
+                if (!rc && split) {
+                    rc = launch_bucket_knn_tree(d_points, nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                                                tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
+                                                stats[5 * j + 2], d_idx, d_dist, sync.side, 2);
+                    (void)hipEventRecord(sync.big, sync.side);
+                }
+                big_pending = split;
             }
+            if (big_pending) (void)hipStreamWaitEvent(stream, sync.big, 0);
+            if (nb > 0) (void)hipEventRecord(ev[nb - 1].b, stream);
             if (rc) break;
             RSFK_HIP(hipStreamSynchronize(stream));
             for (int j = 0; j < nb; ++j) {

@@ -30,7 +30,7 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 
 int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream);
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0);
 
 // bucket_knn_screen.hip
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);

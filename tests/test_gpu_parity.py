@@ -279,7 +279,7 @@ def test_golden_vectors(gpu):
 # ---------------------------------------------------------------------------
 def test_properties_at_scale(gpu, orc):
     import torch
-    N, D, K, T = 300000, 100, 32, 8
+    N, D, K, T = 1000000, 100, 32, 8             # BASELINE config 2 at its full size
     rng = np.random.default_rng(0)
     X = rng.random((N, D), dtype=np.float32)
     dX = torch.from_numpy(X).cuda()
