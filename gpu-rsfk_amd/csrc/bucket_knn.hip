@@ -41,6 +41,12 @@ struct BucketKnnLds {
     float dist[kTile * kDistPitch];
     int ida[kTile];
     int idb[kTile];
+    // last slot of the rows of the two tiles when the rows are known to be sorted (else +inf), and whether a row got a
+    // candidate below it: a row without one is neither read nor written
+    float tau_a[kTile];
+    float tau_b[kTile];
+    int flag_a[kTile];
+    int flag_b[kTile];
 };
 
 // Stage rows ids[0..rows) x dims [d0, d0+32) into dst (zero filled outside).
@@ -75,7 +81,8 @@ template <int SL>
 __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ points, int D, int K,
                                                      const int* __restrict__ ids, const int* __restrict__ starts,
                                                      const int* __restrict__ sizes, int stride, int skip_upto,
-                                                     int* __restrict__ knn_idx, float* __restrict__ knn_dist)
+                                                     int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                     int rows_sorted)
 {
     __shared__ BucketKnnLds L;
     const int bkt = blockIdx.x;
@@ -96,8 +103,16 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
             const bool diag = (I == J);
             __syncthreads();   // previous tile's LDS fully consumed
             if (tid < kTile) {
-                L.ida[tid] = tid < rows ? bid[I * kTile + tid] : -1;
-                L.idb[tid] = tid < cols ? bid[J * kTile + tid] : -1;
+                const int p = tid < rows ? bid[I * kTile + tid] : -1;
+                L.ida[tid] = p;
+                L.tau_a[tid] = (rows_sorted && p >= 0) ? knn_dist[(size_t)p * (size_t)K + (K - 1)] : INFINITY;
+                L.flag_a[tid] = 0;
+            } else if (tid < 2 * kTile) {
+                const int u = tid - kTile;
+                const int p = u < cols ? bid[J * kTile + u] : -1;
+                L.idb[u] = p;
+                L.tau_b[u] = (rows_sorted && p >= 0) ? knn_dist[(size_t)p * (size_t)K + (K - 1)] : INFINITY;
+                L.flag_b[u] = 0;
             }
             const int nrb = (rows + 15) >> 4, ncb = (cols + 15) >> 4;
             float acc[4][4];
@@ -141,30 +156,67 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
                 for (int c = 0; c < 4; ++c) {
                     if (r >= nrb || c >= ncb || (diag && c < r)) continue;
                     const int i = ty + 16 * r, j = tx + 16 * c;
-                    L.dist[i * kDistPitch + j] = acc[r][c];
-                    if (diag && c > r) L.dist[j * kDistPitch + i] = acc[r][c];
+                    const float d = acc[r][c];
+                    L.dist[i * kDistPitch + j] = d;
+                    if (diag && c > r) L.dist[j * kDistPitch + i] = d;
+                    if (i < rows && j < cols && !(diag && i == j)) {       // plain stores of the same value: no ordering needed
+                        if (d < L.tau_a[i]) L.flag_a[i] = 1;
+                        if (diag) { if (d < L.tau_a[j]) L.flag_a[j] = 1; }
+                        else if (d < L.tau_b[j]) L.flag_b[j] = 1;
+                    }
                 }
             __syncthreads();
-            // rows of tile I take the columns of tile J as candidates
-            for (int i = wave; i < rows; i += 4) {
-                const int p = L.ida[i];
-                KnnRow<SL> row;
-                row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
-                const bool ok = lane < cols && !(diag && lane == i);
-                const float d = L.dist[i * kDistPitch + lane];
-                row.offer_lanes(ok, L.idb[lane], d);
-                if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
-            }
-            if (!diag) {
-                // columns of tile J take the rows of tile I as candidates
-                for (int j = wave; j < cols; j += 4) {
-                    const int p = L.idb[j];
+            // Rows of tile I take the columns of tile J as candidates, then (off the diagonal) the columns of tile J
+            // the rows of tile I.  A wavefront walks its rows that have a candidate, the next one's row in flight.
+            for (int side = 0; side < (diag ? 1 : 2); ++side) {
+                const int n_mine = side == 0 ? rows : cols, n_other = side == 0 ? cols : rows;
+                const int* id_mine = side == 0 ? L.ida : L.idb;
+                const int* id_other = side == 0 ? L.idb : L.ida;
+                const int* flag = side == 0 ? L.flag_a : L.flag_b;
+                const int fm = wave + 4 * lane;                       // bit u of the mask: member wave + 4 u
+                uint32_t active = (uint32_t)ballot64(lane < 16 && fm < n_mine && flag[fm < kTile ? fm : 0] != 0);
+                auto next_member = [&]() {
+                    if (active == 0) return -1;
+                    const int u = __ffs(active) - 1;
+                    active &= active - 1;
+                    return wave + 4 * u;
+                };
+                int ci = next_member();
+                int ri[SL];
+                float rd[SL];
+                auto fetch = [&](int i, int (&oi)[SL], float (&od)[SL]) {
+#pragma unroll
+                    for (int sl = 0; sl < SL; ++sl) {
+                        const int k = lane + 64 * sl;
+                        oi[sl] = -2;
+                        od[sl] = INFINITY;
+                        if (i >= 0 && k < K) {
+                            const size_t at = (size_t)id_mine[i] * (size_t)K + k;
+                            oi[sl] = knn_idx[at];
+                            od[sl] = knn_dist[at];
+                        }
+                    }
+                };
+                fetch(ci, ri, rd);
+                while (ci >= 0) {
+                    const int ni = next_member();
+                    int nri[SL];
+                    float nrd[SL];
+                    fetch(ni, nri, nrd);
                     KnnRow<SL> row;
-                    row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
-                    const bool ok = lane < rows;
-                    const float d = L.dist[lane * kDistPitch + j];
-                    row.offer_lanes(ok, L.ida[lane], d);
-                    if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
+#pragma unroll
+                    for (int sl = 0; sl < SL; ++sl) { row.idx[sl] = ri[sl]; row.dist[sl] = rd[sl]; }
+                    row.init_from_regs(K);                            // rows that arrive unsorted are rebuilt here
+                    const bool ok = lane < n_other && !(diag && lane == ci);
+                    const float d = side == 0 ? L.dist[ci * kDistPitch + lane] : L.dist[lane * kDistPitch + ci];
+                    row.offer_lanes(ok, id_other[lane], d);
+                    if (row.changed) {
+                        const size_t at = (size_t)id_mine[ci] * (size_t)K;
+                        row.store(knn_idx + at, knn_dist + at);
+                    }
+                    ci = ni;
+#pragma unroll
+                    for (int sl = 0; sl < SL; ++sl) { ri[sl] = nri[sl]; rd[sl] = nrd[sl]; }
                 }
             }
         }
@@ -174,16 +226,20 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
 namespace {
 
 int launch_general(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
-                   int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream)
+                   int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted = false)
 {
     if (n_buckets <= 0) return 0;
     dim3 grid((unsigned)n_buckets), block(256);
+    const int rs = rows_sorted ? 1 : 0;
     if (K <= 64)
-        hipLaunchKernelGGL(k_bucket_knn<1>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx, knn_dist);
+        hipLaunchKernelGGL(k_bucket_knn<1>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
+                           knn_dist, rs);
     else if (K <= 128)
-        hipLaunchKernelGGL(k_bucket_knn<2>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx, knn_dist);
+        hipLaunchKernelGGL(k_bucket_knn<2>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
+                           knn_dist, rs);
     else
-        hipLaunchKernelGGL(k_bucket_knn<4>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx, knn_dist);
+        hipLaunchKernelGGL(k_bucket_knn<4>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
+                           knn_dist, rs);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -230,7 +286,7 @@ int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_so
             if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
-        } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream)) {
+        } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted)) {
             return 1;
         }
     }
@@ -244,7 +300,8 @@ int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_so
         if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
         skip_upto = medium_bucket_cap();
     }
-    return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream);
+    return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream,
+                          rows_sorted);
 }
 
 }  // namespace rsfk
