@@ -416,6 +416,162 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
 
+// The same for rows so long that the set of one point takes most of the LDS a wavefront could get (K above 64: a point
+// has up to K^2 marks): one workgroup of four wavefronts per point.  The first wavefront gathers the marked ids into
+// the set and compacts it (as above); then every wavefront takes every fourth batch of 64 candidates with its own
+// copy of the row and its own tile, and the first one merges the four rows and stores the result.
+// LDS (ints): table[table_size] | srow[K] | xrow[dpad] | region, region = marked[3/4 table_size] first, then
+// 4 tiles + 3 rows for the exchange.
+template <int SL>
+__global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restrict__ points, int N, int D, int K,
+                                                          const int* __restrict__ old_idx, int* __restrict__ knn_idx,
+                                                          float* __restrict__ knn_dist, int table_size, int dpad,
+                                                          const int* __restrict__ fwd2rev, const uint32_t* __restrict__ pass,
+                                                          const int* __restrict__ todo_in, int n_in,
+                                                          int* __restrict__ todo_out, int* __restrict__ n_out)
+{
+    extern __shared__ __align__(16) int lds_w[];
+    __shared__ int U_s;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int slot = blockIdx.x;
+    if (slot >= (todo_in ? n_in : N)) return;
+    const int p = todo_in ? todo_in[slot] : slot;
+    const int MW = (K + 31) >> 5;
+    int* table = lds_w;
+    int* srow = table + table_size;
+    float* xrow = reinterpret_cast<float*>(srow + ((K + 3) & ~3));
+    int* region = reinterpret_cast<int*>(xrow + dpad);
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+
+    KnnRow<SL> row;
+    row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+    for (int k = threadIdx.x; k < K; k += 256) srow[k] = old_idx[(size_t)p * K + k];
+    const float* xp = points + (size_t)p * D;
+    for (int d = threadIdx.x; d < dpad; d += 256) xrow[d] = d < D ? xp[d] : 0.0f;
+    if (threadIdx.x == 0) U_s = 0;
+    __syncthreads();
+    if (wave == 0) {
+        int bits = 0;
+        for (int k = lane; k < K; k += 64) {
+            const int j = fwd2rev[(size_t)p * K + k];
+            if (j >= 0)
+                for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
+        }
+        const int n_given = wave_sum_i(bits);
+        int U = 0;
+        if (n_given + K + 1 > table_size / 4 * 3) {
+            if (lane == 0) todo_out[atomicAdd(n_out, 1)] = p;
+        } else if (n_given > 0) {
+            int ts = 64;
+            while (ts < 2 * (n_given + K + 1)) ts <<= 1;
+            ts = min(ts, table_size);
+            const int mask = ts - 1;
+            for (int i = lane; i < ts; i += 64) table[i] = kEmpty;
+            wave_lds_sync();
+            if (lane == 0) set_insert(table, mask, p, true);
+#pragma unroll
+            for (int s = 0; s < SL; ++s)
+                if (row.idx[s] >= 0) set_insert(table, mask, row.idx[s], true);
+            int* marked = region;
+            int n_marked = 0;                                     // wave-uniform
+            for (int k0 = 0; k0 < K; k0 += 64) {
+                const int k = k0 + lane;
+                const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
+                int mine = 0;
+                if (j >= 0)
+                    for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
+                int at = n_marked + wave_excl_scan_i(mine);
+                if (j >= 0) {
+                    for (int w = 0; w < MW; ++w) {
+                        uint32_t m = pass[(size_t)j * MW + w];
+                        while (m) {
+                            const int b = __ffs(m) - 1;
+                            m &= m - 1;
+                            marked[at++] = k | ((32 * w + b) << 8);
+                        }
+                    }
+                }
+                n_marked += wave_sum_i(mine);
+            }
+            wave_lds_sync();
+            for (int i0 = 0; i0 < n_marked; i0 += 64) {
+                const int i = i0 + lane;
+                int c = -1;
+                if (i < n_marked) {
+                    const int e = marked[i];
+                    c = old_idx[(size_t)srow[e & 255] * K + (e >> 8)];
+                }
+                if (c >= 0 && c < N) set_insert(table, mask, c, false);
+            }
+            wave_lds_sync();
+            for (int t0 = 0; t0 < ts; t0 += 64) {                 // compact the set in place into the candidate list
+                const int v = table[t0 + lane];
+                const bool is_cand = v >= 0;
+                const uint64_t m = ballot64(is_cand);
+                wave_lds_sync();
+                if (is_cand) table[U + mask_prefix(m)] = v;
+                U += __popcll(m);
+            }
+        }
+        if (lane == 0) U_s = U;
+    }
+    __syncthreads();                                              // the list is complete, `marked` is free
+    const int U = U_s;
+    if (U <= 0) return;
+    ExploreLds L;
+    L.tile = reinterpret_cast<float*>(region + wave * kMergeTile);
+    L.xrow = xrow;
+    L.queue2 = nullptr;
+    L.table = nullptr;
+    L.srow = nullptr;
+    for (int off = 64 * wave; off < U; off += 256) {
+        wave_lds_sync();
+        exact_batch<SL, kMergeChunk>(L, table + off, min(64, U - off), points, D, vec_ok, row);
+    }
+    int* xch = region + 4 * kMergeTile;                           // rows of the wavefronts 1..3: [w - 1][idx | dist][64 SL]
+    if (wave > 0) {
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            xch[((wave - 1) * 2 + 0) * (64 * SL) + lane + 64 * s] = row.idx[s];
+            xch[((wave - 1) * 2 + 1) * (64 * SL) + lane + 64 * s] = __float_as_int(row.dist[s]);
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        for (int w = 0; w < 3; ++w) {
+#pragma unroll
+            for (int s = 0; s < SL; ++s) {
+                const int c = xch[(w * 2 + 0) * (64 * SL) + lane + 64 * s];
+                const float d = __int_as_float(xch[(w * 2 + 1) * (64 * SL) + lane + 64 * s]);
+                row.offer_lanes(lane + 64 * s < K && c >= 0, c, d);
+            }
+        }
+        if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
+    }
+}
+
+// ints of LDS the workgroup-per-point merge needs for a set of `table` entries
+int merge_wg_ints(int table, int dpad, int K, int sl)
+{
+    const int region = std::max(table / 4 * 3, 4 * kMergeTile + 6 * 64 * sl);
+    return (table + ((K + 3) & ~3) + dpad + region + 3) / 4 * 4;
+}
+
+template <int SL>
+int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
+                    int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in, int n_in, int* todo_out,
+                    int* n_out, hipStream_t stream)
+{
+    const size_t lds = (size_t)merge_wg_ints(table, dpad, K, SL) * sizeof(int);
+    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge_wg<SL>),
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int n_work = todo_in ? n_in : N;
+    hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3((unsigned)n_work), dim3(256), lds, stream, points, N, D, K, old_idx,
+                       knn_idx, knn_dist, table, dpad, fwd2rev, pass, todo_in, n_in, todo_out, n_out);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
 int next_pow2(int v)
 {
     int p = 1;
@@ -535,10 +691,30 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         todo = listA;
         int big_table = want, big_waves = 4;
         while (big_waves > 1 && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_waves >>= 1;
-        while (big_table > small_table && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_table >>= 1;
+        // fewer than four wavefronts per workgroup would leave the compute units nearly empty: such sets get one
+        // workgroup per point instead
+        const bool per_wg = big_waves < 4;
+        if (per_wg) {
+            big_table = want;
+            while (big_table > small_table && merge_wg_ints(big_table, dpad, K, sl) > lds_ints) big_table >>= 1;
+        } else {
+            while (big_table > small_table && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_table >>= 1;
+        }
         if (big_table > small_table) {
-            if (dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass,
-                               listA, n_todo, listB, listB + N, stream))
+            int rc = 0;
+            if (!per_wg)
+                rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass,
+                                    listA, n_todo, listB, listB + N, stream);
+            else if (sl == 1)
+                rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
+                                        listB, listB + N, stream);
+            else if (sl == 2)
+                rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
+                                        listB, listB + N, stream);
+            else
+                rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
+                                        listB, listB + N, stream);
+            if (rc)
                 return 1;
             RSFK_HIP(hipMemcpyAsync(host_n, listB + N, sizeof(int), hipMemcpyDeviceToHost, stream));
             RSFK_HIP(hipStreamSynchronize(stream));
