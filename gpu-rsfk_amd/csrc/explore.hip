@@ -421,7 +421,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
 // the set and compacts it (as above); then every wavefront takes every fourth batch of 64 candidates with its own
 // copy of the row and its own tile, and the first one merges the four rows and stores the result.
 // LDS (ints): table[table_size] | srow[K] | xrow[dpad] | region, region = marked[3/4 table_size] first, then
-// 4 tiles + 3 rows for the exchange.
+// 4 tiles + 3 rows for the exchange.  Rows pass through the tiles 32 dimensions at a time (whole 128-byte lines).
+constexpr int kWgChunk = 32;
+constexpr int kWgTile = 64 * (kWgChunk + 4);
 template <int SL>
 __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restrict__ points, int N, int D, int K,
                                                           const int* __restrict__ old_idx, int* __restrict__ knn_idx,
@@ -519,16 +521,16 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     const int U = U_s;
     if (U <= 0) return;
     ExploreLds L;
-    L.tile = reinterpret_cast<float*>(region + wave * kMergeTile);
+    L.tile = reinterpret_cast<float*>(region + wave * kWgTile);
     L.xrow = xrow;
     L.queue2 = nullptr;
     L.table = nullptr;
     L.srow = nullptr;
     for (int off = 64 * wave; off < U; off += 256) {
         wave_lds_sync();
-        exact_batch<SL, kMergeChunk>(L, table + off, min(64, U - off), points, D, vec_ok, row);
+        exact_batch<SL, kWgChunk>(L, table + off, min(64, U - off), points, D, vec_ok, row);
     }
-    int* xch = region + 4 * kMergeTile;                           // rows of the wavefronts 1..3: [w - 1][idx | dist][64 SL]
+    int* xch = region + 4 * kWgTile;                           // rows of the wavefronts 1..3: [w - 1][idx | dist][64 SL]
     if (wave > 0) {
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
@@ -553,7 +555,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
 // ints of LDS the workgroup-per-point merge needs for a set of `table` entries
 int merge_wg_ints(int table, int dpad, int K, int sl)
 {
-    const int region = std::max(table / 4 * 3, 4 * kMergeTile + 6 * 64 * sl);
+    const int region = std::max(table / 4 * 3, 4 * kWgTile + 6 * 64 * sl);
     return (table + ((K + 3) & ~3) + dpad + region + 3) / 4 * 4;
 }
 
