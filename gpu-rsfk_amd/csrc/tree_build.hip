@@ -104,7 +104,8 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
 }
 
 // Screen of the side test for eight points per wavefront (right = n.x < b): lanes 8g..8g+7 work on
-// the point of group g; all lanes of a group return its answer.
+// the point of group g; all lanes of a group return its answer.  (With the 8-bit copy and short rows a group may
+// be LPP = 4 or 2 lanes: 16 or 32 points per wavefront.)
 //
 // The decision is always the one of the exact fp32 test (resolve_exact below: 32 lane-strided fused
 // multiply-add chains + xor butterfly, build_tree_check_points_side.cu:131-149), but most points never
@@ -124,7 +125,7 @@ __device__ __forceinline__ void make_hyperplane_wave(const float* __restrict__ x
 // scale sum_d n_d q_d, undecided band e1 ||n||_1 (hp1 = bound of the 1-norm, hp2 = sum of the components of the
 // normal of the point's node).  Only lane 0 of a group holds the header, so only its right / redo are meaningful
 // (with either copy the callers use lane 0 only).
-template <int NB, bool Q8>
+template <int NB, bool Q8, int LPP = 8>
 __device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, const int (&j)[NB], const float (&b)[NB],
                                              const float (&hp1)[NB], const float (&hp2)[NB],
                                              const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8,
@@ -132,7 +133,8 @@ __device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, co
                                              const bool (&valid)[NB], bool (&right)[NB], bool (&redo)[NB])
 {
     if (Q8) {
-        const int sub = lane_id() & 7;
+        static_assert(LPP == 8 || LPP == 4 || LPP == 2, "lanes per point");
+        const int sub = lane_id() & (LPP - 1);
 #pragma unroll
         for (int u = 0; u < NB; ++u) { right[u] = false; redo[u] = valid[u]; }
         const size_t pitch = (size_t)q8_pitch(D);
@@ -145,7 +147,7 @@ __device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, co
             head[u] = make_uint4(0u, 0u, 0u, 0u);
             if (valid[u] && sub == 0) head[u] = *reinterpret_cast<const uint4*>(q8 + (size_t)id[u] * pitch);
         }
-        for (int k = sub; k < pieces; k += 8) {
+        for (int k = sub; k < pieces; k += LPP) {
             uint4 w[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
@@ -169,7 +171,9 @@ __device__ __forceinline__ void side_screen8(const float* nvec0, int nstride, co
 #pragma unroll
         for (int u = 0; u < NB; ++u) {
             float d = da[u];
-            d += dpp_f<kDppXor1>(d); d += dpp_f<kDppXor2>(d); d += dpp_f<kDppHalfMirror>(d);
+            d += dpp_f<kDppXor1>(d);
+            if (LPP >= 4) d += dpp_f<kDppXor2>(d);
+            if (LPP >= 8) d += dpp_f<kDppHalfMirror>(d);
             const float lo = __uint_as_float(head[u].y), scale = __uint_as_float(head[u].z), e1 = __uint_as_float(head[u].w);
             const float approx = __builtin_fmaf(scale, d, lo * hp2[u]);
             const bool certain = fabsf(approx - b[u]) > e1 * hp1[u];       // false if anything is NaN
@@ -457,7 +461,7 @@ __global__ __launch_bounds__(256) void k_level_planes(const float* __restrict__ 
 
 // Side test of one chunk of one node: sets bit 31 of the permutation entry of
 // every member on the right side and counts the members on the left.
-template <bool Q8>
+template <bool Q8, int LPP>
 __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ points,
                                                  const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8,
                                                  TreeParams P,
@@ -486,8 +490,9 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
     const float b = hp_s[0], n1 = hp_s[1], sn = hp_s[2];
     const int pos0 = nd.start + k * P.chunk;
     const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
-    const int grp = threadIdx.x >> 3, sub8 = threadIdx.x & 7;      // 32 groups of 8 lanes, one point each
-    const int iters = (pos1 - pos0 + kGroups - 1) / kGroups;
+    constexpr int kGroupsL = kBlock / LPP;                           // groups of LPP lanes, one point each
+    const int grp = threadIdx.x / LPP, sub8 = threadIdx.x & (LPP - 1);
+    const int iters = (pos1 - pos0 + kGroupsL - 1) / kGroupsL;
     int lefts = 0;
     for (int it = 0; it < iters; it += kSideBatch) {
         int id[kSideBatch], jz[kSideBatch], pos[kSideBatch];
@@ -495,7 +500,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
         bool valid[kSideBatch], right[kSideBatch], redo[kSideBatch];
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
-            pos[u] = pos0 + (it + u) * kGroups + grp;
+            pos[u] = pos0 + (it + u) * kGroupsL + grp;
             valid[u] = pos[u] < pos1;
             id[u] = valid[u] ? (perm[pos[u]] & kIdMask) : 0;
             jz[u] = 0;
@@ -503,7 +508,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
             h1[u] = n1;
             h2[u] = sn;
         }
-        side_screen8<kSideBatch, Q8>(nvec, 0, jz, bb, h1, h2, pb16, q8, id, P.D, P.band, valid, right, redo);
+        side_screen8<kSideBatch, Q8, LPP>(nvec, 0, jz, bb, h1, h2, pb16, q8, id, P.D, P.band, valid, right, redo);
 #pragma unroll
         for (int u = 0; u < kSideBatch; ++u) {
             if (valid[u] && sub8 == 0) {
@@ -1016,12 +1021,16 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         // n_next := 0 for the level being produced
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
-        if (q8)
-            hipLaunchKernelGGL(k_side<true>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
-                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes);
-        else
-            hipLaunchKernelGGL(k_side<false>, dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],
-                               w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes);
+        // lanes per point in the 8-bit screen: a lane takes 16 coordinates per step
+        const int q8_pieces = q8_padded(D) >> 4;
+#define RSFK_SIDE_LAUNCH(Q, L)                                                                                              \
+        hipLaunchKernelGGL((k_side<Q, L>), dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],    \
+                           w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes)
+        if (!q8) RSFK_SIDE_LAUNCH(false, 8);
+        else if (q8_pieces <= 2) RSFK_SIDE_LAUNCH(true, 2);
+        else if (q8_pieces <= 4) RSFK_SIDE_LAUNCH(true, 4);
+        else RSFK_SIDE_LAUNCH(true, 8);
+#undef RSFK_SIDE_LAUNCH
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
                            w->recs, w->n_rec, w->rec_cap);
