@@ -18,7 +18,7 @@ import numpy as np
 sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), ".."))
 
 from gpu_rsfk.RSFK import RSFK                                          # noqa: E402
-from datasets import load_dataset, get_dataset_options                   # noqa: E402
+from synthetic_datasets import load_dataset, get_dataset_options                  # noqa: E402
 from utils.knn_compare import get_nne_rate, create_recall_eps, exact_knn  # noqa: E402
 
 

@@ -39,7 +39,7 @@ def test_exact_knn_against_scipy():
 
 
 def test_datasets_and_parser(tmp_path):
-    from datasets import load_dataset, get_dataset_options
+    from synthetic_datasets import load_dataset, get_dataset_options
     import knn_experiment1
     for name in get_dataset_options():
         X, y = load_dataset(name, 300, 5)
