@@ -645,10 +645,13 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
     RSFK_CHECK(bf == nullptr || bf->mu == nullptr, "exploration: the general kernel needs an uncentred copy");
-    const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr;
+    const int dpad = bf16_valid(D);
+    const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
+    // (rows too long for the LDS of the merge kernel: every point enumerates its own candidates)
+    const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr &&
+                      4 * merge_wave_ints(small_table, dpad, K) <= 150 * 1024 / 4;
     if (join && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
-    const int dpad = bf16_valid(D);
     const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set
     const int lds_ints = 150 * 1024 / 4;                                // usable LDS per workgroup
     // The set must hold the seeds (K+1) and all candidates of a group of neighbours with room to
@@ -681,8 +684,6 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         int* listA = explore_ws_todo(ws, 0);
         int* listB = explore_ws_todo(ws, 1);
         int* host_n = explore_ws_host_count(ws);
-        const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
-        RSFK_CHECK(4 * merge_wave_ints(small_table, dpad, K) <= lds_ints, "exploration: D too large for the merge kernel");
         if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, f2r, pass, nullptr, 0,
                            listA, listA + N, stream))
             return 1;

@@ -442,7 +442,7 @@ __global__ __launch_bounds__(256) void k_level_planes(const float* __restrict__ 
 {
     extern __shared__ __align__(16) float lds_p[];          // per wavefront: 4 + nvec_len(D) floats
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int ni = blockIdx.x * 4 + wave;
+    const int ni = blockIdx.x * (blockDim.x >> 6) + wave;
     if (ni >= n_nodes) return;
     const int rec = 4 + nvec_len(P.D);
     float* mine = lds_p + (size_t)wave * rec;
@@ -1003,6 +1003,20 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
 
     int cur = 0;
     const size_t side_lds = (size_t)(4 + nvec_len(D)) * sizeof(float);
+    RSFK_CHECK(side_lds <= 150 * 1024, "tree batch: D too large for the LDS of the side test");
+    // k_level_planes: four nodes per workgroup while their records fit in 48 KB, else one
+    const int plane_waves = 4 * side_lds <= 48 * 1024 ? 4 : 1;
+    if (side_lds > 48 * 1024) {
+        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_level_planes), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)side_lds));
+        if (q8) {
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_side<true, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)side_lds));
+        } else {
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_side<false, 8>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)side_lds));
+        }
+    }
     // wide levels
     while (true) {
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
@@ -1011,8 +1025,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         const int n_nodes = w->h_ctr->n_next;
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
-        hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + 3) / 4)), dim3(256), 4 * side_lds, stream, points, P,
-                           w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
+        hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + plane_waves - 1) / plane_waves)), dim3(64 * plane_waves),
+                           plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
         hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], n_nodes, P.chunk, w->chunk_base, w->ctr);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));

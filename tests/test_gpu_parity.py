@@ -589,3 +589,20 @@ def test_rows_made_on_the_device_equal_uploaded_rows(gpu, rng, self_in):
     r._lib.pymodule_rsfk_knn(T, K, N, D, K + 1, 2 * K + 2, 5000, 0, 4, 1, X, hi, hd, log)
     assert np.array_equal(gd, hd)
     assert_knn_equal(gi, gd, hi, hd)
+
+
+@pytest.mark.parametrize("N,D,K", [(1500, 9000, 8), (1200, 20000, 6)])
+def test_very_long_rows(gpu, orc, rng, N, D, K):
+    """Rows far beyond what the LDS-resident fast paths take: the kernels with smaller working sets take over and the
+    lists stay those of the oracle (forest with one exploration pass, and the query-set search)."""
+    import gpu_rsfk
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    r = gpu_rsfk.RSFK(random_state=3)
+    _say("long rows", N, D, K)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=1)
+    oi, od = orc.forest(X, K, 1, K + 1, 2 * K + 2, 5000, 3, 1)
+    assert_knn_equal(gi, gd, oi, od)
+    Q = rng.standard_normal((200, D)).astype(np.float32)
+    ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=1)
+    qi, qd = orc.ann_forest(X, Q, K, 1, K + 1, 2 * K + 2, 5000, 3)
+    assert_knn_equal(ai, ad, qi, qd)
