@@ -30,7 +30,8 @@
  *   - reference defects that are not reproduced: empty leaf slots for empty
  *     sides, the unordered is_leaf write, points stranded when MAX_DEPTH is
  *     hit (they become a leaf here), out-of-range reads for -1 neighbours in
- *     the exploration pass, self-insertion in the exploration pass.
+ *     the exploration pass, self-insertion in the exploration pass, NaN
+ *     distances entering a row in the bucket step (they never enter here).
  *
  * Arithmetic is fp32 with explicitly fused multiply-adds where the CUDA
  * compiler would contract them; compile with -ffp-contract=off so nothing
@@ -339,10 +340,12 @@ static inline int first_max(const float* dist, int K)
 }
 
 /* candidate c at distance d against one row; returns 1 if inserted
- * (compute_knn_from_buckets.cu:1215-1230) */
+ * (compute_knn_from_buckets.cu:1215-1230).  Written as "enters iff d < max" (the form of the exploration kernel,
+ * nearest_neighbors_exploring.cu:124) rather than "stays out iff d >= max" (the bucket kernel): the two differ only
+ * for a NaN distance, which the bucket kernel of the reference would store. */
 static inline int try_insert(int* idx, float* dist, int K, int* maxpos, int c, float d)
 {
-    if (d >= dist[*maxpos]) return 0;
+    if (!(d < dist[*maxpos])) return 0;
     for (int k = 0; k < K; ++k) if (idx[k] == c) return 0;
     idx[*maxpos] = c; dist[*maxpos] = d;
     *maxpos = first_max(dist, K);

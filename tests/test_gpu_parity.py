@@ -606,3 +606,20 @@ def test_very_long_rows(gpu, orc, rng, N, D, K):
     ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=1)
     qi, qd = orc.ann_forest(X, Q, K, 1, K + 1, 2 * K + 2, 5000, 3)
     assert_knn_equal(ai, ad, qi, qd)
+
+
+def test_points_with_nan_coordinates(gpu, orc, rng):
+    """A NaN distance is below no row maximum: such points keep only themselves, nobody holds them, and the rest of
+    the graph is the oracle's (same trees: a NaN side test sends the point left in both)."""
+    import gpu_rsfk
+    N, D, K, T = 6000, 10, 8, 3
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    bad = np.arange(0, N, 7)
+    X[bad] = np.nan
+    _say("nan rows")
+    gi, gd = gpu_rsfk.RSFK(random_state=3).find_nearest_neighbors(X, K, n_trees=T)
+    oi, od = orc.init_lists(N, K, self_in=True)
+    orc.forest(X, K, T, K + 1, 2 * K + 2, 5000, 3, 1, knn_idx=oi, knn_dist=od)
+    assert not np.isnan(gd).any() and not np.isnan(od).any()
+    assert (gi[bad, 0] == bad).all() and (gi[bad, 1:] == -1).all()
+    assert_knn_equal(gi, gd, oi, od)

@@ -169,3 +169,20 @@ def test_forest_merges_into_existing_lists(orc, rng):
         orc.bucket_knn(X, K, perm, lz, idx, dist, starts=ls)
     bad_d, bad_i, _ = compare_knn(i2, d2, idx, dist)
     assert bad_d == 0 and bad_i == 0
+
+
+def test_nan_distances_never_enter_a_row(orc):
+    """Points with NaN coordinates: their distance to anything is NaN, which is below no row maximum."""
+    rng = np.random.default_rng(5)
+    N, D, K = 400, 6, 5
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    bad = np.arange(0, N, 9)
+    X[bad, 2] = np.nan
+    idx, dist = orc.init_lists(N, K, self_in=True)
+    perm, ls, lz, _ = orc.build_tree(X, K + 1, 2 * K + 2, 5000, 0)
+    orc.bucket_knn(X, K, perm, lz, idx, dist, starts=ls)
+    orc.explore(X, K, idx, dist)
+    assert not np.isnan(dist).any()
+    assert (idx[bad, 0] == bad).all() and (idx[bad, 1:] == -1).all()          # their rows keep only themselves
+    good = np.setdiff1d(np.arange(N), bad)
+    assert not np.isin(idx[good], bad).any()                                  # and nobody holds them
