@@ -389,12 +389,13 @@ __global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr
 }
 
 // chunk_base[i] = number of chunks of nodes [0,i); one workgroup.
-__global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict__ nodes, int n_nodes, int chunk,
+__global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict__ nodes, int node_cap, int chunk,
                                                       int* __restrict__ chunk_base, LevelCounters* ctr)
 {
     __shared__ int wsum[16];
     __shared__ int carry_s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n_nodes = min(ctr->n_next, node_cap);       // nodes of the level, left by the previous level's scatter
     if (tid == 0) carry_s = 0;
     __syncthreads();
     for (int base = 0; base < n_nodes; base += 1024) {
@@ -1019,19 +1020,19 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     }
     // wide levels
     while (true) {
+        // one trip to the host per level: the chunk table of the level is made first (from the node count on the
+        // device), then both counts come back together
+        hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], w->node_cap, P.chunk, w->chunk_base, w->ctr);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
         RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
         const int n_nodes = w->h_ctr->n_next;
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
-        hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + plane_waves - 1) / plane_waves)), dim3(64 * plane_waves),
-                           plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
-        hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], n_nodes, P.chunk, w->chunk_base, w->ctr);
-        RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
-        RSFK_HIP(hipStreamSynchronize(stream));
         const int n_chunks = w->h_ctr->n_chunks;
         RSFK_CHECK(n_chunks <= w->chunk_cap, "tree batch: chunk table overflow");
+        hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + plane_waves - 1) / plane_waves)), dim3(64 * plane_waves),
+                           plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
         // n_next := 0 for the level being produced
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
