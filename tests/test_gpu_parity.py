@@ -274,6 +274,12 @@ def test_golden_vectors(gpu):
     import gpu_rsfk
     fi, fd = gpu_rsfk.RSFK(seed).find_nearest_neighbors(X, K, n_trees=3, min_tree_children=MIN, max_tree_children=MAX)
     assert_knn_equal(fi, fd, g["forest_idx"], g["forest_dist"])
+    qi, qd = gpu_rsfk.RSFK(seed).find_nearest_neighbors_ann(X, g["Q"], K, n_trees=3, min_tree_children=MIN,
+                                                            max_tree_children=MAX, ensure_valid_indices=False)
+    assert_knn_equal(qi, qd, g["ann_idx"], g["ann_dist"])
+    indptr, cols, vals = gpu_rsfk.symmetric_knn_graph(g["forest_idx"], g["forest_dist"], drop_self=True)
+    assert np.array_equal(indptr, g["csr_indptr"]) and np.array_equal(cols, g["csr_indices"])
+    assert np.array_equal(vals, g["csr_data"])
 
 
 # ---------------------------------------------------------------------------

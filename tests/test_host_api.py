@@ -145,3 +145,8 @@ def test_golden_vectors_still_come_out_of_the_oracle(orc):
     assert np.array_equal(bi, g["bucket_idx"]) and np.array_equal(bd, g["bucket_dist"])
     fi, fd = sort_rows(*orc.forest(X, K, 3, MIN, MAX, 5000, seed, 1))
     assert np.array_equal(fi, g["forest_idx"]) and np.array_equal(fd, g["forest_dist"])
+    qi, qd = sort_rows(*orc.ann_forest(X, g["Q"], K, 3, MIN, MAX, 5000, seed))
+    assert np.array_equal(qi, g["ann_idx"]) and np.array_equal(qd, g["ann_dist"])
+    indptr, cols, vals = orc.symmetrize(g["forest_idx"], g["forest_dist"], drop_self=True)
+    assert np.array_equal(indptr, g["csr_indptr"]) and np.array_equal(cols, g["csr_indices"])
+    assert np.array_equal(vals, g["csr_data"])
