@@ -48,6 +48,7 @@ int choose_batch(int n_trees, int N, int D, int MIN)
     if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = (size_t)8 << 30;
     const size_t budget = free_b / 4;
     int B = std::min(n_trees, 64);
+    if (const char* e = std::getenv("RSFK_TREE_BATCH")) B = std::min(B, std::max(1, std::atoi(e)));     // for tests
     while (B > 1 && tree_ws_bytes(N, D, MIN, B) > budget) --B;
     return std::max(B, 1);
 }

@@ -629,3 +629,22 @@ def test_points_with_nan_coordinates(gpu, orc, rng):
     assert not np.isnan(gd).any() and not np.isnan(od).any()
     assert (gi[bad, 0] == bad).all() and (gi[bad, 1:] == -1).all()
     assert_knn_equal(gi, gd, oi, od)
+
+
+def test_forest_in_several_batches(gpu, orc, rng, monkeypatch):
+    """Trees are built a batch at a time (all at once when memory allows); two per batch must give the same graph,
+    for the K-NN graph (buckets of both kinds, so both streams of the bucket step are in use) and the query search."""
+    import gpu_rsfk
+    monkeypatch.setenv("RSFK_TREE_BATCH", "2")
+    N, D, K, T = 30000, 20, 32, 5
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    Q = rng.standard_normal((2000, D)).astype(np.float32)
+    r = gpu_rsfk.RSFK(random_state=9)
+    _say("batches")
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=T)
+    oi, od = orc.forest(X, K, T, K + 1, 2 * K + 2, 5000, 9, 1)
+    assert_knn_equal(gi, gd, oi, od)
+    assert r.log_forest.data["Total Leaves"] == [len(orc.build_tree(X, K + 1, 2 * K + 2, 5000, 9 + t)[2]) for t in range(T)]
+    ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T)
+    qi, qd = orc.ann_forest(X, Q, K, T, K + 1, 2 * K + 2, 5000, 9)
+    assert_knn_equal(ai, ad, qi, qd)
