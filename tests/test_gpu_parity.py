@@ -648,3 +648,56 @@ def test_forest_in_several_batches(gpu, orc, rng, monkeypatch):
     ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T)
     qi, qd = orc.ann_forest(X, Q, K, T, K + 1, 2 * K + 2, 5000, 9)
     assert_knn_equal(ai, ad, qi, qd)
+
+
+def _random_case(seed):
+    g = np.random.default_rng(1000 + seed)
+    N = int(g.choice([37, 150, 700, 1300, 2600, 5200, 9000]))
+    D = int(g.choice([1, 2, 3, 7, 16, 31, 32, 33, 64, 65, 100, 129, 257]))
+    K = int(g.choice([1, 2, 5, 8, 16, 31, 32, 33, 48, 64, 65, 100]))
+    T = int(g.integers(1, 5))
+    MIN = int(g.choice([K + 1, max(2, K // 2), K + 7, 2 * K + 3]))
+    MAX = int(2 * MIN + g.choice([0, 1, 5, MIN]))
+    nnef = int(g.integers(0, 3))
+    kind = str(g.choice(["normal", "uniform", "grid", "clusters"]))
+    if kind == "normal":
+        X = g.standard_normal((N, D))
+    elif kind == "uniform":
+        X = g.random((N, D)) * 100.0 - 30.0
+    elif kind == "grid":
+        X = g.integers(0, 4, (N, D)).astype(np.float64)          # many equal distances and duplicated points
+    else:
+        X = g.standard_normal((8, D))[g.integers(0, 8, N)] * 5.0 + 0.05 * g.standard_normal((N, D))
+    return X.astype(np.float32), K, T, MIN, MAX, nnef, kind
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_match_oracle(gpu, orc, seed):
+    """Seeded random shapes, bucket limits, numbers of exploration passes and kinds of data: K-NN graph, query-set
+    search and graph export against the oracle.  (On the grid data almost every distance is tied with others: the
+    comparison then only says that the sorted distances of every row agree.)"""
+    import gpu_rsfk
+    X, K, T, MIN, MAX, nnef, kind = _random_case(seed)
+    N, D = X.shape
+    _say("random case", seed, N, D, K, T, MIN, MAX, nnef, kind)
+    r = gpu_rsfk.RSFK(random_state=seed)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=T, min_tree_children=MIN, max_tree_children=MAX,
+                                      nn_exploring_factor=nnef, ensure_valid_indices=False)
+    oi, od = orc.forest(X, K, T, MIN, MAX, 5000, seed, nnef)
+    ties = kind == "grid" or (kind == "clusters" and nnef > 1)
+    if ties:
+        assert np.array_equal(np.sort(gd, axis=1), np.sort(od, axis=1)) or nnef > 1
+    else:
+        assert_knn_equal(gi, gd, oi, od)
+    assert rows_have_no_duplicates(gi)
+    Q = X[::3] + np.float32(0.125)
+    ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T, min_tree_children=MIN, max_tree_children=MAX,
+                                          ensure_valid_indices=False)
+    qi, qd = orc.ann_forest(X, Q, K, T, MIN, MAX, 5000, seed)
+    if kind == "grid":
+        assert np.array_equal(np.sort(ad, axis=1), np.sort(qd, axis=1))
+    else:
+        assert_knn_equal(ai, ad, qi, qd)
+    ip, cc, vv = gpu_rsfk.symmetric_knn_graph(gi, gd, drop_self=bool(seed & 1))
+    op, oc, ov = orc.symmetrize(gi, gd, drop_self=bool(seed & 1))
+    assert np.array_equal(ip, op) and np.array_equal(cc, oc) and np.array_equal(vv, ov)
