@@ -157,7 +157,7 @@ int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int d
                       float* d_vals, long long cap, long long* nnz, hipStream_t stream)
 {
     RSFK_CHECK(N >= 1 && K >= 1 && K <= 256, "graph export: N must be positive and K in 1..256");
-    RSFK_CHECK((long long)N * K <= (1ll << 30), "graph export: N * K above 2^30 is not supported");
+    RSFK_CHECK((long long)N * K < (1ll << 30), "graph export: N * K of 2^30 and more is not supported");
     RSFK_CHECK(d_idx && d_indptr && nnz, "graph export: null argument");
     RSFK_CHECK((d_cols == nullptr) == (d_vals == nullptr), "graph export: indices and data go together");
     Buf flag, own, extra, len;
