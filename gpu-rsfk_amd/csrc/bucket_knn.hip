@@ -160,9 +160,9 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
                     L.dist[i * kDistPitch + j] = d;
                     if (diag && c > r) L.dist[j * kDistPitch + i] = d;
                     if (i < rows && j < cols && !(diag && i == j)) {       // plain stores of the same value: no ordering needed
-                        if (d < L.tau_a[i]) L.flag_a[i] = 1;
-                        if (diag) { if (d < L.tau_a[j]) L.flag_a[j] = 1; }
-                        else if (d < L.tau_b[j]) L.flag_b[j] = 1;
+                        if (d <= L.tau_a[i]) L.flag_a[i] = 1;
+                        if (diag) { if (d <= L.tau_a[j]) L.flag_a[j] = 1; }
+                        else if (d <= L.tau_b[j]) L.flag_b[j] = 1;
                     }
                 }
             __syncthreads();
@@ -209,11 +209,11 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
                     row.init_from_regs(K);                            // rows that arrive unsorted are rebuilt here
                     const bool ok = lane < n_other && !(diag && lane == ci);
                     const float d = side == 0 ? L.dist[ci * kDistPitch + lane] : L.dist[lane * kDistPitch + ci];
-                    row.offer_lanes(ok, id_other[lane], d);
-                    if (row.changed) {
-                        const size_t at = (size_t)id_mine[ci] * (size_t)K;
-                        row.store(knn_idx + at, knn_dist + at);
-                    }
+                    const size_t at = (size_t)id_mine[ci] * (size_t)K;
+                    const bool okv[1] = {ok};
+                    const int cv[1] = {id_other[lane]};
+                    const float dv[1] = {d};
+                    row.template merge_store<1>(okv, cv, dv, knn_idx + at, knn_dist + at);
                     ci = ni;
 #pragma unroll
                     for (int sl = 0; sl < SL; ++sl) { ri[sl] = nri[sl]; rd[sl] = nrd[sl]; }

@@ -85,11 +85,11 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
             df = a.z - x.z; acc = __builtin_fmaf(df, df, acc);
             df = a.w - x.w; acc = __builtin_fmaf(df, df, acc);
         }
-        // partial sums only grow: once all of them reached the row maximum nothing can enter
-        if (ballot64(lane < n && acc < tau0) == 0) break;
+        // partial sums only grow: once all of them are above the row maximum nothing can enter
+        if (ballot64(lane < n && acc <= tau0) == 0) break;
     }
     wave_lds_sync();
-    row.offer_lanes(lane < n, my_c, acc);
+    row.merge(lane < n, my_c, acc, reinterpret_cast<int*>(L.tile));      // the tile is free: it serves as the merge's scratch
 }
 
 }  // namespace rsfk

@@ -157,7 +157,7 @@ __device__ __forceinline__ void screen_stage_finish(const ScreenCtx& C, const Ex
     const float qn = bf.norms[my_c];
     const float slack = (float)(C.D + 8) * (1.0f / 4194304.0f);      // (D+8) 2^-22: fp32 summation error of both sums
     const float e = ta * (1.02f / 128.0f) + qn * (1.05f / 65536.0f) + da * slack;
-    const bool may = lane < n && (da - e < row.tau);
+    const bool may = lane < n && (da - e <= row.tau);
     const uint64_t pm = ballot64(may);
     if (pm == 0) return;
     if (may) L.queue2[queued2 + mask_prefix(pm)] = my_c;
@@ -545,7 +545,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
             for (int s = 0; s < SL; ++s) {
                 const int c = xch[(w * 2 + 0) * (64 * SL) + lane + 64 * s];
                 const float d = __int_as_float(xch[(w * 2 + 1) * (64 * SL) + lane + 64 * s]);
-                row.offer_lanes(lane + 64 * s < K && c >= 0, c, d);
+                row.merge(lane + 64 * s < K && c >= 0, c, d, region);      // the tiles are free by now
             }
         }
         if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);

@@ -211,7 +211,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
                 const float Q = 2.0001f * S;
                 const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);
                 const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;
-                const bool skip = lower >= ptau[m];       // false if anything is NaN
+                const bool skip = lower > ptau[m];        // false if anything is NaN; a tie at the last slot may still enter (smaller index)
                 const uint64_t bm = ballot64(cid >= 0 && !skip);
                 const int m_lo = 8 * (i >> 2) + (i & 3);
                 if (lane == m_lo) mine = (uint32_t)bm;

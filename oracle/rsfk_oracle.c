@@ -331,24 +331,41 @@ RSFK_OR_EXPORT int rsfk_or_route_queries(const float* points, int N, int D,
 /* K-NN list update rule                                               */
 /* ------------------------------------------------------------------ */
 
-/* position of the first maximum of dist[0..K) (strict '>' scan) */
-static inline int first_max(const float* dist, int K)
+/*
+ * The rows are ordered by (distance, index): entry (d1, c1) is above (d2, c2) iff d1 > d2, or d1 == d2 and
+ * c1 > c2.  An empty slot (-1, +inf or FLT_MAX) is above every candidate that can enter.
+ */
+static inline int pair_above(float d1, int c1, float d2, int c2)
+{
+    return d1 > d2 || (d1 == d2 && c1 > c2);
+}
+
+/* position of the largest (distance, index) of the row */
+static inline int row_max(const int* idx, const float* dist, int K)
 {
     int m = 0;
-    for (int j = 1; j < K; ++j) if (dist[j] > dist[m]) m = j;
+    for (int j = 1; j < K; ++j) if (pair_above(dist[j], idx[j], dist[m], idx[m])) m = j;
     return m;
 }
 
-/* candidate c at distance d against one row; returns 1 if inserted
- * (compute_knn_from_buckets.cu:1215-1230).  Written as "enters iff d < max" (the form of the exploration kernel,
- * nearest_neighbors_exploring.cu:124) rather than "stays out iff d >= max" (the bucket kernel): the two differ only
- * for a NaN distance, which the bucket kernel of the reference would store. */
+/*
+ * Candidate c at distance d against one row; returns 1 if inserted.  The reference lets a candidate enter iff it
+ * is strictly closer than the row's maximum and not in the row, and it then replaces the (first) maximum
+ * (compute_knn_from_buckets.cu:1215-1230, nearest_neighbors_exploring.cu:124-141); among points at exactly the
+ * K-th distance the row then keeps whichever arrived first.  Here a candidate enters iff its (distance, index) is
+ * below the row's largest (distance, index), which it replaces: the row ends with the K smallest (distance, index)
+ * pairs of everything it was offered, whatever the order of arrival.  The two rules differ only among points tied
+ * at a row's K-th distance.  A candidate at +inf or NaN never enters (the reference's bucket kernel would store
+ * a NaN, its exploration kernel would not).
+ */
 static inline int try_insert(int* idx, float* dist, int K, int* maxpos, int c, float d)
 {
-    if (!(d < dist[*maxpos])) return 0;
+    const int m = *maxpos;
+    if (!(d < INFINITY)) return 0;
+    if (!(d < dist[m] || (d == dist[m] && c < idx[m]))) return 0;
     for (int k = 0; k < K; ++k) if (idx[k] == c) return 0;
-    idx[*maxpos] = c; dist[*maxpos] = d;
-    *maxpos = first_max(dist, K);
+    idx[m] = c; dist[m] = d;
+    *maxpos = row_max(idx, dist, K);
     return 1;
 }
 
@@ -376,7 +393,7 @@ RSFK_OR_EXPORT void rsfk_or_bucket_knn(const float* points, int N, int D, int K,
                 cand = (float*)realloc(cand, sizeof(float) * (size_t)capc);
                 maxpos = (int*)realloc(maxpos, sizeof(int) * (size_t)capc);
             }
-            for (int i = 0; i < s; ++i) maxpos[i] = first_max(knn_dist + (size_t)bid[i] * K, K);
+            for (int i = 0; i < s; ++i) maxpos[i] = row_max(knn_idx + (size_t)bid[i] * K, knn_dist + (size_t)bid[i] * K, K);
             for (int off = 1; off < s; ++off) {
                 for (int i = 0; i + off < s; ++i)
                     cand[i] = rsfk_or_sqdist(points + (size_t)bid[i] * D, points + (size_t)bid[i + off] * D, D);
@@ -408,7 +425,7 @@ RSFK_OR_EXPORT void rsfk_or_explore(const float* points, int N, int D, int K,
         int* idx = knn_idx + (size_t)p * K;
         float* dist = knn_dist + (size_t)p * K;
         const float* xp = points + (size_t)p * D;
-        int maxpos = first_max(dist, K);
+        int maxpos = row_max(idx, dist, K);
         for (int i = 0; i < K; ++i) {
             int q = old[(size_t)p * K + i];
             if (q < 0 || q >= N) continue;
@@ -419,10 +436,7 @@ RSFK_OR_EXPORT void rsfk_or_explore(const float* points, int N, int D, int K,
                 for (int j = 0; j < K; ++j) if (idx[j] == c) { dup = 1; break; }
                 if (dup) continue;
                 float d = rsfk_or_sqdist(points + (size_t)c * D, xp, D);
-                if (d < dist[maxpos]) {
-                    idx[maxpos] = c; dist[maxpos] = d;
-                    maxpos = first_max(dist, K);
-                }
+                try_insert(idx, dist, K, &maxpos, c, d);
             }
         }
     }
@@ -550,7 +564,7 @@ RSFK_OR_EXPORT int rsfk_or_ann_forest(int n_trees, int K, int N, int NQ, int D,
         for (int q = 0; q < NQ; ++q) {
             int* idx = q_idx + (size_t)q * K;
             float* dist = q_dist + (size_t)q * K;
-            int maxpos = first_max(dist, K);
+            int maxpos = row_max(idx, dist, K);
             for (int i = 0; i < qz[q]; ++i) {
                 int c = perm[qs[q] + i];
                 float d = rsfk_or_sqdist(queries + (size_t)q * D, points + (size_t)c * D, D);

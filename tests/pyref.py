@@ -5,8 +5,9 @@ inputs.  They are written from the rules, not from the oracle's C code:
             src/kernels/build_tree_update_parents.cu:64-75,106-134 and the
             pair draw per (node, side) of build_tree_create_nodes.cu:86-104,
             expressed recursively over Python lists;
-  insert  : "replace the maximum iff strictly closer and not present"
-            (compute_knn_from_buckets.cu:1215-1230);
+  insert  : "replace the maximum iff below it and not present"
+            (compute_knn_from_buckets.cu:1215-1230), with rows ordered by
+            (distance, index) so that ties at the K-th distance keep the smaller index;
   explore : nearest_neighbors_exploring.cu:70-141;
   route   : the descent of a query point through a tree (src/rsfk.cu:262-356,
             build_tree_update_parents_ann.cu:141-151): side test where the node has
@@ -102,8 +103,8 @@ def route(orc, X, Q, MIN, MAX, MAX_DEPTH, seed):
 
 def insert(idx_row, dist_row, c, d):
     """One candidate against one row (lists, modified in place)."""
-    m = max(range(len(dist_row)), key=lambda j: (dist_row[j], -j))     # first maximum
-    if not (d < dist_row[m]):
+    m = max(range(len(dist_row)), key=lambda j: (dist_row[j], idx_row[j]))     # largest (distance, index)
+    if not (d < float("inf")) or not ((d, c) < (dist_row[m], idx_row[m])):
         return False
     if c in idx_row:
         return False

@@ -1,17 +1,18 @@
 """GPU parity tests: the HIP library, called through its C ABI, against the CPU
 oracle on the same seeded inputs.
 
-Bar: the tree partition (integer work) must be identical; K-NN rows are
-compared as sets and must hold bit-identical distances and identical indices
-except among entries tied at the row's K-th distance (the order in which equal
-candidates arrive is the only freedom the algorithm leaves).
+Bar: the tree partition (integer work) must be identical; K-NN rows, sorted by
+(distance, index), must hold bit-identical distances and identical indices, ties
+included (library and oracle order a row by (distance, index), so no result
+depends on the order in which candidates arrive).
 """
 import os
 
 import numpy as np
 import pytest
 
-from util import assert_knn_equal, check_partition, exact_knn_numpy, recall, rows_have_no_duplicates, sort_rows
+from util import (assert_knn_equal, baseline_points, check_partition, exact_knn_numpy, recall, rows_have_no_duplicates,
+                  sort_rows)
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -230,6 +231,83 @@ def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D,
     assert_knn_equal(gi, gd, oi, od)
 
 
+# The workloads of the benchmark configurations 3, 4 and 5 (clustered D=256; sparse D=784 with K=90 and one
+# exploration pass, the only shape that runs the general bucket kernel with two slots per lane together with the
+# workgroup-per-point exploration merge; standard normal D=32 with buckets of 64..256 points), as forest +
+# exploration through the package against the oracle, at sizes the oracle finishes in seconds.
+@pytest.mark.parametrize("config,N,K,T,kw", [
+    ("c3", 24000, 32, 6, {}),
+    ("c4", 9000, 90, 4, dict(nn_exploring_factor=1)),
+    ("c5", 70000, 32, 5, dict(min_tree_children=64, max_tree_children=256)),
+], ids=["config3_gmm64_d256_k32", "config4_sparse_d784_k90_explore", "config5_normal_d32_buckets64_256"])
+def test_baseline_config_workloads_match_oracle(gpu, orc, config, N, K, T, kw):
+    import gpu_rsfk
+    X = baseline_points(config, N)
+    r = gpu_rsfk.RSFK(random_state=0)
+    _say("forest", config, N, X.shape[1], K, T, kw)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=T, **kw)
+    mn = kw.get("min_tree_children", K + 1)
+    mx = kw.get("max_tree_children", 2 * mn)
+    nnef = kw.get("nn_exploring_factor", 1 if K <= 32 else 0)
+    assert nnef == 1
+    oi, od, olog = orc.forest(X, K, T, mn, mx, 5000, 0, nnef, want_log=True)
+    assert_knn_equal(gi, gd, oi, od)
+    assert rows_have_no_duplicates(gi) and (gi >= 0).all()
+    log = r.log_forest.data
+    assert log["Total Leaves"] == [int(v) for v in olog[3 * T:4 * T]]
+    assert log["Max Leaf Size"] == [int(v) for v in olog[1 * T:2 * T]]
+
+
+# size-independent properties of the same three workloads at their full sizes
+@pytest.mark.parametrize("config,N,K,T,mn,mx", [
+    ("c3", 1000000, 32, 4, 33, 66),
+    ("c4", 70000, 90, 10, 91, 182),
+    ("c5", 10000000, 32, 3, 64, 256),
+], ids=["config3_full_size", "config4_full_size", "config5_full_size"])
+def test_baseline_config_properties_at_full_size(gpu, orc, config, N, K, T, mn, mx):
+    import torch
+    X = baseline_points(config, N)
+    D = X.shape[1]
+    dX = torch.from_numpy(X).cuda()
+    idx = torch.full((N, K), -1, dtype=torch.int32, device="cuda")
+    idx[:, 0] = torch.arange(N, dtype=torch.int32, device="cuda")
+    dist = torch.full((N, K), float("inf"), dtype=torch.float32, device="cuda")
+    dist[:, 0] = 0
+    log = np.zeros(16 * T + 2, np.float32)
+    _say("full size forest", config, N, D, K, T)
+    gpu.knn_forest_device(T, K, N, D, mn, mx, 5000, 0, 0, 0, dX.data_ptr(), idx.data_ptr(), dist.data_ptr(), log)
+    torch.cuda.synchronize()
+    assert (log[1 * T:2 * T] <= mx).all() and (log[2 * T:3 * T] >= mn).all()
+    assert (log[3 * T:4 * T] >= N / mx).all() and (log[3 * T:4 * T] <= N / mn).all()
+    before = dist.max(1).values.clone()
+    assert bool((idx >= 0).all()) and bool((idx < N).all())
+    assert bool((dist[:, 1:] >= dist[:, :-1]).all())                 # rows come back ascending
+    srt = torch.sort(idx, dim=1).values
+    assert not bool((srt[:, 1:] == srt[:, :-1]).any())               # no point twice in a row
+    del srt
+    rng = np.random.default_rng(3)
+    rows = rng.choice(N, 150, replace=False)
+    hi, hd = idx[torch.from_numpy(rows).cuda()].cpu().numpy(), dist[torch.from_numpy(rows).cuda()].cpu().numpy()
+    for r_, p in enumerate(rows):
+        for k in range(0, K, 7):
+            assert hd[r_, k] == orc.sqdist(X[p], X[hi[r_, k]])       # stored distance = distance of the stored neighbour
+    # one exploration pass: the row maximum only falls, and sampled rows are what the oracle's rule gives from the
+    # same graph (the K smallest (distance, index) of the old row and the neighbours of the old neighbours)
+    old = idx.clone()
+    scratch = torch.empty((N, K), dtype=torch.int32, device="cuda")
+    _say("full size explore", config)
+    gpu.explore_device(dX.data_ptr(), N, D, K, idx.data_ptr(), dist.data_ptr(), scratch.data_ptr())
+    torch.cuda.synchronize()
+    assert bool((dist.max(1).values <= before).all())
+    for p in rows[:40]:
+        orow = old[int(p)].cpu().numpy()
+        cand = np.unique(np.concatenate([orow, old[torch.from_numpy(orow).long().cuda()].cpu().numpy().ravel()]))
+        d = np.array([orc.sqdist(X[c], X[p]) for c in cand], np.float32)
+        order = np.lexsort((cand, d))[:K]
+        assert np.array_equal(idx[int(p)].cpu().numpy(), cand[order])
+        assert np.array_equal(dist[int(p)].cpu().numpy(), d[order])
+
+
 def test_reference_package_smoke_tests(gpu):
     """The two live smoke tests of the reference package (RSFK.py:841-903)."""
     import gpu_rsfk
@@ -324,9 +402,17 @@ def test_properties_at_scale(gpu, orc):
     _say("scale explore")
     gpu.explore_device(dX.data_ptr(), N, D, K, idx.data_ptr(), dist.data_ptr(), scratch.data_ptr())
     torch.cuda.synchronize()
-    gd3 = dist.cpu().numpy()
+    gi3, gd3 = idx.cpu().numpy(), dist.cpu().numpy()
     assert (gd3.max(1) <= before).all()
-    assert rows_have_no_duplicates(idx.cpu().numpy())
+    assert rows_have_no_duplicates(gi3)
+    # the oracle's exploration of a sample of rows, from the same graph: row p after the pass = the K smallest
+    # (distance, index) of its old row and the neighbours of its old neighbours
+    for p in rng.choice(N, 200, replace=False):
+        cand = np.unique(np.concatenate([gi2[p], gi2[gi2[p]].ravel()]))
+        cand = cand[cand != p] if p not in gi2[p] else cand
+        d = np.array([orc.sqdist(X[c], X[p]) for c in cand], np.float32)
+        order = np.lexsort((cand, d))[:K]
+        assert np.array_equal(gi3[p], cand[order]) and np.array_equal(gd3[p], d[order])
 
 
 # ---------------------------------------------------------------------------
@@ -370,17 +456,8 @@ def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant
     r = gpu_rsfk.RSFK(random_state=2)
     gi, gd = r.find_nearest_neighbors(X, K, n_trees=3, max_tree_depth=300, nn_exploring_factor=2)
     oi, od = orc.forest(X, K, 3, K + 1, 2 * (K + 1), 300, 2, 2)
-    if kind == "grid":
-        # equal distances everywhere: which of several tied neighbours survives is arrival order; exploration then
-        # walks different (equally good) neighbours, so only the distance profile of each row is comparable
-        from util import sort_rows
-        assert np.array_equal(sort_rows(gi, gd)[1][:, :1], sort_rows(oi, od)[1][:, :1])
-        assert rows_have_no_duplicates(gi) and (gi >= 0).all()
-        for p in rng.choice(N, 60, replace=False):
-            for k in range(K):
-                assert gd[p, k] == orc.sqdist(X[p], X[gi[p, k]])
-    else:
-        assert_knn_equal(gi, gd, oi, od)
+    assert_knn_equal(gi, gd, oi, od)          # "grid": equal distances everywhere, ties go to the smaller index
+    assert rows_have_no_duplicates(gi)
 
 
 def test_workspace_is_reused_and_can_be_released(gpu, rng):
@@ -674,8 +751,8 @@ def _random_case(seed):
 @pytest.mark.parametrize("seed", range(24))
 def test_random_shapes_match_oracle(gpu, orc, seed):
     """Seeded random shapes, bucket limits, numbers of exploration passes and kinds of data: K-NN graph, query-set
-    search and graph export against the oracle.  (On the grid data almost every distance is tied with others: the
-    comparison then only says that the sorted distances of every row agree.)"""
+    search and graph export against the oracle.  On the grid data almost every distance is tied with others and
+    points are duplicated: rows must still be identical, since ties are broken by index everywhere."""
     import gpu_rsfk
     X, K, T, MIN, MAX, nnef, kind = _random_case(seed)
     N, D = X.shape
@@ -684,20 +761,13 @@ def test_random_shapes_match_oracle(gpu, orc, seed):
     gi, gd = r.find_nearest_neighbors(X, K, n_trees=T, min_tree_children=MIN, max_tree_children=MAX,
                                       nn_exploring_factor=nnef, ensure_valid_indices=False)
     oi, od = orc.forest(X, K, T, MIN, MAX, 5000, seed, nnef)
-    ties = kind == "grid" or (kind == "clusters" and nnef > 1)
-    if ties:
-        assert np.array_equal(np.sort(gd, axis=1), np.sort(od, axis=1)) or nnef > 1
-    else:
-        assert_knn_equal(gi, gd, oi, od)
+    assert_knn_equal(gi, gd, oi, od)
     assert rows_have_no_duplicates(gi)
     Q = X[::3] + np.float32(0.125)
     ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=T, min_tree_children=MIN, max_tree_children=MAX,
                                           ensure_valid_indices=False)
     qi, qd = orc.ann_forest(X, Q, K, T, MIN, MAX, 5000, seed)
-    if kind == "grid":
-        assert np.array_equal(np.sort(ad, axis=1), np.sort(qd, axis=1))
-    else:
-        assert_knn_equal(ai, ad, qi, qd)
+    assert_knn_equal(ai, ad, qi, qd)
     ip, cc, vv = gpu_rsfk.symmetric_knn_graph(gi, gd, drop_self=bool(seed & 1))
     op, oc, ov = orc.symmetrize(gi, gd, drop_self=bool(seed & 1))
     assert np.array_equal(ip, op) and np.array_equal(cc, oc) and np.array_equal(vv, ov)

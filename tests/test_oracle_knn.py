@@ -186,3 +186,66 @@ def test_nan_distances_never_enter_a_row(orc):
     assert (idx[bad, 0] == bad).all() and (idx[bad, 1:] == -1).all()          # their rows keep only themselves
     good = np.setdiff1d(np.arange(N), bad)
     assert not np.isin(idx[good], bad).any()                                  # and nobody holds them
+
+
+def _grid_points(n_side, D, rng):
+    """Integer lattice points in shuffled order: every squared distance is a small integer (exact in fp32 in any
+    summation order) and most of them are shared by many pairs."""
+    axes = np.meshgrid(*[np.arange(n_side)] * D, indexing="ij")
+    X = np.stack([a.ravel() for a in axes], 1).astype(np.float32)
+    return X[rng.permutation(X.shape[0])]
+
+
+@pytest.mark.parametrize("n_side,D,K", [(6, 2, 5), (4, 3, 9), (9, 2, 13)])
+def test_ties_keep_the_smaller_index(orc, rng, n_side, D, K):
+    """One bucket with all points of a lattice: the row must be the K smallest (distance, index) pairs -- an
+    independent statement of the rule (integer arithmetic + lexsort), which a rule that keeps the first arrival, a
+    comparison on the distance alone or a reversed index comparison all fail."""
+    X = _grid_points(n_side, D, rng)
+    N = X.shape[0]
+    Xi = X.astype(np.int64)
+    d2 = ((Xi[:, None, :] - Xi[None, :, :]) ** 2).sum(-1)
+    order = np.lexsort((np.broadcast_to(np.arange(N), d2.shape), d2), axis=1)[:, :K]
+    want_i = order.astype(np.int32)
+    want_d = np.take_along_axis(d2, order, 1).astype(np.float32)
+    idx, dist = orc.init_lists(N, K)
+    orc.bucket_knn(X, K, np.arange(N, dtype=np.int32), np.array([N], np.int32), idx, dist, starts=np.array([0], np.int32))
+    si, sd = sort_rows(idx, dist)
+    assert np.array_equal(si, want_i) and np.array_equal(sd, want_d)
+
+
+def test_result_does_not_depend_on_arrival_order(orc, rng):
+    """Same buckets with their members in another order, and the trees in another order: identical rows,
+    on data where almost every distance is tied with others."""
+    X = _grid_points(7, 3, rng)                  # 343 points
+    N, K = X.shape[0], 10
+    trees = [orc.build_tree(X, K + 1, 2 * K + 2, 5000, seed) for seed in range(4)]
+    ia, da = orc.init_lists(N, K)
+    for perm, ls, lz, _ in trees:
+        orc.bucket_knn(X, K, perm, lz, ia, da, starts=ls)
+    ib, db = orc.init_lists(N, K)
+    for perm, ls, lz, _ in reversed(trees):
+        p2 = perm.copy()
+        for s, z in zip(ls, lz):
+            p2[s:s + z] = p2[s:s + z][rng.permutation(z)]
+        orc.bucket_knn(X, K, p2, lz, ib, db, starts=ls)
+    sa, sb = sort_rows(ia, da), sort_rows(ib, db)
+    assert np.array_equal(sa[0], sb[0]) and np.array_equal(sa[1], sb[1])
+    # exploration from the two (equal as sets, differently ordered) states agrees as well
+    orc.explore(X, K, ia, da)
+    orc.explore(X, K, ib, db)
+    sa, sb = sort_rows(ia, da), sort_rows(ib, db)
+    assert np.array_equal(sa[0], sb[0]) and np.array_equal(sa[1], sb[1])
+
+
+def test_infinite_distance_never_enters(orc):
+    """Coordinates so large that the squared distance overflows to +inf: such a candidate stays out of an empty
+    slot (the reference's `dist >= max` test, compute_knn_from_buckets.cu:1215)."""
+    X = np.zeros((6, 2), np.float32)
+    X[3:] = 3e19
+    idx, dist = orc.init_lists(6, 4)
+    orc.bucket_knn(X, 4, np.arange(6, dtype=np.int32), np.array([6], np.int32), idx, dist, starts=np.array([0], np.int32))
+    for p in range(6):
+        mates = {0, 1, 2} if p < 3 else {3, 4, 5}
+        assert set(idx[p][idx[p] >= 0]) == mates
+        assert not np.isin(idx[p], list({0, 1, 2, 3, 4, 5} - mates)).any()
