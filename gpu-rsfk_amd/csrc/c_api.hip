@@ -132,6 +132,12 @@ RSFK_API int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn
                              capacity, nnz, static_cast<hipStream_t>(stream));
 }
 
+RSFK_API int rsfk_symmetrize_count_noalloc(const int* d_knn_indices, int N, int num_neighbors, int drop_self,
+                                           int* d_indptr, long long* nnz, void* stream)
+{
+    return symmetrize_count_noalloc(d_knn_indices, N, num_neighbors, drop_self, d_indptr, nnz, static_cast<hipStream_t>(stream));
+}
+
 RSFK_API int rsfk_symmetrize_host(const int* knn_indices, const float* knn_sqr_distances, int N, int num_neighbors,
                                   int drop_self, int* indptr, int* indices, float* data, long long capacity, long long* nnz)
 {

@@ -65,6 +65,9 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
 // graph_export.hip
 int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int drop_self, int* d_indptr, int* d_cols,
                       float* d_vals, long long cap, long long* nnz, hipStream_t stream);
+// Count-only form of symmetrize_device (d_indptr and *nnz) whose working memory is a fixed device array of the
+// library: no allocation of any kind.  At most 2^20 points and 2^25 slots.
+int symmetrize_count_noalloc(const int* d_idx, int N, int K, int drop_self, int* d_indptr, long long* nnz, hipStream_t stream);
 int symmetrize_host(const int* idx, const float* dist, int N, int K, int drop_self, int* indptr, int* cols, float* vals,
                     long long cap, long long* nnz);
 

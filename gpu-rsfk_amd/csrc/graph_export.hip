@@ -12,6 +12,7 @@
 #include "forest.hpp"
 #include "wave64.hpp"
 #include <cstring>
+#include <mutex>
 #include <rocprim/device/device_scan.hpp>
 #include <rocprim/device/device_segmented_radix_sort.hpp>
 
@@ -203,6 +204,88 @@ int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int d
                                                  static_cast<float*>(vals.p), d_vals, (unsigned)n, (unsigned)N, d_indptr,
                                                  d_indptr + 1, 0, (unsigned)bits, stream));
     RSFK_HIP(hipStreamSynchronize(stream));
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The count-only call (row lengths, d_indptr and the number of entries) for callers that cannot allocate device memory:
+// code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Its working memory -- the edge
+// flags, the three per-point counters and the temporary storage of the prefix sum, which symmetrize_device takes from
+// the workspace pool -- lives in a file-scope device array of fixed size.  Every GPU the library runs on holds its
+// own copy of that array until the process ends; its address on a device is looked up once per device and kept.
+// All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race.
+// ---------------------------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kNaMaxPoints = 1 << 20;                     // N
+constexpr long long kNaMaxSlots = 1ll << 25;              // N * K
+constexpr size_t kNaScanBytes = (size_t)1 << 20;          // temporary storage of the prefix sum over N + 1 row lengths
+constexpr size_t kNaCounterBytes = ((sizeof(int) * ((size_t)kNaMaxPoints + 1) + 255) / 256) * 256;
+constexpr size_t kNaFlagOff = 0;
+constexpr size_t kNaOwnOff = kNaFlagOff + (size_t)kNaMaxSlots;
+constexpr size_t kNaExtraOff = kNaOwnOff + kNaCounterBytes;
+constexpr size_t kNaLenOff = kNaExtraOff + kNaCounterBytes;
+constexpr size_t kNaScanOff = kNaLenOff + kNaCounterBytes;
+constexpr size_t kNaBytes = kNaScanOff + kNaScanBytes;    // 32 MiB + 3 x 4 MiB + 1 MiB
+
+static __device__ __align__(256) unsigned char scratch[kNaBytes];
+
+constexpr int kNaMaxDevices = 64;
+unsigned char* g_scratch_ptr[kNaMaxDevices];              // device address of `scratch` on each device, once known
+std::mutex g_scratch_mutex;
+
+// The device address of the array on the current device.  The array's name is only a host-side handle.
+int scratch_on_current_device(unsigned char** out)
+{
+    int dev = -1;
+    RSFK_HIP(hipGetDevice(&dev));
+    RSFK_CHECK(dev >= 0 && dev < kNaMaxDevices, "graph export: device number out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        RSFK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        RSFK_CHECK(p != nullptr, "graph export: no device address for the working memory");
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void k_zero_counters(int* __restrict__ v, int n)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) v[i] = 0;
+}
+
+}  // namespace
+
+int symmetrize_count_noalloc(const int* d_idx, int N, int K, int drop_self, int* d_indptr, long long* nnz, hipStream_t stream)
+{
+    RSFK_CHECK(d_idx && d_indptr && nnz, "graph export: null argument");
+    RSFK_CHECK(N >= 1 && K >= 1 && K <= 256, "graph export: N must be positive and K in 1..256");
+    RSFK_CHECK(N <= kNaMaxPoints && (long long)N * K <= kNaMaxSlots,
+               "graph export without allocation: at most 2^20 points and 2^25 neighbour slots (N * K)");
+    unsigned char* base = nullptr;
+    if (scratch_on_current_device(&base)) return 1;
+    unsigned char* flag = base + kNaFlagOff;
+    int* n_own = reinterpret_cast<int*>(base + kNaOwnOff);
+    int* ext = reinterpret_cast<int*>(base + kNaExtraOff);
+    int* len = reinterpret_cast<int*>(base + kNaLenOff);
+    void* scan_tmp = base + kNaScanOff;
+    size_t tmp_bytes = 0;
+    RSFK_HIP(rocprim::exclusive_scan(nullptr, tmp_bytes, len, d_indptr, 0, (size_t)N + 1, rocprim::plus<int>(), stream));
+    RSFK_CHECK(tmp_bytes <= kNaScanBytes, "graph export without allocation: the prefix sum needs more temporary storage than reserved");
+    // the counters of the reverse edges must start at zero; the array keeps the previous call's contents
+    hipLaunchKernelGGL(k_zero_counters, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, ext, N);
+    RSFK_HIP(hipGetLastError());
+    if (sym_launch_flags(d_idx, N, K, drop_self, flag, n_own, ext, stream)) return 1;
+    hipLaunchKernelGGL(k_sym_len, dim3((unsigned)(N / 256 + 1)), dim3(256), 0, stream, n_own, ext, N, len);
+    RSFK_HIP(hipGetLastError());
+    RSFK_HIP(rocprim::exclusive_scan(scan_tmp, tmp_bytes, len, d_indptr, 0, (size_t)N + 1, rocprim::plus<int>(), stream));
+    int total = 0;
+    RSFK_HIP(hipMemcpyAsync(&total, d_indptr + N, sizeof(int), hipMemcpyDeviceToHost, stream));
+    RSFK_HIP(hipStreamSynchronize(stream));
+    *nnz = total;
     return 0;
 }
 

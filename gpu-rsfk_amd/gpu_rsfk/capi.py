@@ -22,6 +22,7 @@ SYMBOLS = {
     "rsfk_knn_ann_device": (_ci, [_ci] * 10 + [_vp, _vp, _vp, _vp, _vp, _vp]),
     "rsfk_knn_forest_fresh_host": (_ci, [_ci] * 11 + [_vp, _vp, _vp, _vp]),
     "rsfk_symmetrize_device": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp, _vp]),
+    "rsfk_symmetrize_count_noalloc": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp]),
     "rsfk_symmetrize_host": (_ci, [_vp, _vp, _ci, _ci, _ci, _vp, _vp, _vp, ctypes.c_longlong, _vp]),
     "rsfk_bucket_knn_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _ci, _ci, _vp, _vp, _vp]),
     "rsfk_explore_device": (_ci, [_vp, _ci, _ci, _ci, _vp, _vp, _vp, _vp]),
@@ -146,6 +147,15 @@ def symmetrize_device(d_idx, d_dist, N, K, drop_self, d_indptr, d_cols, d_vals, 
     _check(lib().rsfk_symmetrize_device(_vp(d_idx), _vp(d_dist) if d_dist else None, int(N), int(K), int(bool(drop_self)),
                                         _vp(d_indptr), _vp(d_cols) if d_cols else None, _vp(d_vals) if d_vals else None,
                                         int(capacity), ctypes.byref(nnz), _vp(stream)))
+    return int(nnz.value)
+
+
+def symmetrize_count_noalloc(d_idx, N, K, drop_self, d_indptr, stream=0):
+    """Row offsets and number of entries of the symmetrised graph without any allocation in the library (fixed
+    working memory: N <= 2^20, N * K <= 2^25) -> number of entries."""
+    nnz = ctypes.c_longlong(0)
+    _check(lib().rsfk_symmetrize_count_noalloc(_vp(d_idx), int(N), int(K), int(bool(drop_self)), _vp(d_indptr),
+                                               ctypes.byref(nnz), _vp(stream)))
     return int(nnz.value)
 
 

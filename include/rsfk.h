@@ -118,6 +118,17 @@ int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn_sqr_dist
                            int drop_self, int* d_indptr, int* d_indices, float* d_data, long long capacity,
                            long long* nnz, void* stream);
 
+/* The count-only form of rsfk_symmetrize_device (d_indices = d_data = NULL there): fills d_indptr (N + 1 ints) and *nnz
+ * with the row offsets and the number of entries of the symmetrised graph.  It has no counterpart in the reference.
+ * It is for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc: it calls no hipMalloc, hipFree or other allocating routine.  Its working memory
+ * (edge flags, per-point counters, the temporary storage of the prefix sum) is a fixed array of 45 MiB that every GPU
+ * the library runs on holds until the process ends.  Limits: N <= 2^20 and N * num_neighbors <= 2^25; larger inputs
+ * are refused with an error.  All calls on one GPU share the array, so calls that overlap on one GPU (other
+ * streams, other threads) race; calls on one stream, or serialised by the caller, are safe. */
+int rsfk_symmetrize_count_noalloc(const int* d_knn_indices, int N, int num_neighbors, int drop_self,
+                                  int* d_indptr, long long* nnz, void* stream);
+
 /* ---- stage-level calls with host buffers (copies in and out) ------------ */
 
 /* One tree (RSFK::create_bucket_from_sample_tree, src/rsfk.cu:500-1207).
