@@ -252,7 +252,6 @@ __global__ __launch_bounds__(256) void k_ann_leaf(const float* __restrict__ poin
     __shared__ __align__(16) float xs[kQB * kCH];
     __shared__ int cand[kCG];
     __shared__ int qid_s[kQB];
-    __shared__ int merge_scratch[4][2 * 64 * SL];             // per wavefront, for KnnRow::merge
     const int b = blockIdx.x;
     if (b >= *n_blocks) return;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -348,7 +347,7 @@ __global__ __launch_bounds__(256) void k_ann_leaf(const float* __restrict__ poin
                 const bool okv[2] = {lane < nc, two && lane + 64 < nc};
                 const int cv[2] = {c_lo, c_hi};
                 const float dv[2] = {acc0[i], acc1[i]};
-                row[i].template merge<2>(okv, cv, dv, merge_scratch[wave]);
+                row[i].template merge<2>(okv, cv, dv);
             }
         }
     }

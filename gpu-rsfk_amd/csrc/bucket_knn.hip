@@ -209,11 +209,11 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
                     row.init_from_regs(K);                            // rows that arrive unsorted are rebuilt here
                     const bool ok = lane < n_other && !(diag && lane == ci);
                     const float d = side == 0 ? L.dist[ci * kDistPitch + lane] : L.dist[lane * kDistPitch + ci];
-                    const size_t at = (size_t)id_mine[ci] * (size_t)K;
-                    const bool okv[1] = {ok};
-                    const int cv[1] = {id_other[lane]};
-                    const float dv[1] = {d};
-                    row.template merge_store<1>(okv, cv, dv, knn_idx + at, knn_dist + at);
+                    row.merge(ok, id_other[lane], d);
+                    if (row.changed) {
+                        const size_t at = (size_t)id_mine[ci] * (size_t)K;
+                        row.store(knn_idx + at, knn_dist + at);
+                    }
                     ci = ni;
 #pragma unroll
                     for (int sl = 0; sl < SL; ++sl) { ri[sl] = nri[sl]; rd[sl] = nrd[sl]; }

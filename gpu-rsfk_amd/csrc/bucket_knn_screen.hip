@@ -317,11 +317,11 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             row.idx[0] = cur_ri[u];
             row.dist[0] = cur_rd[u];
             row.init_sorted(K);
-            const size_t at = (size_t)lids[i] * (size_t)K;
-            const bool okv[1] = {lane < s && lane != i};
-            const int cv[1] = {my_id};
-            const float dv[1] = {d};
-            row.template merge_store<1>(okv, cv, dv, knn_idx + at, knn_dist + at);
+            row.merge(lane < s && lane != i, my_id, d);
+            if (row.changed) {
+                const size_t at = (size_t)lids[i] * (size_t)K;
+                row.store(knn_idx + at, knn_dist + at);
+            }
         }
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }

@@ -11,9 +11,9 @@
 //      (arithmetic of euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
 //      the 6 pairs inside each diagonal block are done one per thread;
 //   3. the distance matrix replaces the rows in LDS; a wavefront owns every second
-//      (third) point: per point, the candidates below the row's last slot are merged
-//      into the sorted row by ranking unless the row holds them already
-//      (knn_list.hpp), and only the slots that change are written; the rows of the next four points are in flight meanwhile, and
+//      (third) point: per point, the candidates below the row's last slot are
+//      inserted into the sorted row unless the row holds them already
+//      (knn_list.hpp); the rows of the next four points are in flight meanwhile, and
 //      points without any such candidate are skipped when the rows are known to be
 //      sorted.
 // Registers are kept near 100 and LDS near 20 KB per workgroup so that four
@@ -243,19 +243,19 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
             row.idx[0] = cur_ri[u];
             row.dist[0] = cur_rd[u];
             row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
-            const size_t at = (size_t)lids[i] * (size_t)K;
             if (kCap > 64) {
                 const int j2 = 64 + lane;
                 const float d2 = j2 < s ? dist[i * kDistPitch + j2] : INFINITY;
                 const bool okv[2] = {lane < s && lane != i, j2 < s && j2 != i};
                 const int cv[2] = {my_id, my_id2};
                 const float dv[2] = {d, d2};
-                row.template merge_store<2>(okv, cv, dv, knn_idx + at, knn_dist + at);
+                row.template merge<2>(okv, cv, dv);
             } else {
-                const bool okv[1] = {lane < s && lane != i};
-                const int cv[1] = {my_id};
-                const float dv[1] = {d};
-                row.template merge_store<1>(okv, cv, dv, knn_idx + at, knn_dist + at);
+                row.merge(lane < s && lane != i, my_id, d);
+            }
+            if (row.changed) {
+                const size_t at = (size_t)lids[i] * (size_t)K;
+                row.store(knn_idx + at, knn_dist + at);
             }
         }
 #pragma unroll

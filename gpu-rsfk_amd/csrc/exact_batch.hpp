@@ -89,7 +89,7 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
         if (ballot64(lane < n && acc <= tau0) == 0) break;
     }
     wave_lds_sync();
-    row.merge(lane < n, my_c, acc, reinterpret_cast<int*>(L.tile));      // the tile is free: it serves as the merge's scratch
+    row.merge(lane < n, my_c, acc);
 }
 
 }  // namespace rsfk

@@ -545,7 +545,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
             for (int s = 0; s < SL; ++s) {
                 const int c = xch[(w * 2 + 0) * (64 * SL) + lane + 64 * s];
                 const float d = __int_as_float(xch[(w * 2 + 1) * (64 * SL) + lane + 64 * s]);
-                row.merge(lane + 64 * s < K && c >= 0, c, d, region);      // the tiles are free by now
+                row.merge(lane + 64 * s < K && c >= 0, c, d);
             }
         }
         if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);

@@ -14,12 +14,16 @@
 // the smaller index.  A candidate at +inf (or NaN) never enters, as in the
 // reference.
 //
-// A row is kept sorted ascending by (distance, index), so the maximum is the last
-// slot.  A batch of up to 64 candidates per register (one per lane) is merged by
-// ranking, not by repeated insertion: for every candidate that may enter, one
-// pass counts the row slots above it (a ballot and a population count) and bumps
-// a per-slot and a per-candidate counter; afterwards every row slot and every
-// candidate knows its place in the merged row and moves there in one step.
+// The reference keeps a row unordered and rescans it for the new maximum after
+// every insertion; here a row is kept sorted ascending by (distance, index), so
+// the maximum is the last slot and an insertion is a one-lane shift of the tail
+// (DPP wave_shr:1).  The slots above a candidate form a suffix of the row, so one
+// comparison per slot gives the mask of the lanes that change, and that mask
+// shifted by one gives the lanes that take the value of the slot below: no
+// reduction and no re-reading of the maximum between the candidates of a batch.
+// (Merging a batch by ranking -- a count per candidate and per slot, then one
+// scatter -- was measured slower: about as many vector instructions per accepted
+// candidate and three times the scalar ones.)
 // Rows that arrive unsorted (anything the caller passes in) are detected on load
 // and rebuilt; rows are always written back sorted.  Slot positions are not part
 // of the interface.
@@ -34,6 +38,16 @@ __device__ __forceinline__ bool pair_above(float d1, int c1, float d2, int c2)
 {
     return d1 > d2 || (d1 == d2 && c1 > c2);
 }
+
+// Comparisons as masks over the wavefront (one bit per lane), without a boolean per lane in between.
+__device__ __forceinline__ uint64_t mask_eq_i(int a, int b) { return __builtin_amdgcn_sicmp(a, b, 32 /* eq */); }
+__device__ __forceinline__ uint64_t mask_pair_above(float d1, int c1, float d2, int c2)
+{
+    return __builtin_amdgcn_fcmpf(d1, d2, 2 /* ordered > */) |
+           (__builtin_amdgcn_fcmpf(d1, d2, 1 /* ordered == */) & __builtin_amdgcn_sicmp(c1, c2, 38 /* signed > */));
+}
+// this lane's bit of a mask
+__device__ __forceinline__ bool lane_bit(uint64_t mask) { return __builtin_amdgcn_inverse_ballot_w64(mask); }
 
 template <int SL>
 struct KnnRow {
@@ -62,28 +76,43 @@ struct KnnRow {
         return d < INFINITY && (d < tau || (d == tau && c < tau_i));
     }
 
-    // Insert (c, d) at its sorted position; the last slot falls off.  Requires enters(c, d).
-    __device__ __forceinline__ void insert_sorted(int c, float d)
+    // Insert the wave-uniform candidate (c, d), finite and not in the row, at its place; the last slot falls off.
+    // Returns false (and changes nothing) when the candidate is above the last slot.  tau / tau_i are not refreshed.
+    __device__ __forceinline__ bool insert_at_place(int c, float d)
     {
-        const int lane = lane_id();
-        float carry_d = 0.0f;
-        int carry_i = 0;
+        uint64_t above[SL];
+        uint64_t any = 0;
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
-            float sd = wave_shr1_f(dist[s]);          // lane l <- lane l-1, lane 0 <- 0
-            int si = wave_shr1_i(idx[s]);
-            if (s > 0 && lane == 0) { sd = carry_d; si = carry_i; }
-            if (s == 0 && lane == 0) si = -3;         // nothing below slot 0
-            if (s + 1 < SL) { carry_d = read_lane_f(dist[s], 63); carry_i = read_lane_i(idx[s], 63); }
-            const bool gt = pair_above(dist[s], idx[s], d, c) && lane + s * kWave < kk;   // this slot moves up (or receives the candidate)
-            const bool from_below = pair_above(sd, si, d, c);                             // the slot below moves up into this one
-            const float nd = from_below ? sd : d;
-            const int ni = from_below ? si : c;
-            dist[s] = gt ? nd : dist[s];
-            idx[s] = gt ? ni : idx[s];
+            above[s] = mask_pair_above(dist[s], idx[s], d, c);
+            const int live = kk - s * kWave;                 // slots of this register that belong to the row
+            if (live < kWave) above[s] &= live > 0 ? ((1ull << live) - 1) : 0;
+            any |= above[s];
         }
-        refresh_tau();
-        changed = true;
+        if (any == 0) return false;
+        float nd[SL];
+        int ni[SL];
+        uint64_t carry = 0;                                  // the last slot of the register below moves up too
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            const uint64_t from_below = (above[s] << 1) | carry;
+            carry = above[s] >> 63;
+            float sd = wave_shr1_f(dist[s]);                 // lane l <- lane l-1
+            int si = wave_shr1_i(idx[s]);
+            if (s > 0) {
+                const float bd = read_lane_f(dist[s - 1], 63);
+                const int bi = read_lane_i(idx[s - 1], 63);
+                sd = lane_bit(1ull) ? bd : sd;
+                si = lane_bit(1ull) ? bi : si;
+            }
+            const float md = lane_bit(from_below) ? sd : d;
+            const int mi = lane_bit(from_below) ? si : c;
+            nd[s] = lane_bit(above[s]) ? md : dist[s];
+            ni[s] = lane_bit(above[s]) ? mi : idx[s];
+        }
+#pragma unroll
+        for (int s = 0; s < SL; ++s) { dist[s] = nd[s]; idx[s] = ni[s]; }
+        return true;
     }
 
     // values already in registers and known to be sorted
@@ -116,28 +145,23 @@ struct KnnRow {
             refresh_tau();
             return;
         }
-        // rebuild by insertion into an empty row
+        // rebuild: the old entries are merged into an empty row
         int oi[SL];
         float od[SL];
+        bool okv[SL];
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
             oi[s] = idx[s];
             od[s] = dist[s];
             const bool live = lane + s * kWave < K;
+            okv[s] = live && oi[s] >= 0;
             idx[s] = live ? -1 : -2;
             dist[s] = INFINITY;
         }
         tau = INFINITY;
         tau_i = -1;
-#pragma unroll
-        for (int s = 0; s < SL; ++s) {
-            for (int l = 0; l < kWave; ++l) {
-                if (s * kWave + l >= K) break;
-                const float d = read_lane_f(od[s], l);
-                const int c = read_lane_i(oi[s], l);
-                offer<true>(c, d);
-            }
-        }
+        merge<SL>(okv, oi, od);
+        refresh_tau();
         changed = true;
     }
 
@@ -163,148 +187,41 @@ struct KnnRow {
         }
     }
 
-    // wave-uniform candidate (c, d); CHECK_DUP = the row may already hold c
-    template <bool CHECK_DUP>
-    __device__ __forceinline__ void offer(int c, float d)
-    {
-        if (!enters(c, d)) return;
-        if (CHECK_DUP) {
-            bool mine = false;
-#pragma unroll
-            for (int s = 0; s < SL; ++s) mine |= (idx[s] == c);
-            if (ballot64(mine) != 0) return;
-        }
-        insert_sorted(c, d);
-    }
-
-    // Ranks up to 64 CL candidates -- candidate u of a lane is (c[u], d[u]), there iff ok[u] -- against the row and
-    // against each other.  Result: acc[u] = lanes whose candidate u is new to the row and below its last slot;
-    // shift[s] = how many of those lie below slot (s, lane); pos[u] = place of this lane's candidate u in the merged
-    // sequence (meaningful where acc[u] has the lane's bit).  The merged sequence is cut at K by the caller.
-    // Returns false when no candidate enters.
+    // Merge a batch of up to 64 CL candidates -- candidate u of a lane is (c[u], d[u]), there iff ok[u] -- into the
+    // row.  The candidates below the last slot are taken in lane order; one that the row holds already (by index), or
+    // that is no longer below the last slot when its turn comes, is dropped.  A point may occur more than once in a
+    // batch: its second occurrence finds it in the row.
     template <int CL>
-    __device__ __forceinline__ bool rank(const bool (&ok)[CL], const int (&c)[CL], const float (&d)[CL], uint64_t (&acc)[CL],
-                                         int (&shift)[SL], int (&pos)[CL]) const
+    __device__ __forceinline__ void merge(const bool (&ok)[CL], const int (&c)[CL], const float (&d)[CL])
     {
-        uint64_t any = 0;
+        bool any_in = false;
 #pragma unroll
         for (int u = 0; u < CL; ++u) {
-            acc[u] = ballot64(ok[u] && enters(c[u], d[u]));
-            any |= acc[u];
-        }
-        if (any == 0) return false;
-        const int lane = lane_id();
-        int rr[CL];           // slots of the row below the candidate
-#pragma unroll
-        for (int s = 0; s < SL; ++s) shift[s] = 0;
-#pragma unroll
-        for (int u = 0; u < CL; ++u) { pos[u] = 0; rr[u] = 0; }
-        const bool several = CL > 1 || (any & (any - 1)) != 0;
-        int n_acc = 0;
-#pragma unroll
-        for (int u = 0; u < CL; ++u) {
-            uint64_t todo = acc[u];
+            uint64_t todo = ballot64(ok[u] && enters(c[u], d[u]));
             while (todo != 0) {
                 const int j = first_lane(todo);
                 todo &= todo - 1;
                 const float dj = read_lane_f(d[u], j);
                 const int cj = read_lane_i(c[u], j);
-                // the row holds it, or an earlier candidate of this batch is the same point
-                bool mine = false;
+                uint64_t same = 0;
 #pragma unroll
-                for (int s = 0; s < SL; ++s) mine |= (idx[s] == cj);
-                uint64_t same = ballot64(mine);
-                if (several) {
-#pragma unroll
-                    for (int u2 = 0; u2 <= u; ++u2) {
-                        const uint64_t earlier = u2 < u ? acc[u2] : (acc[u] & ((1ull << j) - 1));
-                        same |= ballot64(c[u2] == cj) & earlier;
-                    }
-                }
-                if (same != 0) {
-                    acc[u] &= ~(1ull << j);
-                    continue;
-                }
-                int above = 0;
-#pragma unroll
-                for (int s = 0; s < SL; ++s) {
-                    const bool ab = pair_above(dist[s], idx[s], dj, cj);
-                    shift[s] += ab ? 1 : 0;
-                    above += __popcll(ballot64(ab));
-                }
-                rr[u] = lane == j ? kWave * SL - above : rr[u];
-                if (several) {
-#pragma unroll
-                    for (int u2 = 0; u2 < CL; ++u2) pos[u2] += pair_above(d[u2], c[u2], dj, cj) ? 1 : 0;
-                }
-                ++n_acc;
+                for (int s = 0; s < SL; ++s) same |= mask_eq_i(idx[s], cj);
+                if (same != 0) continue;
+                if (insert_at_place(cj, dj)) any_in = true;
             }
         }
-#pragma unroll
-        for (int u = 0; u < CL; ++u) pos[u] += rr[u];
-        return n_acc > 0;
+        if (any_in) {
+            refresh_tau();
+            changed = true;
+        }
     }
 
-    // Merge a batch into the row held in registers.  scratch: 2 * 64 * SL ints of LDS that belong to this wavefront
-    // for the duration of the call (the caller orders its own earlier accesses to them with wave_lds_sync()).
-    // The candidates of one batch are distinct points or exact repeats (same index, same distance).
-    template <int CL>
-    __device__ __forceinline__ void merge(const bool (&ok)[CL], const int (&c)[CL], const float (&d)[CL], int* scratch)
-    {
-        uint64_t acc[CL];
-        int shift[SL], pos[CL];
-        if (!rank<CL>(ok, c, d, acc, shift, pos)) return;
-        const int lane = lane_id();
-        int* s_idx = scratch;
-        int* s_dist = scratch + kWave * SL;
-#pragma unroll
-        for (int s = 0; s < SL; ++s) {
-            const int k2 = lane + s * kWave + shift[s];
-            if (k2 < kk) { s_idx[k2] = idx[s]; s_dist[k2] = __float_as_int(dist[s]); }
-        }
-#pragma unroll
-        for (int u = 0; u < CL; ++u)
-            if (((acc[u] >> lane) & 1) != 0 && pos[u] < kk) { s_idx[pos[u]] = c[u]; s_dist[pos[u]] = __float_as_int(d[u]); }
-        wave_lds_sync();
-#pragma unroll
-        for (int s = 0; s < SL; ++s) {
-            const int k = lane + s * kWave;
-            if (k < kk) { idx[s] = s_idx[k]; dist[s] = __int_as_float(s_dist[k]); }
-        }
-        wave_lds_sync();
-        refresh_tau();
-        changed = true;
-    }
-
-    __device__ __forceinline__ void merge(bool ok, int c, float d, int* scratch)
+    __device__ __forceinline__ void merge(bool ok, int c, float d)
     {
         const bool okv[1] = {ok};
         const int cv[1] = {c};
         const float dv[1] = {d};
-        merge<1>(okv, cv, dv, scratch);
-    }
-
-    // Merge a batch and write the resulting row to memory; the registers are not updated (last use of the row).
-    // Only the slots that change are written, unless the row was rebuilt on load.
-    template <int CL>
-    __device__ __forceinline__ void merge_store(const bool (&ok)[CL], const int (&c)[CL], const float (&d)[CL],
-                                                int* __restrict__ gidx, float* __restrict__ gdist)
-    {
-        uint64_t acc[CL];
-        int shift[SL], pos[CL];
-        if (!rank<CL>(ok, c, d, acc, shift, pos)) {
-            if (changed) store(gidx, gdist);
-            return;
-        }
-        const int lane = lane_id();
-#pragma unroll
-        for (int s = 0; s < SL; ++s) {
-            const int k2 = lane + s * kWave + shift[s];
-            if ((shift[s] > 0 || changed) && k2 < kk) { gidx[k2] = idx[s]; gdist[k2] = dist[s]; }
-        }
-#pragma unroll
-        for (int u = 0; u < CL; ++u)
-            if (((acc[u] >> lane) & 1) != 0 && pos[u] < kk) { gidx[pos[u]] = c[u]; gdist[pos[u]] = d[u]; }
+        merge<1>(okv, cv, dv);
     }
 };
 
