@@ -4,13 +4,17 @@ A step is one complete build (forest of random-sample trees with bucket K-NN,
 then the exploration passes) on inputs that are already resident in HBM, through
 the C-ABI entry point ``rsfk_knn_forest_device``.  Default workload: BASELINE
 config 2, N=1,000,000 x D=100 uniform points, K=32, 50 trees, one exploration
-pass, buckets 33..66.  Prints one JSON line.
+pass, buckets 33..66; ``--config c1..c5`` selects any of the five.  Prints one
+JSON line.  ``host_call_seconds`` is the region the reference times
+(``RSFK._last_search_time``: host arrays in, host arrays out).
 
-The roofline object is for the bucket K-NN kernel: algorithmic bytes per launch
+The roofline object is for the bucket K-NN step: algorithmic bytes per launch
 (one launch = one tree) = N*(4D + 4 + 16K) -- every point row gathered once, every
 id read once, every K-NN row (index + distance) read once and written once --
-divided by the average duration of a launch measured with HIP events recorded on
-the launching stream inside the library (they come back in the per-tree log).
+or, where the arithmetic intensity is above the machine balance, 3 D P flops
+(P = pairs of the tree's buckets), divided by the average duration of a launch
+measured with HIP events recorded on the launching stream inside the library
+(they come back in the per-tree log).
 """
 import argparse
 import json
@@ -200,11 +204,50 @@ def bench_graph(args):
     print(json.dumps(out))
 
 
+# The benchmark configurations: (workload, N, D, K, trees, min, max, exploration passes)
+CONFIGS = {
+    "c1": ("uniform", 10000, 32, 16, 4, 32, 128, 1),
+    "c2": ("uniform", 1000000, 100, 32, 50, 33, 66, 1),
+    "c3": ("gmm64", 1000000, 256, 32, 20, 33, 66, 1),
+    "c4": ("sparse", 70000, 784, 90, 10, 91, 182, 1),
+    "c5": ("normal", 10000000, 32, 32, 10, 64, 256, 1),
+}
+FP32_PEAK_TFLOPS = 157.3
+
+
+def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
+    """Roofline object of the bucket K-NN step of one tree (one step of the forest loop = one tree's launches).
+
+    Bytes: N (4D + 4 + 16K) per tree.  Flops: 3 D P with P = pairs of the tree's buckets, estimated from the number of
+    buckets L the run reported as N (N / L - 1) / 2 (equal buckets: a lower bound of the true sum).  The bound is the
+    one the workload's arithmetic intensity selects: fp32 when flops / bytes exceeds peak flops / peak bandwidth."""
+    alg_bytes = float(N) * (4 * D + 4 + 16 * K)
+    mean_leaves = float(np.mean(leaf_counts)) if len(leaf_counts) else max(1.0, N / (0.75 * mx))
+    pairs = 0.5 * N * (N / mean_leaves - 1.0)
+    alg_flops = 3.0 * D * pairs
+    balance = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+    small = K <= 64 and mx <= 72
+    kernel = ("k_bucket_knn_small / k_bucket_knn_gram (buckets <= 64) + k_bucket_knn_small<72> (65..72)" if small
+              else "k_bucket_knn / k_bucket_knn_gram (64 x 64 tiles of the pair matrix)")
+    if alg_flops / alg_bytes > balance:
+        ach = alg_flops / knn_s / 1e12 if knn_s > 0 else 0.0
+        return {"kernel": kernel, "bound": "mfma", "achieved": round(ach, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / FP32_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops_per_launch": alg_flops,
+                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4), "launches_per_step": T,
+                "note": "flops = 3 D P of the direct-difference path (fp32 peak 157.3 TFLOP/s); HBM traffic: see profiles/"}
+    ach = alg_bytes / knn_s / 1e9 if knn_s > 0 else 0.0
+    return {"kernel": kernel, "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_launch": alg_bytes,
+            "algorithmic_flops_per_launch": alg_flops, "avg_launch_ms": round(knn_s * 1e3, 4), "launches_per_step": T,
+            "note": "traffic (HBM bytes per launch from FETCH_SIZE / WRITE_SIZE) is not measured by this run: see profiles/"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS), help="one of the benchmark configurations (sets the shape flags)")
     ap.add_argument("--n", type=int, default=1000000)
     ap.add_argument("--d", type=int, default=100)
     ap.add_argument("--k", type=int, default=32)
@@ -214,19 +257,29 @@ def main():
     ap.add_argument("--max-children", type=int, default=-1)
     ap.add_argument("--workload", default="uniform", choices=["uniform", "normal", "gmm64", "sparse"])
     ap.add_argument("--recall-queries", type=int, default=10000)
-    ap.add_argument("--cpu-sample", type=int, default=200000, help="rows of the workload the CPU baseline runs on (0 = skip)")
+    ap.add_argument("--cpu-sample", type=int, default=-1,
+                    help="rows of the workload the CPU baseline runs on (0 = skip; default: what about 30 s of CPU time cover, the whole workload if that suffices)")
+    ap.add_argument("--cpu-full", action="store_true", help="CPU baseline on the whole workload (minutes at the large configurations)")
+    ap.add_argument("--host-calls", type=int, default=2, help="timed calls of RSFK.find_nearest_neighbors (host buffers in and out)")
     ap.add_argument("--path", default="knng", choices=["knng", "ann", "graph"],
                     help="knng = K-NN-graph build (the headline metric); ann = query-set search; graph = CSR export")
     ap.add_argument("--queries", type=int, default=-1, help="query points of --path ann (default: as many as points)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on one GPU only (--gpus 1); nothing here uses a second GPU")
+    if args.config:
+        args.workload, args.n, args.d, args.k, args.trees, args.min_children, args.max_children, args.explore = CONFIGS[args.config]
     if args.path == "ann":
+        if args.cpu_sample < 0:
+            args.cpu_sample = 100000
         return bench_ann(args)
     if args.path == "graph":
+        if args.cpu_sample < 0:
+            args.cpu_sample = 1
         return bench_graph(args)
 
     import torch
+    import gpu_rsfk
     from gpu_rsfk import capi
     from gpu_rsfk.RSFK import ForestLog
 
@@ -275,28 +328,37 @@ def main():
     hits = (approx[:, :, None] == truth[:, None, :]).any(2).sum().item()
     recall = hits / float(nq * K)
 
-    # roofline of the bucket K-NN kernel
+    # the call the reference times (python/gpu_rsfk/RSFK.py:329,368: host arrays in, host arrays out)
+    host_s = None
+    if args.host_calls > 0:
+        r = gpu_rsfk.RSFK(random_state=0)
+        ts = []
+        for _ in range(args.host_calls):
+            r.find_nearest_neighbors(X, K, n_trees=T, min_tree_children=mn, max_tree_children=mx,
+                                     nn_exploring_factor=args.explore)
+            ts.append(r._last_search_time)
+        host_s = float(min(ts))
+
     fls = [ForestLog(l) for l in logs]
     knn_s = float(np.mean([np.mean(f.data["KNN Sets Updates"]) for f in fls])) if fls and T > 0 else 0.0
     tree_s = float(np.mean([np.mean(f.data["Total Tree Building Time"]) for f in fls])) if fls and T > 0 else 0.0
     expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
-    alg_bytes = float(N) * (4 * D + 4 + 16 * K)
-    achieved = alg_bytes / knn_s / 1e9 if knn_s > 0 else 0.0
-    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload, each scaled by
-    # what the same counter reads for a plain copy of known size (FETCH x2.0, WRITE x1.0); only known for the
-    # default workload
-    default_workload = (args.workload == "uniform" and (N, D, K) == (1000000, 100, 32) and (mn, mx) == (33, 66))
-    traffic = 1.13e9 if default_workload else None
-    roofline = {"kernel": "k_bucket_knn_small (buckets <= 64 and 65..72)", "bound": "hbm", "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4),
-                "launches_per_step": T}
+    leaves = fls[0].data["Total Leaves"] if fls and T > 0 else []
+    roofline = bucket_roofline(N, D, K, T, mn, mx, knn_s, leaves)
 
-    # CPU baseline: the oracle (a port of the reference algorithm) on a bounded sample
+    # CPU baseline: the oracle (a port of the reference algorithm, OpenMP) on the same workload -- whole with
+    # --cpu-full, else on its first rows, as many as about 30 s of CPU time cover (the rate per point of a smaller
+    # input is higher: shallower trees, same work per bucket)
     cpu = None
-    if args.cpu_sample > 0:
+    if args.cpu_sample != 0:
         from oracle import rsfk_oracle as orc
-        ns = min(args.cpu_sample, N)
+        if args.cpu_full:
+            ns = N
+        elif args.cpu_sample > 0:
+            ns = min(args.cpu_sample, N)
+        else:
+            per_point = T * (D * (0.75 * mx) * 1.5 + 40.0 * D) + args.explore * K * K * D * 0.6      # rough flop count
+            ns = int(min(N, max(20000, 35.0 * 1.2e9 * orc.num_threads() / per_point)))
         Xs = np.ascontiguousarray(X[:ns])
         oi, od = orc.init_lists(ns, K)
         c0 = time.perf_counter()
@@ -304,7 +366,8 @@ def main():
         cs = time.perf_counter() - c0
         cpu = {"value": round(ns / cs, 1), "unit": "points/s", "cores": orc.num_threads(), "kind": "port",
                "seconds": round(cs, 3),
-               "sample": "first %d rows of the same workload, same D, K, %d trees, %d exploration pass(es), OpenMP" % (ns, T, args.explore)}
+               "sample": ("the whole workload" if ns == N else "first %d rows of the workload" % ns) +
+                         ", same D, K, %d trees, %d exploration pass(es), OpenMP with %d threads" % (T, args.explore, orc.num_threads())}
 
     out = {
         "metric": "knng_build_points_per_sec",
@@ -319,9 +382,11 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "%s N=%d D=%d K=%d n_trees=%d buckets=%d..%d exploration=%d seed=0" % (
-            args.workload, N, D, K, T, mn, mx, args.explore)},
+        "config": {"workload": "%s%s N=%d D=%d K=%d n_trees=%d buckets=%d..%d exploration=%d seed=0" % (
+            (args.config + " = ") if args.config else "", args.workload, N, D, K, T, mn, mx, args.explore)},
         "build_seconds": round(sec_per_step, 5),
+        "host_call_seconds": None if host_s is None else round(host_s, 5),
+        "host_call_points_per_sec": None if host_s is None else round(N / host_s, 1),
         "recall_at_k": round(recall, 4),
         "recall_queries": nq,
         "phase_seconds": {"tree_build_per_tree": round(tree_s, 6), "bucket_knn_per_tree": round(knn_s, 6),

@@ -24,6 +24,8 @@
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
 #include "forest.hpp"
+#include <algorithm>
+#include <cstdlib>
 
 namespace rsfk {
 
@@ -246,16 +248,66 @@ int launch_general(const float* points, int D, int K, const int* ids, const int*
 
 }  // namespace
 
+namespace {
+
+__global__ __launch_bounds__(256) void k_max_size(const int* __restrict__ sizes, int n, int* __restrict__ out)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    int v = i < n ? sizes[i] : 0;
+    v = max(v, __shfl_xor(v, 32, 64));
+    v = max(v, __shfl_xor(v, 16, 64));
+    v = max(v, __shfl_xor(v, 8, 64));
+    v = max(v, __shfl_xor(v, 4, 64));
+    v = max(v, __shfl_xor(v, 2, 64));
+    v = max(v, __shfl_xor(v, 1, 64));
+    if ((threadIdx.x & 63) == 0 && v > 0) atomicMax(out, v);
+}
+
+// size of the largest bucket of a table in device memory (one trip to the host)
+int largest_bucket(const int* sizes, int n, hipStream_t stream, int* out)
+{
+    void* d = nullptr;
+    if (ws_alloc(&d, sizeof(int))) return 1;
+    int v = 0;
+    hipError_t e = hipMemcpyAsync(d, &v, sizeof(int), hipMemcpyHostToDevice, stream);
+    if (e == hipSuccess) {
+        hipLaunchKernelGGL(k_max_size, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, sizes, n, static_cast<int*>(d));
+        e = hipMemcpyAsync(&v, d, sizeof(int), hipMemcpyDeviceToHost, stream);
+    }
+    if (e == hipSuccess) e = hipStreamSynchronize(stream);
+    ws_free(d);
+    if (e != hipSuccess) { set_last_error(std::string("largest bucket: ") + hipGetErrorString(e)); return 1; }
+    *out = v;
+    return 0;
+}
+
+}  // namespace
+
+int bucket_gram_from()
+{
+    // Off unless asked for: on the shapes measured so far (bucket sizes 33..256, D 32..784, K 32 and 90) the direct
+    // kernels are faster -- their time goes into the merges and the waits between phases, not into the fp32 chains
+    // the screen saves.
+    const char* e = std::getenv("RSFK_GRAM_FROM");
+    if (e && *e) return std::max(0, std::atoi(e));
+    return 0x7fffffff;
+}
+
 // Host launcher for an arbitrary list of buckets.  All pointers are device pointers.  max_bucket: size of
 // the largest bucket if known, otherwise -1.
 int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
                       const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream)
 {
-    (void)N;
     if (n_buckets <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    if (bucket_gram_from() == 0) {
+        // RSFK_GRAM_FROM=0: the screened kernel for every call; it needs sorted rows and the size of the largest bucket
+        if (launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
+        if (max_bucket < 0 && largest_bucket(sizes, n_buckets, stream, &max_bucket)) return 1;
+        return launch_bucket_knn_gram(points, D, K, ids, starts, sizes, n_buckets, stride, 2, max_bucket, knn_idx, knn_dist, stream);
+    }
     int skip_upto = 0;
     if (K <= 64) {
         // buckets of up to 72 points go to the specialised kernels; the general one skips them
@@ -275,12 +327,30 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // known to be sorted by distance.  bf: bfloat16 copy of the points to send the small buckets to the screened kernel
 // (needs sorted rows), else null.  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
 // kinds touch different rows, so the two parts of one tree may run side by side).
-int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
+int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
                            int* knn_idx, float* knn_dist, hipStream_t stream, int part)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    if (gram && rows_sorted) {
+        // pair matrix screened on the matrix cores; buckets of 65..72 points (K <= 64) keep their own kernel
+        if (n_small > 0 && part != 2 &&
+            launch_bucket_knn_gram(points, D, K, ids, starts, sizes, n_small, 0, 2, kBucketSplit, knn_idx, knn_dist, stream))
+            return 1;
+        if (n_big <= 0 || part == 1) return 0;
+        const int off = leaf_cap - n_big;
+        int from = kBucketSplit + 1;
+        if (K <= 64) {
+            if (launch_bucket_knn_medium(points, D, K, ids, starts + off, sizes + off, n_big, 0, rows_sorted, knn_idx, knn_dist, stream))
+                return 1;
+            if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
+            from = medium_bucket_cap() + 1;
+        }
+        if (max_bucket < 0 && largest_bucket(sizes + off, n_big, stream, &max_bucket)) return 1;
+        return launch_bucket_knn_gram(points, D, K, ids, starts + off, sizes + off, n_big, 0, from, max_bucket, knn_idx, knn_dist,
+                                      stream);
+    }
     if (n_small > 0 && part != 2) {
         if (K <= 64 && bf != nullptr && rows_sorted) {
             if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;

@@ -149,6 +149,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
         for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        const int gram_from = bucket_gram_from();
         SideStream sync;
         if (std::getenv("RSFK_KNN_ONE_STREAM") == nullptr && sync.open()) return 1;
         int rc = 0;
@@ -172,11 +173,12 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                     (void)hipEventRecord(sync.start, stream);                    // everything before this tree
                     (void)hipStreamWaitEvent(sync.side, sync.start, 0);
                 }
-                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                const bool gram = t0 + j >= gram_from;
+                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
                                             d_idx, d_dist, stream, split ? 1 : 0);
                 if (!rc && split) {
-                    rc = launch_bucket_knn_tree(d_points, nullptr, true, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                    rc = launch_bucket_knn_tree(d_points, nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
                                                 stats[5 * j + 2], d_idx, d_dist, sync.side, 2);
                     (void)hipEventRecord(sync.big, sync.side);

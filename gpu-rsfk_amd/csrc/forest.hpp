@@ -28,7 +28,14 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       const int* sizes, int n_buckets, int stride, int max_bucket, int* knn_idx, float* knn_dist,
                       hipStream_t stream);
 
-int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, int D, int K, const int* ids,
+// bucket_knn_gram.hip
+int launch_bucket_knn_gram(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int n_buckets, int stride, int min_size, int max_size, int* knn_idx, float* knn_dist,
+                           hipStream_t stream);
+// trees from this index on take the kernel that screens the pair matrix on the matrix cores (RSFK_GRAM_FROM)
+int bucket_gram_from();
+
+int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
                            int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0);
 

@@ -86,7 +86,12 @@ def test_tree_edge_cases(gpu, orc, rng):
     (1200, 1, 4, 5, 10), (2500, 3, 1, 2, 4), (2000, 130, 64, 65, 130), (1500, 20, 65, 66, 140),
     (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
 ])
-def test_bucket_knn_matches_oracle(gpu, orc, rng, N, D, K, MIN, MAX):
+@pytest.mark.parametrize("kernel", ["direct", "gram"])
+def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
+    """kernel: "direct" = fp32 chains for every pair; "gram" = the kernel that bounds the pair matrix on the matrix
+    cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0)."""
+    if kernel == "gram":
+        monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K)
     gi, gd = orc.init_lists(N, K)
@@ -240,8 +245,11 @@ def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D,
     ("c4", 9000, 90, 4, dict(nn_exploring_factor=1)),
     ("c5", 70000, 32, 5, dict(min_tree_children=64, max_tree_children=256)),
 ], ids=["config3_gmm64_d256_k32", "config4_sparse_d784_k90_explore", "config5_normal_d32_buckets64_256"])
-def test_baseline_config_workloads_match_oracle(gpu, orc, config, N, K, T, kw):
+@pytest.mark.parametrize("kernel", ["direct", "gram"])
+def test_baseline_config_workloads_match_oracle(gpu, orc, monkeypatch, config, N, K, T, kw, kernel):
     import gpu_rsfk
+    if kernel == "gram":
+        monkeypatch.setenv("RSFK_GRAM_FROM", "1")          # every tree but the first through the screened bucket kernel
     X = baseline_points(config, N)
     r = gpu_rsfk.RSFK(random_state=0)
     _say("forest", config, N, X.shape[1], K, T, kw)
@@ -434,15 +442,18 @@ def _hard_inputs(rng, kind, N, D):
     raise ValueError(kind)
 
 
-@pytest.mark.parametrize("variant", ["default", "bucket_screen"])
+@pytest.mark.parametrize("variant", ["default", "bucket_screen", "bucket_gram"])
 @pytest.mark.parametrize("kind", ["offset", "grid", "tiny", "mixed", "clusters"])
 def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant):
     """The bfloat16 screens only skip work whose outcome is certain: trees, bucket K-NN and exploration on inputs
     that defeat a 8-bit mantissa must still be identical to the fp32 oracle.  "bucket_screen" also switches the
-    small buckets to the kernel that screens pairs with the matrix cores (RSFK_BUCKET_SCREEN=1)."""
+    small buckets to the kernel that screens pairs with the matrix cores on the bfloat16 copy (RSFK_BUCKET_SCREEN=1),
+    "bucket_gram" all buckets to the one that splits the fp32 rows into two bfloat16 numbers (RSFK_GRAM_FROM=0)."""
     import gpu_rsfk
     if variant == "bucket_screen":
         monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
+    if variant == "bucket_gram":
+        monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     N, D, K = 6000, 24, 10
     X = _hard_inputs(rng, kind, N, D)
     perm, ls, lz, st = orc.build_tree(X, K + 1, 2 * (K + 1), 300, 2)
