@@ -6,10 +6,13 @@
 //   1. the rows of the bucket, 64 dimensions at a time, are requested from HBM at
 //      once and written to LDS; a row is read by consecutive lanes, 16 bytes each
 //      (coalesced);
-//   2. each thread owns one 4x4 block of the upper triangle of the pair matrix and
-//      accumulates its 16 distances with sequential fused multiply-add chains
-//      (arithmetic of euclidean_distance_sqr, compute_knn_from_buckets.cu:40-54);
-//      the 6 pairs inside each diagonal block are done one per thread;
+//   2. the pair matrix is cut into 2x2 blocks (members 2a, 2a+1 against 2b, 2b+1);
+//      the blocks of the upper triangle are dealt out to the threads round by round
+//      and a thread accumulates the 4 distances of a block with sequential fused
+//      multiply-add chains (arithmetic of euclidean_distance_sqr,
+//      compute_knn_from_buckets.cu:40-54).  Small blocks keep the lanes busy whatever
+//      the bucket size: a bucket of 50 points has 325 blocks = 3 rounds of 128 threads,
+//      where one 4x4 block per thread left 50 of 128 lanes idle for 16 distances;
 //   3. the distance matrix replaces the rows in LDS; a wavefront owns every second
 //      (third) point: per point, the candidates below the row's last slot are
 //      inserted into the sorted row unless the row holds them already
@@ -30,19 +33,18 @@ namespace {
 
 constexpr int kMaxChunk = 64;               // dimensions staged at once
 
-// CAP = largest bucket, THREADS = workgroup size (one 4x4 block of the pair matrix per thread must do),
-// SPACING = LDS rows between members 4t, 4t+1, 4t+2, 4t+3: the 4x4 block of thread t reads rows t, t+SPACING,
-// t+2 SPACING, t+3 SPACING -- consecutive t give conflict-free 16-byte reads (the pitch is an odd number of
-// 16-byte units) and the four rows of one block fall in different banks.
+// CAP = largest bucket, THREADS = workgroup size, SPACING = LDS rows between members 2t and 2t+1: the 2x2 block
+// (a, b) reads rows a, a + SPACING, b, b + SPACING -- consecutive a (consecutive threads) give conflict-free 16-byte
+// reads (the pitch is an odd number of 16-byte units).
 template <int CAP, int THREADS, int SPACING>
 struct SmallCfg {
     static constexpr int kWaves = THREADS / 64;
-    static constexpr int kBlocks = CAP / 4;
-    static constexpr int kLdsRows = (kBlocks - 1) + 3 * SPACING + 1;
+    static constexpr int kBlocks = CAP / 2;
+    static constexpr int kLdsRows = (kBlocks - 1) + SPACING + 1;
     static constexpr int kDistPitch = CAP + 1;
     static constexpr int kMaxLoads = (CAP * (kMaxChunk / 4) + THREADS - 1) / THREADS;   // 16-byte loads per thread and chunk
-    static_assert(CAP % 4 == 0 && CAP <= 128 && THREADS % 64 == 0 && THREADS >= CAP, "shape");
-    static_assert(kBlocks * (kBlocks - 1) / 2 <= THREADS && 6 * kBlocks <= THREADS, "one block of the pair matrix per thread");
+    static constexpr int kMaxRounds = (kBlocks * (kBlocks + 1) / 2 + THREADS - 1) / THREADS;  // 2x2 blocks per thread
+    static_assert(CAP % 2 == 0 && CAP <= 128 && THREADS % 64 == 0 && THREADS >= CAP, "shape");
     static_assert(SPACING >= kBlocks, "LDS rows of different members must not collide");
     static_assert((CAP + kWaves - 1) / kWaves <= 32, "members of a wavefront must fit a 32-bit mask");
 };
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
     using Cfg = SmallCfg<CAP, THREADS, SPACING>;
     constexpr int kCap = CAP, kThreads = THREADS, kWaves = Cfg::kWaves, kSpacing = SPACING;
     constexpr int kDistPitch = Cfg::kDistPitch, kMaxLoads = Cfg::kMaxLoads;
-    auto phys_row = [](int m) { return (m >> 2) + kSpacing * (m & 3); };     // LDS row of bucket member m
+    auto phys_row = [](int m) { return (m >> 1) + kSpacing * (m & 1); };     // LDS row of bucket member m
     // dynamic LDS: [rows | dist] (region_floats) | ids[64] | tau[64] | flag[64]
     extern __shared__ __align__(16) float lds_f[];
     float* rows = lds_f;
@@ -85,27 +87,30 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
     }
     __syncthreads();
 
-    // work assignment: off-diagonal 4x4 blocks (ti < tj) one per thread, then the 6 pairs of each diagonal block
-    const int n = (s + 3) >> 2;
-    const int noff = n * (n - 1) / 2;
-    int ti = 0, tj = 0;
-    const bool has_tile = tid < noff;
-    if (has_tile) {
-        int rem = tid;
-        while (rem >= n - 1 - ti) { rem -= n - 1 - ti; ++ti; }
-        tj = ti + 1 + rem;
-    }
-    const bool has_diag = tid < 6 * n;
-    const int dt = tid / 6, dq = tid - 6 * dt;
-    const int dr = dq < 3 ? 0 : (dq < 5 ? 1 : 2);
-    const int dc = dq < 3 ? dq + 1 : (dq < 5 ? dq - 1 : 3);
-
-    float acc[4][4];
+    // work assignment.  With n2 blocks of two members, the unordered block pairs (a, b) are (a, (a + o) mod n2) for
+    // the offsets o = 0 .. (n2 - 1) / 2 and all a, plus o = n2 / 2 with a < n2 / 2 when n2 is even: block pair number
+    // k = o n2 + a, k < n_tiles.  Thread t takes k = t, t + THREADS, ...
+    constexpr int kMaxRounds = Cfg::kMaxRounds;
+    const int n2 = (s + 1) >> 1;
+    const int n_tiles = n2 * (((n2 - 1) >> 1) + 1) + ((n2 & 1) ? 0 : (n2 >> 1));
+    const int rounds = (n_tiles + kThreads - 1) / kThreads;            // at most kMaxRounds
+    const float inv_n2 = 1.0f / (float)n2;
+    int tile_ab[kMaxRounds];                                           // a | b << 8, or -1
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < kMaxRounds; ++r) {
+        const int k = tid + r * kThreads;
+        // k / n2 (exact: k < 1024 and (k + 0.5) / n2 is never within 1 / 128 of an integer)
+        const int o = (int)(((float)k + 0.5f) * inv_n2);
+        const int a = k - o * n2;
+        int bb = a + o;
+        if (bb >= n2) bb -= n2;
+        tile_ab[r] = k < n_tiles ? (a | (bb << 8)) : -1;
+    }
+    float acc[kMaxRounds][4];
+#pragma unroll
+    for (int r = 0; r < kMaxRounds; ++r)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
-    float dacc = 0.0f;
 
     for (int d0 = 0; d0 < D; d0 += chunk) {
         const int np = min(chunk, (D - d0 + 3) & ~3) >> 2;      // 16-byte pieces per row in this chunk
@@ -140,38 +145,28 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
             }
         }
         __syncthreads();
-        if (has_tile) {
-            const float* ra = &rows[ti * pitch];
-            const float* rb = &rows[tj * pitch];
-            for (int q = 0; q < np; ++q) {
-                float4 av[4], bv[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) av[r] = *reinterpret_cast<const float4*>(ra + kSpacing * r * pitch + 4 * q);
+        for (int r = 0; r < kMaxRounds; ++r) {
+            if (r < rounds && tile_ab[r] >= 0) {
+                const float* ra = &rows[(tile_ab[r] & 255) * pitch];
+                const float* rb = &rows[(tile_ab[r] >> 8) * pitch];
+                for (int q = 0; q < np; ++q) {
+                    float4 av[2], bv[2];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) bv[c] = *reinterpret_cast<const float4*>(rb + kSpacing * c * pitch + 4 * q);
+                    for (int x = 0; x < 2; ++x) av[x] = *reinterpret_cast<const float4*>(ra + kSpacing * x * pitch + 4 * q);
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
+                    for (int y = 0; y < 2; ++y) bv[y] = *reinterpret_cast<const float4*>(rb + kSpacing * y * pitch + 4 * q);
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        float df;
-                        df = av[r].x - bv[c].x; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
-                        df = av[r].y - bv[c].y; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
-                        df = av[r].z - bv[c].z; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
-                        df = av[r].w - bv[c].w; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
-                    }
-            }
-        }
-        if (has_diag) {
-            const float* ra = &rows[(dt + kSpacing * dr) * pitch];
-            const float* rb = &rows[(dt + kSpacing * dc) * pitch];
-            for (int q = 0; q < np; ++q) {
-                const float4 a = *reinterpret_cast<const float4*>(ra + 4 * q);
-                const float4 b = *reinterpret_cast<const float4*>(rb + 4 * q);
-                float df;
-                df = a.x - b.x; dacc = __builtin_fmaf(df, df, dacc);
-                df = a.y - b.y; dacc = __builtin_fmaf(df, df, dacc);
-                df = a.z - b.z; dacc = __builtin_fmaf(df, df, dacc);
-                df = a.w - b.w; dacc = __builtin_fmaf(df, df, dacc);
+                    for (int x = 0; x < 2; ++x)
+#pragma unroll
+                        for (int y = 0; y < 2; ++y) {
+                            float df;
+                            df = av[x].x - bv[y].x; acc[r][2 * x + y] = __builtin_fmaf(df, df, acc[r][2 * x + y]);
+                            df = av[x].y - bv[y].y; acc[r][2 * x + y] = __builtin_fmaf(df, df, acc[r][2 * x + y]);
+                            df = av[x].z - bv[y].z; acc[r][2 * x + y] = __builtin_fmaf(df, df, acc[r][2 * x + y]);
+                            df = av[x].w - bv[y].w; acc[r][2 * x + y] = __builtin_fmaf(df, df, acc[r][2 * x + y]);
+                        }
+                }
             }
         }
     }
@@ -182,18 +177,19 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
         if (d <= tau[i]) flag[i] = 1;            // plain stores of the same value: no ordering needed
         if (d <= tau[j]) flag[j] = 1;
     };
-    if (has_tile) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
+    for (int r = 0; r < kMaxRounds; ++r) {
+        if (r < rounds && tile_ab[r] >= 0) {
+            const int a = tile_ab[r] & 255, bb = tile_ab[r] >> 8;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int i = 4 * ti + r, j = 4 * tj + c;
-                if (i < s && j < s) put(i, j, acc[r][c]);
-            }
-    }
-    if (has_diag) {
-        const int i = 4 * dt + dr, j = 4 * dt + dc;
-        if (j < s) put(i, j, dacc);
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int y = 0; y < 2; ++y) {
+                    const int i = 2 * a + x, j = 2 * bb + y;
+                    // a block on the diagonal holds one pair of distinct members
+                    if (i < s && j < s && (a != bb || (x == 0 && y == 1))) put(i, j, acc[r][2 * x + y]);
+                }
+        }
     }
 
     __syncthreads();                           // distance matrix complete
@@ -299,7 +295,7 @@ int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, c
 {
     if (n_buckets <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
-    return launch_cfg<64, 128, 17>(points, D, K, ids, starts, sizes, n_buckets, stride, 2, rows_sorted, knn_idx, knn_dist,
+    return launch_cfg<64, 128, 33>(points, D, K, ids, starts, sizes, n_buckets, stride, 2, rows_sorted, knn_idx, knn_dist,
                                    stream);
 }
 
@@ -309,7 +305,7 @@ int launch_bucket_knn_medium(const float* points, int D, int K, const int* ids, 
 {
     if (n_buckets <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 64, "small-bucket kernel: K must be in 1..64");
-    return launch_cfg<72, 192, 19>(points, D, K, ids, starts, sizes, n_buckets, stride, 65, rows_sorted, knn_idx, knn_dist,
+    return launch_cfg<72, 192, 37>(points, D, K, ids, starts, sizes, n_buckets, stride, 65, rows_sorted, knn_idx, knn_dist,
                                    stream);
 }
 
