@@ -227,8 +227,11 @@ def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
     alg_flops = 3.0 * D * pairs
     balance = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
     small = K <= 64 and mx <= 72
-    kernel = ("k_bucket_knn_small / k_bucket_knn_gram (buckets <= 64) + k_bucket_knn_small<72> (65..72)" if small
-              else "k_bucket_knn / k_bucket_knn_gram (64 x 64 tiles of the pair matrix)")
+    gram = os.environ.get("RSFK_GRAM_FROM")
+    kernel = ("k_bucket_knn_small<64> (buckets <= 64) + k_bucket_knn_small<72> (65..72)" if small
+              else "k_bucket_knn (64 x 64 tiles of the pair matrix)" + ("" if mx <= 72 or K > 64 else " + k_bucket_knn_small for the buckets up to 72 points"))
+    if gram is not None:
+        kernel += "; k_bucket_knn_gram from tree %s on (RSFK_GRAM_FROM)" % gram
     if alg_flops / alg_bytes > balance:
         ach = alg_flops / knn_s / 1e12 if knn_s > 0 else 0.0
         return {"kernel": kernel, "bound": "mfma", "achieved": round(ach, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",

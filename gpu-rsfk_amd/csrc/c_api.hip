@@ -276,7 +276,11 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
 
 RSFK_API const char* rsfk_last_error(void) { return last_error(); }
 
-RSFK_API void rsfk_release_workspace(void) { ws_release_all(); }
+RSFK_API void rsfk_release_workspace(void)
+{
+    ws_release_all();
+    release_copy_buffers();
+}
 
 RSFK_API int rsfk_device_count(void)
 {

@@ -91,8 +91,24 @@ struct Q8Guard {
     Q8Copy c;
     ~Q8Guard() { q8_copy_free(&c); }
 };
+// start / stop events of one tree's K-NN update; released when the owner goes out of scope, on every path
 struct EventPair {
     hipEvent_t a = nullptr, b = nullptr;
+    EventPair() = default;
+    EventPair(const EventPair&) = delete;
+    EventPair& operator=(const EventPair&) = delete;
+    EventPair(EventPair&& o) noexcept : a(o.a), b(o.b) { o.a = nullptr; o.b = nullptr; }
+    int create()
+    {
+        RSFK_HIP(hipEventCreate(&a));
+        RSFK_HIP(hipEventCreate(&b));
+        return 0;
+    }
+    ~EventPair()
+    {
+        if (a) (void)hipEventDestroy(a);
+        if (b) (void)hipEventDestroy(b);
+    }
 };
 
 // Side tests of the trees are screened on the 8-bit copy when its quantisation error is within a small factor
@@ -125,6 +141,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     RSFK_CHECK(n_trees >= 0, "forest: n_trees must not be negative");
     RSFK_CHECK(K <= 256, "forest: K above 256 is not supported");
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
+    if (n_trees == 0 && nnef <= 0) return 0;          // nothing to do: no copies are made, nothing is queued
     const double t_forest0 = now_s();
     Bf16Guard bf;
     if (bf16_copy_alloc(&bf.c, N, D)) return 1;
@@ -148,7 +165,8 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
         std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
-        for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        for (auto& e : ev)
+            if (e.create()) return 1;
         const int gram_from = bucket_gram_from();
         SideStream sync;
         if (std::getenv("RSFK_KNN_ONE_STREAM") == nullptr && sync.open()) return 1;
@@ -199,6 +217,12 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                     log_forest[(size_t)2 * n_trees + t] = (float)stats[5 * j + 3];   // Min Leaf Size
                     log_forest[(size_t)3 * n_trees + t] = (float)stats[5 * j + 0];   // Total Leaves
                     log_forest[(size_t)5 * n_trees + t] = (float)(tb / nb);          // Total Tree Building Time
+                    // the trees of a batch are built together, level by level: a tree's share of the batch's kernels
+                    const float* ph = tree_ws_phase_seconds(ws.w);
+                    log_forest[(size_t)7 * n_trees + t] = ph[0] / nb;                // Check Points Side Time (k_side)
+                    log_forest[(size_t)11 * n_trees + t] = ph[1] / nb;               // Create Nodes Time (k_level_planes)
+                    log_forest[(size_t)12 * n_trees + t] = ph[2] / nb;               // Update Nodes Time (k_scatter)
+                    log_forest[(size_t)13 * n_trees + t] = ph[3] / nb;               // Bucket Creation Time (k_tail)
                     log_forest[(size_t)15 * n_trees + t] = ms * 1e-3f;               // KNN Sets Updates
                 }
                 if (verbose >= 2)
@@ -206,7 +230,6 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                                 stats[5 * j + 1], stats[5 * j + 0], stats[5 * j + 3], stats[5 * j + 2], ms * 1e-3);
             }
         }
-        for (auto& e : ev) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
         if (rc) return rc;
     }
     const double t_forest = now_s() - t_forest0;
@@ -269,7 +292,8 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
         if (ws_alloc(&planes.p, sizeof(float) * (size_t)rec_cap * (size_t)ann_plane_pitch(D))) return 1;
         std::vector<int> stats((size_t)5 * B);
         std::vector<EventPair> ev((size_t)B);
-        for (auto& e : ev) { RSFK_HIP(hipEventCreate(&e.a)); RSFK_HIP(hipEventCreate(&e.b)); }
+        for (auto& e : ev)
+            if (e.create()) return 1;
         int rc = 0;
         for (int tb0 = 0; tb0 < n_trees && rc == 0; tb0 += B) {
             const int nb = std::min(B, n_trees - tb0);
@@ -304,7 +328,6 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
                                 stats[5 * j + 0], stats[5 * j + 3], stats[5 * j + 2], ms * 1e-3);
             }
         }
-        for (auto& e : ev) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
         if (rc) return rc;
     }
     const double t_total = now_s() - t0;
@@ -360,22 +383,22 @@ int knn_forest_host(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_
     if (ws_alloc(&dp.p, nd * sizeof(float))) return 1;
     if (ws_alloc(&di.p, nk * sizeof(int))) return 1;
     if (ws_alloc(&dd.p, nk * sizeof(float))) return 1;
-    RSFK_HIP(hipMemcpy(dp.p, points, nd * sizeof(float), hipMemcpyHostToDevice));
+    if (copy_to_device(dp.p, points, nd * sizeof(float))) return 1;
     if (fresh_rows) {
         const unsigned grid = (unsigned)std::min<size_t>((nk + 255) / 256, 65536);
         hipLaunchKernelGGL(k_fresh_rows, dim3(grid), dim3(256), 0, nullptr, static_cast<int*>(di.p), static_cast<float*>(dd.p),
                            nk, K, fresh_rows == 2 ? 1 : 0);
         RSFK_HIP(hipGetLastError());
     } else {
-        RSFK_HIP(hipMemcpy(di.p, knn_idx, nk * sizeof(int), hipMemcpyHostToDevice));
-        RSFK_HIP(hipMemcpy(dd.p, knn_dist, nk * sizeof(float), hipMemcpyHostToDevice));
+        if (copy_to_device(di.p, knn_idx, nk * sizeof(int))) return 1;
+        if (copy_to_device(dd.p, knn_dist, nk * sizeof(float))) return 1;
     }
     const int rc = knn_forest_device(n_trees, K, N, D, MIN, MAX, MAX_DEPTH, verbose, seed, nnef,
                                      static_cast<const float*>(dp.p), static_cast<int*>(di.p),
                                      static_cast<float*>(dd.p), log_forest, nullptr);
     if (rc) return rc;
-    RSFK_HIP(hipMemcpy(knn_idx, di.p, nk * sizeof(int), hipMemcpyDeviceToHost));
-    RSFK_HIP(hipMemcpy(knn_dist, dd.p, nk * sizeof(float), hipMemcpyDeviceToHost));
+    if (copy_to_host(knn_idx, di.p, nk * sizeof(int))) return 1;
+    if (copy_to_host(knn_dist, dd.p, nk * sizeof(float))) return 1;
     return 0;
 }
 

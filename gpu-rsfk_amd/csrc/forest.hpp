@@ -19,6 +19,7 @@ const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
 int tree_small_threshold();
+const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w);
 int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, const uint8_t* q8, int N, int D,
                      int MIN, int MAX,
                      int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream);
@@ -51,6 +52,11 @@ int launch_bucket_knn_medium(const float* points, int D, int K, const int* ids, 
                              int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream);
 int launch_bucket_knn_small(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
                             int n_buckets, int stride, bool rows_sorted, int* knn_idx, float* knn_dist, hipStream_t stream);
+
+// host_copy.hip: pageable host memory <-> device memory through pinned buffers, on several threads
+int copy_to_device(void* dev_ptr, const void* host_ptr, size_t bytes);
+int copy_to_host(void* host_ptr, const void* dev_ptr, size_t bytes);
+void release_copy_buffers();
 
 // explore_join.hip
 struct ExploreWorkspace;

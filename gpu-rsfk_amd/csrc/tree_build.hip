@@ -890,6 +890,9 @@ struct TreeBatchWorkspace {
     TreeRec* recs = nullptr;             // B x rec_cap
     int* n_rec = nullptr;                // B
     int rec_cap = 0;
+    // events around the kernels of a wide level (hyperplanes | side test | scatter) and around the tail kernel
+    hipEvent_t ev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    float phase_s[4] = {0.f, 0.f, 0.f, 0.f};   // of the last batch: side tests, hyperplanes, scatter, tail kernel
 };
 
 static void free_ws(TreeBatchWorkspace& w)
@@ -899,6 +902,8 @@ static void free_ws(TreeBatchWorkspace& w)
     for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
+    for (hipEvent_t e : w.ev)
+        if (e) (void)hipEventDestroy(e);
     w = TreeBatchWorkspace();
 }
 
@@ -965,8 +970,12 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     if (dmalloc(&w->ctr, (size_t)1)) return 1;
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_ctr), sizeof(LevelCounters)));
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stats), sizeof(TreeStats) * (size_t)B));
+    for (hipEvent_t& e : w->ev) RSFK_HIP(hipEventCreate(&e));
     return 0;
 }
+
+// seconds the last batch spent in: side tests, hyperplanes of the wide levels, scatter, tail kernel
+const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w) { return w->phase_s; }
 
 // Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  pb16 = rows of the bfloat16 copy of the points (may be
 // null: every side test then reads the fp32 row).  On return perm[0] of
@@ -1018,6 +1027,16 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
                                          (int)side_lds));
         }
     }
+    for (float& v : w->phase_s) v = 0.0f;
+    bool level_timed = false;                 // ev[0..3] bracket the three kernels of the previous level
+    auto add_level_times = [&]() {
+        if (!level_timed) return;
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, w->ev[0], w->ev[1]) == hipSuccess) w->phase_s[1] += ms * 1e-3f;
+        if (hipEventElapsedTime(&ms, w->ev[1], w->ev[2]) == hipSuccess) w->phase_s[0] += ms * 1e-3f;
+        if (hipEventElapsedTime(&ms, w->ev[2], w->ev[3]) == hipSuccess) w->phase_s[2] += ms * 1e-3f;
+        level_timed = false;
+    };
     // wide levels
     while (true) {
         // one trip to the host per level: the chunk table of the level is made first (from the node count on the
@@ -1025,17 +1044,20 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], w->node_cap, P.chunk, w->chunk_base, w->ctr);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
+        add_level_times();
         RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
         const int n_nodes = w->h_ctr->n_next;
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
         const int n_chunks = w->h_ctr->n_chunks;
         RSFK_CHECK(n_chunks <= w->chunk_cap, "tree batch: chunk table overflow");
+        (void)hipEventRecord(w->ev[0], stream);
         hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + plane_waves - 1) / plane_waves)), dim3(64 * plane_waves),
                            plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
         // n_next := 0 for the level being produced
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
+        (void)hipEventRecord(w->ev[1], stream);
         // lanes per point in the 8-bit screen: a lane takes 16 coordinates per step
         const int q8_pieces = q8_padded(D) >> 4;
 #define RSFK_SIDE_LAUNCH(Q, L)                                                                                              \
@@ -1046,9 +1068,12 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         else if (q8_pieces <= 4) RSFK_SIDE_LAUNCH(true, 4);
         else RSFK_SIDE_LAUNCH(true, 8);
 #undef RSFK_SIDE_LAUNCH
+        (void)hipEventRecord(w->ev[2], stream);
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
                            w->recs, w->n_rec, w->rec_cap);
+        (void)hipEventRecord(w->ev[3], stream);
+        level_timed = true;
         RSFK_HIP(hipGetLastError());
         cur ^= 1;
     }
@@ -1065,6 +1090,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
                            2 * (size_t)node_cap * sizeof(SmallNode) + (size_t)P.small;
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         const bool tail_q8 = q8 != nullptr && std::getenv("RSFK_TAIL_BF16") == nullptr;
+        (void)hipEventRecord(w->ev[4], stream);
         if (tail_q8) {
             RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          (int)lds));
@@ -1078,11 +1104,16 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
                                w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr,
                                w->recs, w->n_rec, w->rec_cap);
         }
+        (void)hipEventRecord(w->ev[5], stream);
         RSFK_HIP(hipGetLastError());
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
     RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
     RSFK_HIP(hipStreamSynchronize(stream));
+    if (n_tail > 0) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, w->ev[4], w->ev[5]) == hipSuccess) w->phase_s[3] = ms * 1e-3f;
+    }
     RSFK_CHECK(!w->h_ctr->overflow, "tree batch: queue overflow in the tail phase");
     for (int t = 0; t < nb; ++t) {
         const int total = w->h_stats[t].n_leaves + w->h_stats[t].n_big;

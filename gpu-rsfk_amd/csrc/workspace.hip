@@ -3,9 +3,12 @@
 // hipMalloc / hipFree of a few hundred megabytes cost tens to hundreds of microseconds each and a call needs
 // about thirty of them, so blocks are kept after use and handed out again to the next call that asks for the
 // same size on the same device (a build repeated with the same shapes allocates nothing).  Idle blocks are
-// capped at a quarter of the device memory; rsfk_release_workspace() returns all of them to the driver.
+// capped at RSFK_WORKSPACE_POOL_MB megabytes (default: a quarter of the device memory, at most 16 GiB; 0 keeps
+// nothing); rsfk_release_workspace() returns all of them to the driver.
 // The reference allocates and frees inside every tree level (src/rsfk.cu:640-1180).
 #include "rsfk_common.hpp"
+#include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <vector>
@@ -19,7 +22,23 @@ struct Pool {
     std::multimap<std::pair<int, size_t>, void*> idle;     // (device, bytes) -> block
     std::map<void*, std::pair<int, size_t>> live;           // blocks handed out
     size_t idle_bytes = 0;
+    size_t idle_cap = 0;                                    // set on first use
+    bool cap_known = false;
 };
+
+// most idle bytes the pool keeps (asked of the device once)
+size_t idle_cap_locked(Pool& P)
+{
+    if (!P.cap_known) {
+        P.cap_known = true;
+        size_t free_b = 0, total_b = 0;
+        P.idle_cap = (size_t)4 << 30;
+        if (hipMemGetInfo(&free_b, &total_b) == hipSuccess) P.idle_cap = std::min<size_t>(total_b / 4, (size_t)16 << 30);
+        const char* e = std::getenv("RSFK_WORKSPACE_POOL_MB");
+        if (e && *e) P.idle_cap = (size_t)std::max(0ll, std::atoll(e)) << 20;
+    }
+    return P.idle_cap;
+}
 
 Pool& pool()
 {
@@ -82,9 +101,7 @@ void ws_free(void* p)
         }
         key = it->second;
         P.live.erase(it);
-        size_t free_b = 0, total_b = 0;
-        const bool known = hipMemGetInfo(&free_b, &total_b) == hipSuccess;
-        if (!known || P.idle_bytes + key.second <= total_b / 4) {
+        if (P.idle_bytes + key.second <= idle_cap_locked(P)) {
             P.idle.insert({key, p});
             P.idle_bytes += key.second;
             return;

@@ -30,6 +30,20 @@ def random_motion(points, random_motion_force):
         points[:, d] = points[:, d] + random_motion_force * np.random.uniform(-range_uniform, range_uniform, N)
 
 
+MAX_NEIGHBORS = 256      # a K-NN row is held by one wavefront, up to four slots per lane
+
+
+def _check_sizes(points, K, n_trees=0):
+    """The entry points of the reference's interface have no status return (a failure inside the library ends
+    the process, as in the reference), so what the library would refuse is refused here, with an exception."""
+    if points.ndim != 2 or points.shape[0] < 1 or points.shape[1] < 1:
+        raise ValueError("points must be a matrix with at least one row and one column")
+    if K is not None and not (1 <= K <= MAX_NEIGHBORS):
+        raise ValueError("num_nearest_neighbors = {}: this library supports 1..{} neighbours".format(K, MAX_NEIGHBORS))
+    if n_trees < 0:
+        raise ValueError("n_trees must not be negative")
+
+
 class ForestLog(object):
     """Per-tree series decoded from the ``float32[16*n_trees+2]`` log that the
     library fills (names and order: reference RSFK.py:71-88)."""
@@ -164,6 +178,7 @@ class RSFK(object):
             if verbose > 0:
                 print("Automatically setting n_trees to {}".format(n_trees))
         n_trees = int(n_trees)
+        _check_sizes(points, K, n_trees)
 
         if add_bit_random_motion:
             random_motion(points, random_motion_force)
@@ -259,6 +274,9 @@ class RSFK(object):
             if verbose > 0:
                 print("Automatically setting n_trees to {}".format(n_trees))
         n_trees = int(n_trees)
+        _check_sizes(points, K, n_trees)
+        if query_points.ndim != 2 or query_points.shape[1] != D:
+            raise ValueError("query_points must be a matrix with the columns of points")
 
         if add_bit_random_motion:
             random_motion(points, random_motion_force)
@@ -310,6 +328,7 @@ class RSFK(object):
         min_tree_children = int(min_tree_children)
         N = points.shape[0]
         D = points.shape[1]
+        _check_sizes(points, None)
 
         if min_tree_children < 0:
             raise Exception('min_tree_children = {} \t => min_tree_children must be at least 1'.format(min_tree_children))
@@ -343,34 +362,36 @@ class RSFK(object):
         return total_leaves, max_child, nodes_buckets, bucket_sizes
 
 
-def test1():
-    """Smoke check of the reference package (RSFK.py:841-862): no -1 index."""
-    test_N, test_D, test_K = 3000, 200, 30
-    dataX = np.random.random((test_N, test_D))
-    rptk = RSFK(random_state=0)
-    indices, dist = rptk.find_nearest_neighbors(dataX, test_K, max_tree_children=128, max_tree_depth=5000,
-                                                n_trees=10, random_motion_force=0.01, nn_exploring_factor=2,
-                                                add_bit_random_motion=True, verbose=2)
-    negative_indices = np.sum(indices == -1)
-    if negative_indices > 0:
-        raise Exception('{} Negative indices'.format(negative_indices))
+def _check_knn_graph_build():
+    """A small K-NN graph with jittered input and two exploration passes: every slot must be filled
+    (the property the reference's first built-in check asserts, RSFK.py:841-862)."""
+    rng = np.random.default_rng(0)
+    n, dim, k = 3000, 200, 30
+    x = rng.random((n, dim))
+    knn, _ = RSFK(random_state=0).find_nearest_neighbors(
+        x, k, n_trees=10, max_tree_children=128, nn_exploring_factor=2, add_bit_random_motion=True,
+        random_motion_force=0.01, verbose=2)
+    empty = int((knn < 0).sum())
+    if empty:
+        raise Exception("%d empty neighbour slots in the K-NN graph" % empty)
 
 
-def test2():
-    """Smoke check of the reference package (RSFK.py:864-903)."""
-    n_points, n_dim = 2 ** 12, 99
-    points = np.random.random((n_points, n_dim))
-    min_tree_children = int(n_points / 30)
-    max_tree_children = 3 * min_tree_children
-    print("Number of points {}".format(n_points))
-    print("Number of dimensions {}".format(n_dim))
-    rsfk = RSFK(random_state=0)
-    total_leaves, max_child, nodes_buckets, bucket_sizes = rsfk.cluster_by_sample_tree(
-        points, min_tree_children=min_tree_children, max_tree_children=max_tree_children,
-        max_tree_depth=5000, random_motion_force=0.1, verbose=2, add_bit_random_motion=False)
-    print("Total leaves: {}".format(total_leaves))
+def _check_single_tree_partition():
+    """One random-sample tree on 4096 points of 99 dimensions: the call returns a partition
+    (what the reference's second built-in check runs, RSFK.py:864-903) and it covers every point once."""
+    rng = np.random.default_rng(1)
+    n, dim = 4096, 99
+    x = rng.random((n, dim))
+    smallest = n // 30
+    print("points: %d, dimensions: %d, bucket sizes: %d..%d" % (n, dim, smallest, 3 * smallest))
+    leaves, widest, members, sizes = RSFK(random_state=0).cluster_by_sample_tree(
+        x, min_tree_children=smallest, max_tree_children=3 * smallest, verbose=2)
+    print("buckets: %d, largest: %d" % (leaves, widest))
+    if int(sizes.sum()) != n or not np.array_equal(np.sort(members[members >= 0]), np.arange(n)):
+        raise Exception("the buckets do not cover every point exactly once")
 
 
 def test():
-    test1()
-    test2()
+    """The package's built-in smoke run (same entry point as the reference's ``gpu_rsfk.test``)."""
+    _check_knn_graph_build()
+    _check_single_tree_partition()

@@ -208,6 +208,11 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
     assert log["Min Leaf Size"] == [int(v) for v in olog[8:12]]
     assert log["Total Leaves"] == [int(v) for v in olog[12:16]]
     assert all(t > 0 for t in log["KNN Sets Updates"]) and r._last_search_time > 0
+    # the phases that have a counterpart here carry their time: side tests, hyperplanes of the wide levels,
+    # scatter (the reference's node update) and the kernel that finishes the small subtrees (its bucket creation)
+    for name in ("Check Points Side Time", "Create Nodes Time", "Update Nodes Time", "Bucket Creation Time"):
+        assert all(t > 0 for t in log[name]), name
+        assert sum(log[name]) < sum(log["Total Tree Building Time"])
     assert (gi >= 0).all()
 
 

@@ -150,3 +150,22 @@ def test_golden_vectors_still_come_out_of_the_oracle(orc):
     indptr, cols, vals = orc.symmetrize(g["forest_idx"], g["forest_dist"], drop_self=True)
     assert np.array_equal(indptr, g["csr_indptr"]) and np.array_equal(cols, g["csr_indices"])
     assert np.array_equal(vals, g["csr_data"])
+
+
+def test_sizes_the_library_would_refuse_raise_in_python(capi):
+    """K above 256, no rows, negative n_trees: an exception before the call, not exit(1) inside the library."""
+    import gpu_rsfk
+    r = gpu_rsfk.RSFK(random_state=0)
+    X = np.zeros((10, 3), np.float32)
+    with pytest.raises(ValueError):
+        r.find_nearest_neighbors(X, 300)
+    with pytest.raises(ValueError):
+        r.find_nearest_neighbors(X, 0)
+    with pytest.raises(ValueError):
+        r.find_nearest_neighbors(np.zeros((0, 3), np.float32), 4)
+    with pytest.raises(ValueError):
+        r.find_nearest_neighbors(X, 4, n_trees=-5)
+    with pytest.raises(ValueError):
+        r.find_nearest_neighbors_ann(X, np.zeros((4, 2), np.float32), 4)
+    with pytest.raises(ValueError):
+        r.cluster_by_sample_tree(np.zeros((0, 3), np.float32))
