@@ -228,7 +228,11 @@ def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
     balance = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
     small = K <= 64 and mx <= 72
     gram = os.environ.get("RSFK_GRAM_FROM")
-    kernel = ("k_bucket_knn_small<64> (buckets <= 64) + k_bucket_knn_small<72> (65..72)" if small
+    scr = os.environ.get("RSFK_BUCKET_SCREEN")
+    first = (4 if D >= 128 else 8) if not scr else (int(scr) if scr.isdigit() else None)
+    kernel = (("k_bucket_knn_small<64> (buckets <= 64" + ("" if first is None else "; trees 0..%d" % (first - 1) if first > 0 else "; no tree")
+               + ")" + ("" if first is None else " / k_bucket_knn_screen (later trees: pair matrix bounded on the matrix cores)")
+               + " + k_bucket_knn_small<72> (65..72)") if small
               else "k_bucket_knn (64 x 64 tiles of the pair matrix)" + ("" if mx <= 72 or K > 64 else " + k_bucket_knn_small for the buckets up to 72 points"))
     if gram is not None:
         kernel += "; k_bucket_knn_gram from tree %s on (RSFK_GRAM_FROM)" % gram

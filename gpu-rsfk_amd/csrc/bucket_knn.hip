@@ -311,7 +311,11 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
     int skip_upto = 0;
     if (K <= 64) {
         // buckets of up to 72 points go to the specialised kernels; the general one skips them
-        if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
+        if (bucket_screen_from(D, K) == 0) {
+            // RSFK_BUCKET_SCREEN=0: the screened kernel for every call; it needs sorted rows
+            if (launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
+            if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_buckets, stride, knn_idx, knn_dist, stream)) return 1;
+        } else if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
             return 1;
         if (max_bucket >= 0 && max_bucket <= small_bucket_cap()) return 0;
         if (launch_bucket_knn_medium(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
@@ -324,10 +328,10 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
 // (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  rows_sorted: every K-NN row is
-// known to be sorted by distance.  bf: bfloat16 copy of the points to send the small buckets to the screened kernel
-// (needs sorted rows), else null.  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
+// known to be sorted by distance.  screen: the small buckets go to the kernel that bounds the pair matrix on the matrix
+// cores first (needs sorted rows, K <= 64).  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
 // kinds touch different rows, so the two parts of one tree may run side by side).
-int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_sorted, bool gram, int D, int K, const int* ids,
+int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
                            int* knn_idx, float* knn_dist, hipStream_t stream, int part)
 {
@@ -352,8 +356,8 @@ int launch_bucket_knn_tree(const float* points, const Bf16Copy* bf, bool rows_so
                                       stream);
     }
     if (n_small > 0 && part != 2) {
-        if (K <= 64 && bf != nullptr && rows_sorted) {
-            if (launch_bucket_knn_screen(points, *bf, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, stream)) return 1;
+        if (K <= 64 && screen && rows_sorted) {
+            if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted)) {

@@ -47,16 +47,12 @@
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
 #include "forest.hpp"
+#include "mfma_split.hpp"
 #include <algorithm>
 
 namespace rsfk {
 
 namespace {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int kGT = 64;                       // points per tile side
 constexpr int kGThreads = 256;
@@ -65,33 +61,6 @@ constexpr int kGMaxChunk = 128;               // dimensions staged at once (a mu
 constexpr int kGBatch = 4;                    // pairs per thread between two passes over the chunks (long rows only)
 constexpr int kGMeta = 6 * kGT + 4;           // ints of LDS for ids, last slots, norms, flags and the pair counter
 constexpr int kGAhead = 4;                    // K-NN rows a wavefront requests together
-
-// Two fp32 values -> their bfloat16 heads (packed) and the bfloat16 heads of what the first rounding left over.
-__device__ __forceinline__ void split2(float a, float b, uint32_t& hi, uint32_t& lo)
-{
-    const f32x2 v = {a, b};
-    hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-    const f32x2 r = {a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xffff0000u)};
-    lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(r, bf16x2));
-}
-
-// Eight consecutive values of a row in LDS -> matrix-core operands (heads and remainders); adds their squares to nrm.
-__device__ __forceinline__ void load_split(const float* __restrict__ p, bf16x8& hi, bf16x8& lo, float& nrm)
-{
-    const float4 u = *reinterpret_cast<const float4*>(p);
-    const float4 v = *reinterpret_cast<const float4*>(p + 4);
-    uint4 h, l;
-    split2(u.x, u.y, h.x, l.x);
-    split2(u.z, u.w, h.y, l.y);
-    split2(v.x, v.y, h.z, l.z);
-    split2(v.z, v.w, h.w, l.w);
-    hi = __builtin_bit_cast(bf16x8, h);
-    lo = __builtin_bit_cast(bf16x8, l);
-    nrm = __builtin_fmaf(u.x, u.x, nrm); nrm = __builtin_fmaf(u.y, u.y, nrm);
-    nrm = __builtin_fmaf(u.z, u.z, nrm); nrm = __builtin_fmaf(u.w, u.w, nrm);
-    nrm = __builtin_fmaf(v.x, v.x, nrm); nrm = __builtin_fmaf(v.y, v.y, nrm);
-    nrm = __builtin_fmaf(v.z, v.z, nrm); nrm = __builtin_fmaf(v.w, v.w, nrm);
-}
 
 // The rows of one tile on their way from HBM to LDS: PASSES 16-byte pieces per thread.  1 << lpr_shift lanes work on
 // a row (8..32, at least the pieces of a chunk); zeros beyond D and for the rows beyond `rows`.
@@ -411,8 +380,7 @@ int launch_bucket_knn_gram(const float* points, int D, int K, const int* ids, co
     while ((1 << lpr_shift) < (chunk >> 2)) ++lpr_shift;  // lanes per row while staging: 8, 16 or 32
     const size_t lds = (size_t)(max_tiles > 1 ? 2 : 1) * kGT * pitch * 4 + (size_t)kGT * kGDistPitch * 4 + (size_t)kGMeta * 4 +
                        (size_t)kGT * kGT * 2;
-    const float dp = (float)d16;
-    const float c_err = 3.1f / 65536.0f + (3.1f * dp + 8.0f) / 8388608.0f + (dp + 2.0f) / 16777216.0f;
+    const float c_err = split_gram_error_coefficient(d16);
     const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);
     RSFK_CHECK(one_minus_gamma > 0.5f, "screened bucket kernel: D too large");
 #define RSFK_GRAM_CASE(SLV, PV)                                                                                            \

@@ -1,237 +1,241 @@
-// Bucket K-NN for buckets of at most 64 points and K <= 64 when a bfloat16 copy of
-// the points exists: same function and same results as the kernel in
+// Bucket K-NN for buckets of at most 64 points and K <= 64 with the pair matrix
+// bounded on the matrix cores first: same function and same results as the kernel in
 // bucket_knn_small.hip (see bucket_knn.hip for the reference kernels both replace),
-// but most pair distances are never computed.
+// same decomposition (one bucket per workgroup of two wavefronts, many workgroups
+// per compute unit), but the sequential fp32 chains -- nearly all of the arithmetic
+// of that kernel, and what bounds it -- are only run for the pairs that may change a
+// row.
 //
-// A pair (i, j) of a bucket changes nothing unless its distance is smaller than
-// the last slot of row i or of row j.  After the first few trees that holds for a
-// small fraction of the pairs, so the kernel first bounds every pair from below:
+// A pair (i, j) changes nothing unless its distance is at most the last slot of row
+// i or of row j.  Once the rows are good that holds for a small share of the pairs
+// (none at all in most buckets of clustered high-dimensional data), so:
 //
-//   1. Gram matrix of the bucket's bfloat16 rows with the matrix cores
-//      (v_mfma_f32_32x32x16_bf16, operands straight from global memory, one to
-//      three 32x32 tiles): d~ = n_i + n_j - 2 G_ij approximates the distance, and
-//      a bound on |d~ - exact fp32 result| follows from the norms alone.  With
-//      S = n_i + n_j (norms of the bfloat16 rows), u = 2^-8:
-//        rounding to bfloat16:   |d(real) - d~(real)| <= 2u sqrt(d~ Q) + u^2 Q,  Q = 2 S  (Cauchy-Schwarz)
-//        Gram matrix and norms:  |d~(computed) - d~(real)| <= E1 = (D' + 16) 2^-21 S
-//        fp32 chain:             result >= d(real) (1 - gamma),  gamma = (D + 8) 2^-22
-//      so the pair is dropped iff  d~ - E1 - 1.01 (2u sqrt((d~ + E1) Q) + u^2 Q) >= (limit + 1e-30) / (1 - gamma),
-//      limit = max(last slot of row i, last slot of row j); the inequality is evaluated
-//      without the square root (both sides squared when the left side is not negative).
-//      This never drops a pair that the exact arithmetic would have inserted;
-//   2. the remaining pairs go to a list in LDS; the fp32 rows are staged through LDS
-//      in slices of at most 52 dimensions and each thread runs the sequential fused
-//      multiply-add chains (arithmetic of euclidean_distance_sqr,
-//      compute_knn_from_buckets.cu:40-54) of its pairs of the list;
-//   3. the exact distances land in a triangular matrix in LDS (+inf elsewhere) and
-//      the rows are updated as in the other kernel; rows without any candidate below
-//      their last slot are neither read nor written.
+//   1. the fp32 rows pass through LDS, kChunk dimensions at a time, the next chunk
+//      travelling while this one is used; the wavefronts read them as matrix-core
+//      operands, every value split into two bfloat16 numbers (mfma_split.hpp), and
+//      accumulate the three 32 x 32 quadrants of the upper triangle of the Gram
+//      matrix (wavefront 0: the first diagonal quadrant and the off-diagonal one,
+//      wavefront 1: the second diagonal quadrant) and the squared norms;
+//   2. with S = n_i + n_j and d~ = S - 2 G_ij the real-number distance is at least
+//      d~ - c S (c: split_gram_error_coefficient) and the fp32 chain of the exact
+//      path returns at least (1 - gamma) times the real-number distance,
+//      gamma = (D + 8) 2^-22: the pair is dropped iff
+//      (d~ - c S)(1 - gamma) > max(last slot of row i, last slot of row j).
+//      NaN or infinite intermediate values never drop a pair;
+//   3. the pairs that are left go to a list in LDS.  If it is empty the workgroup is
+//      done.  Otherwise the rows pass through LDS once more (not when D <= kChunk:
+//      they are still there) and each thread runs the sequential fused multiply-add
+//      chains of its pairs of the list (arithmetic of euclidean_distance_sqr,
+//      compute_knn_from_buckets.cu:40-54: a pair has the same distance value as in
+//      every other kernel);
+//   4. the exact distances go into the bucket's distance matrix in LDS (+inf
+//      elsewhere) and the rows that got a candidate are merged as in the other kernel.
 //
-// Requires every K-NN row to be sorted by distance on entry (the last slot is the
-// maximum); launch_sort_rows establishes that once per build.
+// Requires every K-NN row to be sorted on entry (the last slot is its maximum);
+// launch_sort_rows establishes that once per build.
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
 #include "forest.hpp"
+#include "mfma_split.hpp"
+#include <algorithm>
+#include <cstdlib>
 
 namespace rsfk {
 
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-
 constexpr int kCap = kBucketSplit;          // largest bucket this kernel takes
-static_assert(kCap == 64, "two 32-row operand halves and lane-per-candidate merge assume 64");
+static_assert(kCap == 64, "two 32-row operand blocks and lane-per-candidate merge assume 64");
 constexpr int kThreads = 128;
-constexpr int kWaves = kThreads / 64;
-constexpr int kMaxChunk = 52;               // dimensions staged at once
-constexpr int kLanesPerRow = 16;            // a row of a slice is loaded by 16 lanes, 16 bytes each (13 used at most)
-constexpr int kRowsPerStep = kThreads / kLanesPerRow;
-constexpr int kLoads = kCap / kRowsPerStep; // 16-byte loads per thread and slice
+constexpr int kDistPitch = kCap + 1;
+constexpr int kChunk = 64;                 // dimensions staged at once (a multiple of 16)
 constexpr int kMaxPairs = kCap * (kCap - 1) / 2;
-constexpr int kPairsPerThread = (kMaxPairs + kThreads - 1) / kThreads;
-static_assert(kMaxChunk / 4 <= kLanesPerRow, "a slice must fit the lanes of a row");
+constexpr int kMaxRounds = (kMaxPairs + kThreads - 1) / kThreads;     // listed pairs per thread
+constexpr int kListSlots = (kMaxPairs + 7) & ~7;
 
-constexpr float kU = 1.0f / 256.0f;                           // unit roundoff of bfloat16 (8 significant bits)
-constexpr float kC2 = 1.01f * kU * kU * 2.0001f;              // coefficient of S in the u^2 Q term
-constexpr float kC3 = (2.02f * kU) * (2.02f * kU) * 2.0001f;  // (1.01 2u)^2 Q / S
+// LDS after the row / distance region: ids, last slots, flags, norms as seen by either wavefront, pair counter, list
+struct ScreenMeta {
+    int lids[kCap];
+    float tau[kCap];
+    int flag[kCap];
+    float nrm[2][kCap];
+    int n_pairs[4];
+    uint16_t list[kListSlots];
+};
 
-// entry of pair (a, b), a < b, in the triangular matrix
-__device__ __forceinline__ int tri_at(int a, int b) { return ((b * (b - 1)) >> 1) + a; }
+// The rows of the bucket on their way from HBM to LDS: 16 lanes (a quarter wavefront) per row, a lane moves 16 bytes
+// of kLoads rows.  Zeros beyond D and for the rows beyond s.
+struct RowLoads {
+    static constexpr int kPieces = kChunk / 4;
+    static constexpr int kRowsPerPass = kThreads / kPieces;
+    static constexpr int kLoads = kCap / kRowsPerPass;
+    float4 v[kLoads];
 
-// Screen one 32x32 tile of the Gram matrix.  Accumulator i of lane l belongs to row member
-// m = mbase + 8 (i / 4) + i % 4 (mbase = first member of the operand half + 4 (l / 32)) and column
-// member n.  Returns the mask of accumulators whose pair (m < n < s) must be computed exactly.
-// taup = (last slot + 1e-30) / (1 - gamma) per member.
-__device__ __forceinline__ uint32_t screen_tile(const f32x16& g, int mbase, int n, int s, const float* nrm,
-                                                const float* taup, float kappa)
-{
-    const float nn = nrm[n], tn = taup[n];
-    uint32_t bits = 0;
+    __device__ __forceinline__ void request(const int* __restrict__ lids, int s, const float* __restrict__ points, int D,
+                                            int d0, bool vec_ok)
+    {
+        const int piece = threadIdx.x & (kPieces - 1);
+        const int r0 = threadIdx.x / kPieces;
+        const int d = d0 + 4 * piece;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int m = mbase + 8 * (i >> 2) + (i & 3);
-        const float S = nrm[m] + nn;
-        const float limit = fmaxf(taup[m], tn);
-        const float dt = __builtin_fmaf(-2.0f, g[i], S);            // distance of the bfloat16 rows
-        const float e1 = kappa * S;                                 // accumulation errors of G and the norms
-        const float dhi = fmaxf(dt + e1, 0.0f);
-        const float a = dt - e1 - kC2 * S - limit;
-        const bool skip = a >= 0.0f && a * a >= kC3 * dhi * S;      // false if anything is NaN
-        if (m < n && n < s && !skip) bits |= 1u << i;
+        for (int i = 0; i < kLoads; ++i) {
+            const int m = r0 + i * kRowsPerPass;
+            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < s && d < D) {
+                const float* src = points + (size_t)lids[m] * (size_t)D + d;
+                if (vec_ok) {
+                    v[i] = *reinterpret_cast<const float4*>(src);
+                } else {
+                    v[i].x = src[0];
+                    if (d + 1 < D) v[i].y = src[1];
+                    if (d + 2 < D) v[i].z = src[2];
+                    if (d + 3 < D) v[i].w = src[3];
+                }
+            }
+        }
     }
-    return bits;
-}
 
-__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* __restrict__ points,
-                                                                   const uint16_t* __restrict__ brows,
-                                                                   const float* __restrict__ bnorms, int D, int K,
+    __device__ __forceinline__ void commit(float* __restrict__ rows, int pitch) const
+    {
+        const int piece = threadIdx.x & (kPieces - 1);
+        const int r0 = threadIdx.x / kPieces;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i)
+            *reinterpret_cast<float4*>(&rows[(r0 + i * kRowsPerPass) * pitch + 4 * piece]) = v[i];
+    }
+};
+
+// SINGLE: D <= kChunk, the rows are staged once and stay in LDS until the exact chains have run.
+template <bool SINGLE>
+__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* __restrict__ points, int D, int K,
                                                                    const int* __restrict__ ids,
                                                                    const int* __restrict__ starts,
-                                                                   const int* __restrict__ sizes,
+                                                                   const int* __restrict__ sizes, int stride,
                                                                    int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                                   int chunk, int pitch, int region_floats, int bpitch,
-                                                                   int ksteps, float kappa, float inv_one_minus_gamma)
+                                                                   float c_err, float one_minus_gamma)
 {
-    // dynamic LDS: [rows | triangular distance matrix] (region_floats) | ids[64] | tau[64] | taup[64] | nrm[64] |
-    //              n_pairs | flag[64] | list
-    extern __shared__ __align__(16) float lds_f[];
-    float* rows = lds_f;
-    float* tri = lds_f;                      // same storage, used after the last read of rows
-    int* lids = reinterpret_cast<int*>(lds_f + region_floats);
-    float* tau = reinterpret_cast<float*>(lids + kCap);
-    float* taup = tau + kCap;
-    float* nrm = taup + kCap;
-    int* n_pairs = reinterpret_cast<int*>(nrm + kCap);
-    int* flag = n_pairs + 4;                 // member has a candidate below its last slot
-    uint16_t* list = reinterpret_cast<uint16_t*>(flag + kCap);
+    constexpr int kPitch = kChunk + 4;                    // an odd number of 16-byte units: rows start in different banks
+    constexpr int kRegion = kCap * kPitch > kCap * kDistPitch ? kCap * kPitch : kCap * kDistPitch;
+    __shared__ __align__(16) float region[kRegion];       // the rows, later the distance matrix
+    __shared__ ScreenMeta M;
+    float* rows = region;
+    float* dist = region;
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
     if (s < 2 || s > kCap) return;
-    const int* bid = ids + (size_t)starts[bkt];
+    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+    const int n_chunks = SINGLE ? 1 : (D + kChunk - 1) / kChunk;
 
     if (tid < kCap) {
         const int id = tid < s ? bid[tid] : -1;
-        const float t = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
-        lids[tid] = id;
-        tau[tid] = t;
-        taup[tid] = (t + 1e-30f) * inv_one_minus_gamma;
-        nrm[tid] = id >= 0 ? bnorms[id] : 0.0f;
+        M.lids[tid] = id;
+        M.tau[tid] = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
+        M.flag[tid] = 0;
     }
-    if (tid < kCap) flag[tid] = 0;
-    if (tid == 0) *n_pairs = 0;
+    if (tid == kCap) M.n_pairs[0] = 0;
     __syncthreads();
 
-    // fp32 rows of a slice: lane pc of a group of 16 loads piece pc of rows rg, rg + 8, ...; requested early,
-    // written to LDS when the previous slice has been consumed
-    const int pc = tid & (kLanesPerRow - 1), rg = tid / kLanesPerRow;
-    // two slices are in flight: A holds slices 0, 2, ..., B slices 1, 3, ...
-    float4 preA[kLoads], preB[kLoads];
-    auto request = [&](float4 (&pre)[kLoads], int d0) {
-        const int np = d0 < D ? min(chunk, (D - d0 + 3) & ~3) >> 2 : 0;      // 16-byte pieces per row in this slice
-#pragma unroll
-        for (int i = 0; i < kLoads; ++i) {
-            pre[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            const int m = rg + kRowsPerStep * i;
-            if (pc < np && m < s) {
-                const float* src = points + (size_t)lids[m] * (size_t)D + 4 * pc + d0;
-                if (vec_ok) {
-                    pre[i] = *reinterpret_cast<const float4*>(src);
-                } else {
-                    const int left = D - d0 - 4 * pc;
-                    pre[i].x = src[0];
-                    if (left > 1) pre[i].y = src[1];
-                    if (left > 2) pre[i].z = src[2];
-                    if (left > 3) pre[i].w = src[3];
-                }
-            }
-        }
-        return np;
-    };
-    int npA = 0, npB = 0;
-
-    // ---- 1. screen: wavefront 0 takes the tiles (half 0 x half 0) and (half 0 x half 1), wavefront 1 the
-    //         tile (half 1 x half 1); members beyond s read the row of member 0 and are ignored
+    // ---- 1. Gram quadrants and norms
+    const bool two_blocks = s > 32;
+    const bool act0 = wave == 0 || two_blocks;            // this wavefront's diagonal quadrant (block `wave`)
+    const bool act1 = wave == 0 && two_blocks;            // quadrant (block 0, block 1)
+    RowLoads ld;
     {
-        const bool two_halves = s > 32;
-        const int hx = wave;                                     // operand half of this wavefront's first tile
-        if (hx == 0 || two_halves) {
-            const int mx = 32 * hx + (lane & 31), my = 32 + (lane & 31);
-            const uint16_t* rx = brows + (size_t)lids[mx < s ? mx : 0] * (size_t)bpitch + 8 * (lane >> 5);
-            const uint16_t* ry = brows + (size_t)lids[my < s ? my : 0] * (size_t)bpitch + 8 * (lane >> 5);
-            const bool second = hx == 0 && two_halves;
-            f32x16 gxx, gxy;
+        f32x16 g0, g1;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { gxx[i] = 0.0f; gxy[i] = 0.0f; }
-            for (int k0 = 0; k0 < ksteps; k0 += 8) {           // operands of eight steps (128 dimensions) in flight
-                bf16x8 x[8], y[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (k0 + u < ksteps) {
-                        x[u] = *reinterpret_cast<const bf16x8*>(rx + 16 * (k0 + u));
-                        if (second) y[u] = *reinterpret_cast<const bf16x8*>(ry + 16 * (k0 + u));
-                        else y[u] = x[u];
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (k0 + u < ksteps) {
-                        gxx = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], x[u], gxx, 0, 0, 0);
-                        if (second) gxy = __builtin_amdgcn_mfma_f32_32x32x16_bf16(x[u], y[u], gxy, 0, 0, 0);
+        for (int i = 0; i < 16; ++i) { g0[i] = 0.0f; g1[i] = 0.0f; }
+        float n0 = 0.0f, n1 = 0.0f;
+        const float* pa = rows + (32 * wave + (lane & 31)) * kPitch + 8 * (lane >> 5);
+        const float* pb = rows + (32 + (lane & 31)) * kPitch + 8 * (lane >> 5);
+        ld.request(M.lids, s, points, D, 0, vec_ok);
+        for (int c = 0; c < n_chunks; ++c) {
+            if (!SINGLE && c > 0) __syncthreads();       // the previous chunk has been consumed
+            ld.commit(rows, kPitch);
+            __syncthreads();
+            if (!SINGLE && c + 1 < n_chunks) ld.request(M.lids, s, points, D, (c + 1) * kChunk, vec_ok);
+            const int ksteps = min(kChunk, (D - c * kChunk + 15) & ~15) >> 4;
+            if (act0) {
+                for (int k = 0; k < ksteps; ++k) {
+                    bf16x8 ah, al;
+                    load_split(pa + 16 * k, ah, al, n0);
+                    g0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, ah, g0, 0, 0, 0);
+                    g0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, al, g0, 0, 0, 0);
+                    g0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, ah, g0, 0, 0, 0);
+                    if (act1) {
+                        bf16x8 bh, bl;
+                        load_split(pb + 16 * k, bh, bl, n1);
+                        g1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bh, g1, 0, 0, 0);
+                        g1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah, bl, g1, 0, 0, 0);
+                        g1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(al, bh, g1, 0, 0, 0);
                     }
                 }
             }
-            // the fp32 rows of the first two slices travel while the tiles are screened
-            npA = request(preA, 0);
-            npB = request(preB, chunk);
-            const int mbase = 32 * hx + 4 * (lane >> 5);
-            for (int t = 0; t < (second ? 2 : 1); ++t) {
-                const int n = t == 0 ? mx : my;
-                uint32_t bits = screen_tile(t == 0 ? gxx : gxy, mbase, n, s, nrm, taup, kappa);
-                const int cnt = __popc(bits);
-                int at = cnt ? atomicAdd(n_pairs, cnt) : 0;
-                while (bits) {
-                    const int i = __ffs(bits) - 1;
-                    bits &= bits - 1;
-                    const int m = mbase + 8 * (i >> 2) + (i & 3);
-                    list[at++] = (uint16_t)(m | (n << 6));
-                }
-            }
-        } else {
-            npA = request(preA, 0);
-            npB = request(preB, chunk);
         }
+        // a lane holds the squares of half of the dimensions of its row: add the two halves
+        n0 += __shfl_xor(n0, 32, 64);
+        n1 += __shfl_xor(n1, 32, 64);
+        float* nrm = M.nrm[wave];                     // a wavefront only reads back what it wrote itself
+        if (lane < 32) {
+            nrm[32 * wave + lane] = n0;
+            if (wave == 0) nrm[32 + lane] = n1;
+        }
+        wave_lds_sync();
+
+        // ---- 2. screen.  Accumulator i of lane l is pair (m, n), m = 32 qi + 8 (i / 4) + i % 4 + 4 (l / 32),
+        //         n = 32 qj + l % 32; in a diagonal quadrant only m < n counts
+        auto screen = [&](const f32x16& g, int qi, int qj) {
+            const int n = 32 * qj + (lane & 31);
+            const float nn = nrm[n];
+            const float tn = M.tau[n];
+            const int mbase = 32 * qi + 4 * (lane >> 5);
+            uint32_t bits = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int m = mbase + 8 * (i >> 2) + (i & 3);
+                const float S = nrm[m] + nn;
+                const float dt = __builtin_fmaf(-2.0f, g[i], S);
+                const float lower = (dt - __builtin_fmaf(c_err, S, 1e-35f)) * one_minus_gamma;
+                const bool drop = lower > fmaxf(M.tau[m], tn);                // false if anything is NaN
+                const bool valid = n < s && (qi == qj ? m < n : m < s);
+                if (valid && !drop) bits |= 1u << i;
+            }
+            const int cnt = __popc(bits);
+            int at = cnt ? atomicAdd(&M.n_pairs[0], cnt) : 0;
+            while (bits) {
+                const int i = __ffs(bits) - 1;
+                bits &= bits - 1;
+                const int m = mbase + 8 * (i >> 2) + (i & 3);
+                M.list[at++] = (uint16_t)(m | (n << 6));
+            }
+        };
+        if (act0) screen(g0, wave, wave);
+        if (act1) screen(g1, 0, 1);
     }
     __syncthreads();
-    const int n_list = *n_pairs;
-    const int rounds = (n_list + kThreads - 1) / kThreads;      // pairs per thread, at most kPairsPerThread
+    const int n_list = M.n_pairs[0];
+    if (n_list == 0) return;                          // no pair of this bucket can change a row
 
-    // ---- 2. exact distances of the listed pairs
-    float acc[kPairsPerThread];
+    // ---- 3. exact distances of the listed pairs: thread t takes entries t, t + 128, ...
+    const int rounds = (n_list + kThreads - 1) / kThreads;
+    float acc[kMaxRounds];
 #pragma unroll
-    for (int k = 0; k < kPairsPerThread; ++k) acc[k] = 0.0f;
-    auto consume = [&](float4 (&pre)[kLoads], int np_now, bool first) {
-        if (!first) __syncthreads();                 // the previous slice has been consumed
-        if (pc < np_now) {
+    for (int r = 0; r < kMaxRounds; ++r) acc[r] = 0.0f;
+    auto entry = [&](int r) {                         // idle threads compute pair (0, 0)
+        const int p = tid + r * kThreads;
+        return p < n_list ? (uint32_t)M.list[p] : 0u;
+    };
+    auto chains = [&](int np) {
 #pragma unroll
-            for (int i = 0; i < kLoads; ++i) {
-                const int m = rg + kRowsPerStep * i;
-                if (m < s) *reinterpret_cast<float4*>(&rows[m * pitch + 4 * pc]) = pre[i];
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < kPairsPerThread; ++k) {
-            if (k < rounds) {
-                const int p = tid + k * kThreads;
-                const uint32_t e = p < n_list ? list[p] : 0u;      // idle threads compute pair (0, 0)
-                const float* ra = rows + (e & 63u) * (uint32_t)pitch;
-                const float* rb = rows + (e >> 6) * (uint32_t)pitch;
-                float a = acc[k];
-                for (int q = 0; q < np_now; ++q) {
+        for (int r = 0; r < kMaxRounds; ++r) {
+            if (r < rounds) {
+                const uint32_t e = entry(r);
+                const float* ra = rows + (e & 63u) * (uint32_t)kPitch;
+                const float* rb = rows + (e >> 6) * (uint32_t)kPitch;
+                float a = acc[r];
+                for (int q = 0; q < np; ++q) {
                     const float4 x = *reinterpret_cast<const float4*>(ra + 4 * q);
                     const float4 y = *reinterpret_cast<const float4*>(rb + 4 * q);
                     float df;
@@ -240,56 +244,55 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                     df = x.z - y.z; a = __builtin_fmaf(df, df, a);
                     df = x.w - y.w; a = __builtin_fmaf(df, df, a);
                 }
-                acc[k] = a;
+                acc[r] = a;
             }
         }
     };
-    for (int d0 = 0; d0 < D; d0 += 2 * chunk) {
-        consume(preA, npA, d0 == 0);
-        if (d0 + 2 * chunk < D) npA = request(preA, d0 + 2 * chunk);
-        if (d0 + chunk < D) {
-            consume(preB, npB, false);
-            if (d0 + 3 * chunk < D) npB = request(preB, d0 + 3 * chunk);
+    if (SINGLE) {
+        chains((D + 3) >> 2);                         // the rows are still in LDS
+    } else {
+        ld.request(M.lids, s, points, D, 0, vec_ok);
+        for (int c = 0; c < n_chunks; ++c) {
+            __syncthreads();
+            ld.commit(rows, kPitch);
+            __syncthreads();
+            if (c + 1 < n_chunks) ld.request(M.lids, s, points, D, (c + 1) * kChunk, vec_ok);
+            chains(min(kChunk, (D - c * kChunk + 3) & ~3) >> 2);
         }
     }
-    __syncthreads();                           // rows no longer needed: the region becomes the distance matrix
-    const int n_tri = (s * (s - 1)) >> 1;
-    for (int i = tid; i < n_tri; i += kThreads) tri[i] = INFINITY;
+    __syncthreads();                                  // rows no longer needed: the region becomes the distance matrix
+    for (int i = tid; i < kCap * kDistPitch; i += kThreads) dist[i] = INFINITY;
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < kPairsPerThread; ++k) {
-        const int p = tid + k * kThreads;
-        if (p < n_list) {
-            const uint32_t e = list[p];
-            const int r = (int)(e & 63u), c = (int)(e >> 6);
-            const float d = acc[k];
-            tri[tri_at(r, c)] = d;
-            if (d <= tau[r]) flag[r] = 1;            // plain stores of the same value: no ordering needed
-            if (d <= tau[c]) flag[c] = 1;
+    for (int r = 0; r < kMaxRounds; ++r) {
+        if (tid + r * kThreads < n_list) {
+            const uint32_t e = entry(r);
+            const int i = (int)(e & 63u), j = (int)(e >> 6);
+            const float d = acc[r];
+            dist[i * kDistPitch + j] = d;
+            dist[j * kDistPitch + i] = d;
+            if (d <= M.tau[i]) M.flag[i] = 1;         // plain stores of the same value: no ordering needed
+            if (d <= M.tau[j]) M.flag[j] = 1;
         }
     }
     __syncthreads();
 
-    // ---- 3. top-K update.  A wavefront owns every second member and walks those that have a candidate below
-    //         their last slot, with the rows of the next two in flight.
-    const int my_id = lids[lane];
-    // bit u: member wave + 2 u has a candidate
-    uint32_t active = (uint32_t)ballot64(lane < 32 && flag[(wave + kWaves * lane) & (kCap - 1)] != 0);
-    auto candidate = [&](int i) {
-        const int a = min(i, lane), b = max(i, lane);
-        return (lane < s && lane != i) ? tri[tri_at(a, b)] : INFINITY;
-    };
+    // ---- 4. top-K update: a wavefront walks its members that have a candidate, four at a time, with the rows of the
+    //         next four in flight
+    const int my_id = M.lids[lane];
+    const int fm = wave + 2 * lane;                   // bit u: member wave + 2 u has a candidate
+    uint32_t active = (uint32_t)ballot64(lane < 32 && M.flag[fm < kCap ? fm : 0] != 0);
     auto next_member = [&]() {
         if (active == 0) return -1;
         const int u = __ffs(active) - 1;
         active &= active - 1;
-        return wave + kWaves * u;
+        return wave + 2 * u;
     };
     auto load_row = [&](int i, int& ri, float& rd) {
         ri = -2;
         rd = INFINITY;
         if (i >= 0 && lane < K) {
-            const size_t at = (size_t)lids[i] * (size_t)K + lane;
+            const size_t at = (size_t)M.lids[i] * (size_t)K + lane;
             ri = knn_idx[at];
             rd = knn_dist[at];
         }
@@ -312,14 +315,13 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         for (int u = 0; u < kAhead; ++u) {
             const int i = cur_i[u];
             if (i < 0) break;
-            const float d = candidate(i);
             KnnRow<1> row;
             row.idx[0] = cur_ri[u];
             row.dist[0] = cur_rd[u];
             row.init_sorted(K);
-            row.merge(lane < s && lane != i, my_id, d);
+            row.merge(lane < s && lane != i, my_id, dist[i * kDistPitch + lane]);
             if (row.changed) {
-                const size_t at = (size_t)lids[i] * (size_t)K;
+                const size_t at = (size_t)M.lids[i] * (size_t)K;
                 row.store(knn_idx + at, knn_dist + at);
             }
         }
@@ -353,36 +355,37 @@ int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t st
     return 0;
 }
 
-// Buckets of at most 64 points given by (starts, sizes); rows sorted on entry.
-int launch_bucket_knn_screen(const float* points, const Bf16Copy& bf, int D, int K, const int* ids, const int* starts,
-                             const int* sizes, int n_buckets, int* knn_idx, float* knn_dist, hipStream_t stream)
+// Buckets of 2..64 points (others are skipped); every K-NN row sorted on entry.
+int launch_bucket_knn_screen(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                             int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream)
 {
     if (n_buckets <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 64, "screened small-bucket kernel: K must be in 1..64");
-    RSFK_CHECK(bf.rows != nullptr && bf.norms != nullptr && starts != nullptr, "screened small-bucket kernel: missing input");
-    const int dpad = (D + 3) & ~3;
-    const int n_slices = (dpad + kMaxChunk - 1) / kMaxChunk;
-    const int chunk = (((dpad + n_slices - 1) / n_slices) + 3) & ~3;
-    RSFK_CHECK(chunk >= 4 && chunk <= kMaxChunk, "screened small-bucket kernel: slice width");
-    int pitch = chunk;
-    if (((pitch >> 2) & 1) == 0) pitch += 4;              // odd number of 16-byte units: rows start in different banks
-    RSFK_CHECK(kCap * pitch < 65536, "screened small-bucket kernel: LDS offsets must fit 16 bits");
-    const int region = std::max(kCap * pitch, kMaxPairs);
-    const int region_floats = (region + 3) & ~3;
-    const size_t lds = (size_t)region_floats * 4 + (size_t)(5 * kCap + 4) * 4 + (size_t)kMaxPairs * 2;
-    const int ksteps = (bf16_valid(D) + 15) / 16;
-    RSFK_CHECK(ksteps * 16 <= bf16_pitch(D), "screened small-bucket kernel: bfloat16 rows too short");
-    const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21
-    const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
+    RSFK_CHECK(K >= 1 && K <= 64 && D >= 1, "screened small-bucket kernel: K must be in 1..64 and D positive");
+    const float c_err = split_gram_error_coefficient((D + 15) & ~15);
+    const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);
     RSFK_CHECK(one_minus_gamma > 0.5f, "screened small-bucket kernel: D too large");
-    const float inv_one_minus_gamma = 1.000001f / one_minus_gamma;                  // rounded up
-    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bucket_knn_screen),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(k_bucket_knn_screen, dim3((unsigned)n_buckets), dim3(kThreads), lds, stream, points, bf.rows,
-                       bf.norms, D, K, ids, starts, sizes, knn_idx, knn_dist, chunk, pitch, region_floats,
-                       bf16_pitch(D), ksteps, kappa, inv_one_minus_gamma);
+    const dim3 grid((unsigned)n_buckets), block(kThreads);
+    if (D <= kChunk)
+        hipLaunchKernelGGL(k_bucket_knn_screen<true>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx,
+                           knn_dist, c_err, one_minus_gamma);
+    else
+        hipLaunchKernelGGL(k_bucket_knn_screen<false>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx,
+                           knn_dist, c_err, one_minus_gamma);
     RSFK_HIP(hipGetLastError());
     return 0;
+}
+
+// First tree of a build whose small buckets take the screened kernel (later trees too).  RSFK_BUCKET_SCREEN=<tree>
+// overrides (0 = every tree and the stage-level call, "off" = never).
+int bucket_screen_from(int D, int K)
+{
+    if (K > 64) return 0x7fffffff;
+    const char* e = std::getenv("RSFK_BUCKET_SCREEN");
+    if (e && *e) return (e[0] >= '0' && e[0] <= '9') ? std::atoi(e) : 0x7fffffff;
+    // The first trees of a build change most rows with most pairs, and every pair that passes the screen costs more
+    // here than in the direct kernel; measured on uniform (D = 100) and clustered (D = 256) points the screened kernel
+    // is the faster one from the 8th and the 4th tree on.
+    return D >= 128 ? 4 : 8;
 }
 
 }  // namespace rsfk

@@ -147,10 +147,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (bf16_copy_alloc(&bf.c, N, D)) return 1;
     if (bf16_copy_fill(bf.c, d_points, N, D, stream)) return 1;
 
-    // RSFK_BUCKET_SCREEN=1 sends the small buckets to the kernel that screens pairs on the bfloat16 copy
-    // before computing exact distances (same results; not faster on the workloads measured so far)
-    const char* env_screen = std::getenv("RSFK_BUCKET_SCREEN");
-    const bool screen = K <= 64 && env_screen && env_screen[0] == '1';
+    const int screen_from = bucket_screen_from(D, K);
 
     Q8Guard q8;
     const uint8_t* q8_rows = nullptr;
@@ -192,11 +189,11 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                     (void)hipStreamWaitEvent(sync.side, sync.start, 0);
                 }
                 const bool gram = t0 + j >= gram_from;
-                rc = launch_bucket_knn_tree(d_points, screen ? &bf.c : nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                rc = launch_bucket_knn_tree(d_points, t0 + j >= screen_from, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
                                             d_idx, d_dist, stream, split ? 1 : 0);
                 if (!rc && split) {
-                    rc = launch_bucket_knn_tree(d_points, nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                    rc = launch_bucket_knn_tree(d_points, false, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
                                                 stats[5 * j + 2], d_idx, d_dist, sync.side, 2);
                     (void)hipEventRecord(sync.big, sync.side);

@@ -86,12 +86,18 @@ def test_tree_edge_cases(gpu, orc, rng):
     (1200, 1, 4, 5, 10), (2500, 3, 1, 2, 4), (2000, 130, 64, 65, 130), (1500, 20, 65, 66, 140),
     (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
 ])
-@pytest.mark.parametrize("kernel", ["direct", "gram"])
+@pytest.mark.parametrize("kernel", ["direct", "gram", "screen"])
 def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
     """kernel: "direct" = fp32 chains for every pair; "gram" = the kernel that bounds the pair matrix on the matrix
-    cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0)."""
+    cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0); "screen" = the same
+    idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=0; other buckets, and K > 64,
+    take the direct kernels)."""
     if kernel == "gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "0")
+    if kernel == "screen":
+        if K > 64 or MIN > 64:
+            pytest.skip("no bucket of this shape reaches the screened small-bucket kernel")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "0")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K)
     gi, gd = orc.init_lists(N, K)
@@ -226,7 +232,7 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
 def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, T, kw, variant):
     import gpu_rsfk
     if variant == "bucket_screen":
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")       # every tree but the first through the screened small-bucket kernel
     X = rng.standard_normal((N, D)).astype(np.float32)
     r = gpu_rsfk.RSFK(random_state=17)
     _say("forest", N, D, K, T, kw)
@@ -250,11 +256,17 @@ def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D,
     ("c4", 9000, 90, 4, dict(nn_exploring_factor=1)),
     ("c5", 70000, 32, 5, dict(min_tree_children=64, max_tree_children=256)),
 ], ids=["config3_gmm64_d256_k32", "config4_sparse_d784_k90_explore", "config5_normal_d32_buckets64_256"])
-@pytest.mark.parametrize("kernel", ["direct", "gram"])
+@pytest.mark.parametrize("kernel", ["direct", "gram", "screen"])
 def test_baseline_config_workloads_match_oracle(gpu, orc, monkeypatch, config, N, K, T, kw, kernel):
     import gpu_rsfk
     if kernel == "gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "1")          # every tree but the first through the screened bucket kernel
+    if kernel == "screen":
+        if config != "c3":
+            pytest.skip("no bucket of this configuration reaches the screened small-bucket kernel")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
+    else:
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "off")
     X = baseline_points(config, N)
     r = gpu_rsfk.RSFK(random_state=0)
     _say("forest", config, N, X.shape[1], K, T, kw)
@@ -452,11 +464,12 @@ def _hard_inputs(rng, kind, N, D):
 def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant):
     """The bfloat16 screens only skip work whose outcome is certain: trees, bucket K-NN and exploration on inputs
     that defeat a 8-bit mantissa must still be identical to the fp32 oracle.  "bucket_screen" also switches the
-    small buckets to the kernel that screens pairs with the matrix cores on the bfloat16 copy (RSFK_BUCKET_SCREEN=1),
-    "bucket_gram" all buckets to the one that splits the fp32 rows into two bfloat16 numbers (RSFK_GRAM_FROM=0)."""
+    buckets of up to 64 points to the two-wavefront kernel that bounds the pair matrix on the matrix cores
+    (RSFK_BUCKET_SCREEN=0: every tree and the stage-level call), "bucket_gram" all buckets to the tiled kernel that
+    does the same (RSFK_GRAM_FROM=0)."""
     import gpu_rsfk
     if variant == "bucket_screen":
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "0")
     if variant == "bucket_gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     N, D, K = 6000, 24, 10
