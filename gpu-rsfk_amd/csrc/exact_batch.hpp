@@ -39,10 +39,15 @@ __device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int 
 }
 
 // Exact distances of the first n candidates of `list` to the point, then offer them.  CH = dimensions
-// staged per step (32 or 16): a step moves 64 rows x CH floats through the tile.
-template <int SL, int CH = kChunk>
+// staged per step (32 or 16): a step moves 64 rows x CH floats through the tile.  tau_cap: a bound the caller
+// knows for the row's final last slot (candidates above it need not be finished), else +inf.  DEEP: the loads of
+// two steps are in flight while a third is being used (two register buffers that take turns, so that waiting for
+// one does not wait for the other): for kernels with few wavefronts per SIMD, whose gathers would otherwise wait
+// for each other.
+template <int SL, int CH = kChunk, bool DEEP = false>
 __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
-                                            const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row)
+                                            const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row,
+                                            float tau_cap = INFINITY)
 {
     constexpr int kPieces = CH / 4;         // 16-byte pieces of a row per step = lanes per row
     constexpr int kRows = 64 / kPieces;     // rows per load instruction
@@ -56,22 +61,26 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
         const int r = i * kRows + sub;
-        rp[i] = points + (size_t)list[r < n ? r : 0] * (size_t)D;      // rows beyond n repeat row 0 (ignored later)
+        rp[i] = r < n ? points + (size_t)list[r] * (size_t)D : nullptr;    // nothing is read for the rows beyond n
     }
-    float4 pre[kLoads];
+    float4 pre[DEEP ? 2 : 1][kLoads];
+    auto request = [&](float4 (&buf)[kLoads], int d0) {
+        if (d0 < D) {
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], piece * 4, D, vec_ok);
+            for (int i = 0; i < kLoads; ++i)
+                buf[i] = rp[i] ? load_piece(rp[i], d0 + piece * 4, D, vec_ok) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
     float acc = 0.0f;
-    const float tau0 = row.tau;
-    for (int d0 = 0; d0 < D; d0 += CH) {
+    const float tau0 = fminf(row.tau, tau_cap);
+    // one step: the buffer's values (dimensions d0 ..) go through the tile, the buffer is refilled with the step
+    // `ahead` dimensions later, the chains advance.  Returns false when no candidate can enter any more.
+    auto step = [&](float4 (&buf)[kLoads], int d0, int ahead) {
         wave_lds_sync();                 // previous step's tile reads are done
 #pragma unroll
         for (int i = 0; i < kLoads; ++i)
-            *reinterpret_cast<float4*>(&L.tile[(i * kRows + sub) * kP + piece * 4]) = pre[i];
-        if (d0 + CH < D) {
-#pragma unroll
-            for (int i = 0; i < kLoads; ++i) pre[i] = load_piece(rp[i], d0 + CH + piece * 4, D, vec_ok);
-        }
+            *reinterpret_cast<float4*>(&L.tile[(i * kRows + sub) * kP + piece * 4]) = buf[i];
+        request(buf, d0 + ahead);
         wave_lds_sync();
         const int pieces = min(kPieces, (D - d0 + 3) >> 2);
         const float* mine = &L.tile[lane * kP];
@@ -86,10 +95,22 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
             df = a.w - x.w; acc = __builtin_fmaf(df, df, acc);
         }
         // partial sums only grow: once all of them are above the row maximum nothing can enter
-        if (ballot64(lane < n && acc <= tau0) == 0) break;
+        return ballot64(lane < n && acc <= tau0) != 0;
+    };
+    bool finished = true;
+    request(pre[0], 0);
+    if (DEEP) {
+        request(pre[1], CH);
+        for (int d0 = 0; d0 < D; d0 += 2 * CH) {
+            if (!step(pre[0], d0, 2 * CH)) { finished = false; break; }
+            if (d0 + CH < D && !step(pre[1], d0 + CH, 2 * CH)) { finished = false; break; }
+        }
+    } else {
+        for (int d0 = 0; d0 < D; d0 += CH)
+            if (!step(pre[0], d0, CH)) { finished = false; break; }
     }
     wave_lds_sync();
-    row.merge(lane < n, my_c, acc);
+    row.merge(lane < n && finished, my_c, acc);          // unfinished sums are all above the last slot
 }
 
 }  // namespace rsfk

@@ -416,160 +416,259 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
 
-// The same for rows so long that the set of one point takes most of the LDS a wavefront could get (K above 64: a point
-// has up to K^2 marks): one workgroup of four wavefronts per point.  The first wavefront gathers the marked ids into
-// the set and compacts it (as above); then every wavefront takes every fourth batch of 64 candidates with its own
-// copy of the row and its own tile, and the first one merges the four rows and stores the result.
-// LDS (ints): table[table_size] | srow[K] | xrow[dpad] | region, region = marked[3/4 table_size] first, then
-// 4 tiles + 3 rows for the exchange.  Rows pass through the tiles 32 dimensions at a time (whole 128-byte lines).
+// The same for rows so long that the set of one point takes most of the LDS a wavefront could get (K above about 45:
+// a point has up to K^2 marks): one workgroup of four wavefronts per point, and the candidates are taken in the
+// order of their lower bounds.
+//
+// A candidate can only end up in the row if its exact distance is at most the row's last slot at the end, and that
+// slot falls fast once the nearest candidates are in.  In the order of the marks most candidates enter at some
+// moment and are pushed out again later (three quarters of them on 70,000 x 784 rows with K = 90), each at the price
+// of gathering a whole fp32 row.  Here:
+//   1. all threads list the marked (neighbour, slot) pairs of the point together with the lower bound L the join
+//      kept for each (explore_join.hip; 0 when it kept none), one 32-bit word per pair;
+//   2. every wavefront walks its quarter of the list kWgRounds times with a rising limit -- the distances at the
+//      1/8, 2/8, ... of its own copy of the row, which improves from round to round, capped by the smallest last slot
+//      any wavefront has reached (shared through LDS) -- and takes the pairs whose bound lies between the previous
+//      limit and this one: near candidates first, without sorting anything.  A pair whose bound is above the shared
+//      last slot at its turn is never looked at.  The others have their id read, pass through a hash set (seeded
+//      with the row; drops repeats -- only a saving: a repeated candidate would be rejected by the row), wait until 64
+//      of them are together, get the exact distance and are merged into the wavefront's copy of the row;
+//   3. the first wavefront merges the four rows and stores the result.
+// A bound is below the exact distance of its pair, the shared last slot is never below the final one: a dropped
+// candidate could not have been in the final row, so the result is the one of any other order.
+// (Sorting the list by the bounds first, a bitonic network over up to 4096 words in LDS, cost more than it saved.)
+// LDS (ints): table[kWgTable] | srow[K] | jrow[K] | xrow[dpad] | marked[cap] | 4 tiles | 3 rows for the exchange | 4 x 128 ids.
 constexpr int kWgChunk = 32;
 constexpr int kWgTile = 64 * (kWgChunk + 4);
+constexpr int kWgTable = 2048;              // hash set; when three quarters are taken, new ids are no longer recorded
+constexpr int kWgMinCap = 1024;             // the kernel is not used when fewer marks than this would fit
+
+constexpr int kWgRounds = 8;
+constexpr int kWgMaxCap = 6656;             // marks per point: 26 steps of the walk of a wavefront
+constexpr int kWgMaxSteps = kWgMaxCap / 256;
+
+// distance in slot k of a row (k is the same in all lanes)
+template <int SL>
+__device__ __forceinline__ float row_slot_dist(const KnnRow<SL>& row, int k)
+{
+    float v = INFINITY;
+#pragma unroll
+    for (int s = 0; s < SL; ++s)
+        if ((k >> 6) == s) v = read_lane_f(row.dist[s], k & 63);
+    return v;
+}
+
 template <int SL>
 __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restrict__ points, int N, int D, int K,
                                                           const int* __restrict__ old_idx, int* __restrict__ knn_idx,
-                                                          float* __restrict__ knn_dist, int table_size, int dpad,
+                                                          float* __restrict__ knn_dist, int cap, int dpad,
                                                           const int* __restrict__ fwd2rev, const uint32_t* __restrict__ pass,
+                                                          const uint16_t* __restrict__ bounds,
                                                           const int* __restrict__ todo_in, int n_in,
                                                           int* __restrict__ todo_out, int* __restrict__ n_out)
 {
     extern __shared__ __align__(16) int lds_w[];
-    __shared__ int U_s;
+    __shared__ int wave_tot[4];
+    __shared__ int n_set_s;
+    __shared__ uint32_t tau_s;                                    // bits of the smallest last slot reached so far
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int slot = blockIdx.x;
     if (slot >= (todo_in ? n_in : N)) return;
     const int p = todo_in ? todo_in[slot] : slot;
-    const int MW = (K + 31) >> 5;
+    const int MW = (K + 31) >> 5, KP = MW * 32;
     int* table = lds_w;
-    int* srow = table + table_size;
-    float* xrow = reinterpret_cast<float*>(srow + ((K + 3) & ~3));
-    int* region = reinterpret_cast<int*>(xrow + dpad);
+    int* srow = table + kWgTable;
+    int* jrow = srow + ((K + 3) & ~3);                            // place of graph entry (p, k) in the reversed graph
+    float* xrow = reinterpret_cast<float*>(jrow + ((K + 3) & ~3));
+    uint32_t* marked = reinterpret_cast<uint32_t*>(xrow + dpad);
+    int* tiles = reinterpret_cast<int*>(marked + cap);
+    int* xch = tiles + 4 * kWgTile;                               // rows on their way to another wavefront: [3][idx | dist][64 SL]
+    int* ids = xch + 6 * 64 * SL + 128 * wave;                    // this wavefront's candidates: a batch and what is left over
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
     KnnRow<SL> row;
     row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
-    for (int k = threadIdx.x; k < K; k += 256) srow[k] = old_idx[(size_t)p * K + k];
     const float* xp = points + (size_t)p * D;
     for (int d = threadIdx.x; d < dpad; d += 256) xrow[d] = d < D ? xp[d] : 0.0f;
-    if (threadIdx.x == 0) U_s = 0;
-    __syncthreads();
-    if (wave == 0) {
-        int bits = 0;
-        for (int k = lane; k < K; k += 64) {
-            const int j = fwd2rev[(size_t)p * K + k];
-            if (j >= 0)
-                for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
-        }
-        const int n_given = wave_sum_i(bits);
-        int U = 0;
-        if (n_given + K + 1 > table_size / 4 * 3) {
-            if (lane == 0) todo_out[atomicAdd(n_out, 1)] = p;
-        } else if (n_given > 0) {
-            int ts = 64;
-            while (ts < 2 * (n_given + K + 1)) ts <<= 1;
-            ts = min(ts, table_size);
-            const int mask = ts - 1;
-            for (int i = lane; i < ts; i += 64) table[i] = kEmpty;
-            wave_lds_sync();
-            if (lane == 0) set_insert(table, mask, p, true);
-#pragma unroll
-            for (int s = 0; s < SL; ++s)
-                if (row.idx[s] >= 0) set_insert(table, mask, row.idx[s], true);
-            int* marked = region;
-            int n_marked = 0;                                     // wave-uniform
-            for (int k0 = 0; k0 < K; k0 += 64) {
-                const int k = k0 + lane;
-                const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
-                int mine = 0;
-                if (j >= 0)
-                    for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
-                int at = n_marked + wave_excl_scan_i(mine);
-                if (j >= 0) {
-                    for (int w = 0; w < MW; ++w) {
-                        uint32_t m = pass[(size_t)j * MW + w];
-                        while (m) {
-                            const int b = __ffs(m) - 1;
-                            m &= m - 1;
-                            marked[at++] = k | ((32 * w + b) << 8);
-                        }
-                    }
-                }
-                n_marked += wave_sum_i(mine);
-            }
-            wave_lds_sync();
-            for (int i0 = 0; i0 < n_marked; i0 += 64) {
-                const int i = i0 + lane;
-                int c = -1;
-                if (i < n_marked) {
-                    const int e = marked[i];
-                    c = old_idx[(size_t)srow[e & 255] * K + (e >> 8)];
-                }
-                if (c >= 0 && c < N) set_insert(table, mask, c, false);
-            }
-            wave_lds_sync();
-            for (int t0 = 0; t0 < ts; t0 += 64) {                 // compact the set in place into the candidate list
-                const int v = table[t0 + lane];
-                const bool is_cand = v >= 0;
-                const uint64_t m = ballot64(is_cand);
-                wave_lds_sync();
-                if (is_cand) table[U + mask_prefix(m)] = v;
-                U += __popcll(m);
-            }
-        }
-        if (lane == 0) U_s = U;
+    for (int i = threadIdx.x; i < kWgTable; i += 256) table[i] = kEmpty;
+
+    // ---- 1. the marked pairs of the point; thread k takes neighbour k (K <= 256)
+    const int k = threadIdx.x;
+    const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
+    if (k < K) {
+        srow[k] = old_idx[(size_t)p * K + k];
+        jrow[k] = j;
     }
-    __syncthreads();                                              // the list is complete, `marked` is free
-    const int U = U_s;
-    if (U <= 0) return;
+    int mine = 0;
+    if (j >= 0)
+        for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
+    const int in_wave = wave_excl_scan_i(mine);
+    if (lane == 63) wave_tot[wave] = in_wave + mine;
+    if (threadIdx.x == 0) {
+        n_set_s = 0;
+        tau_s = __float_as_uint(row.tau);
+    }
+    __syncthreads();
+    int at = in_wave, n_marked = 0;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        if (w < wave) at += wave_tot[w];
+        n_marked += wave_tot[w];
+    }
+    if (n_marked == 0) return;
+    if (n_marked > cap) {
+        if (threadIdx.x == 0) todo_out[atomicAdd(n_out, 1)] = p;
+        return;
+    }
+    if (j >= 0) {
+        for (int w = 0; w < MW; ++w) {
+            uint32_t m = pass[(size_t)j * MW + w];
+            while (m) {
+                const int b = __ffs(m) - 1;
+                m &= m - 1;
+                marked[at++] = (uint32_t)((32 * w + b) << 8) | (uint32_t)k;
+            }
+        }
+    }
+    if (wave == 0) {                                              // seeds: ids that are in the row already
+        const int mask = kWgTable - 1;
+        int seeded = 0;
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+            if (row.idx[s] >= 0) { set_insert(table, mask, row.idx[s], true); ++seeded; }
+        seeded = wave_sum_i(seeded);
+        if (lane == 0) atomicAdd(&n_set_s, seeded);
+    }
+    __syncthreads();
+    if (bounds) {
+        // the bounds of the listed pairs, by all threads (a thread's own marks one after the other would wait for
+        // one 2-byte read at a time)
+        for (int i0 = threadIdx.x; i0 < n_marked; i0 += 4 * 256) {
+            uint32_t e[4], lb[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + 256 * u;
+                e[u] = i < n_marked ? marked[i] : 0u;
+                lb[u] = i < n_marked ? (uint32_t)bounds[(size_t)jrow[e[u] & 255u] * KP + ((e[u] >> 8) & 255u)] : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (i0 + 256 * u < n_marked) marked[i0 + 256 * u] = e[u] | (lb[u] << 16);
+        }
+        __syncthreads();
+    }
+
+    // ---- 2. my quarter of the list, nearer bounds first
     ExploreLds L;
-    L.tile = reinterpret_cast<float*>(region + wave * kWgTile);
+    L.tile = reinterpret_cast<float*>(tiles + wave * kWgTile);
     L.xrow = xrow;
     L.queue2 = nullptr;
     L.table = nullptr;
     L.srow = nullptr;
-    for (int off = 64 * wave; off < U; off += 256) {
+    int have = 0;                                                 // candidates waiting in ids (wave-uniform)
+    auto run_batch = [&]() {
         wave_lds_sync();
-        exact_batch<SL, kWgChunk>(L, table + off, min(64, U - off), points, D, vec_ok, row);
-    }
-    int* xch = region + 4 * kWgTile;                           // rows of the wavefronts 1..3: [w - 1][idx | dist][64 SL]
-    if (wave > 0) {
+        const int n_now = min(64, have);
+        const float cap_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
+        exact_batch<SL, kWgChunk, true>(L, ids, n_now, points, D, vec_ok, row, cap_now);
+        if (lane == 0) atomicMin(&tau_s, __float_as_uint(row.tau));   // non-negative floats order like their bits
+        have -= n_now;
+        const int left = lane < have ? ids[64 + lane] : 0;        // the candidates beyond the batch move to the front
+        wave_lds_sync();
+        if (lane < have) ids[lane] = left;
+    };
+    float prev = -1.0f;                                           // bounds are never negative
+    for (int r = 0; r < kWgRounds; ++r) {
+        const float thr = r + 1 < kWgRounds ? row_slot_dist(row, max(0, K * (r + 1) / kWgRounds - 1)) : INFINITY;
+        if (!(thr > prev)) continue;
+        // first the ids of everything this round takes (all reads travel together), then the candidates one step
+        // of the walk after the other
+        const float tau_round = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
+        const float lim = fminf(thr, tau_round);
+        int c[kWgMaxSteps];
 #pragma unroll
-        for (int s = 0; s < SL; ++s) {
-            xch[((wave - 1) * 2 + 0) * (64 * SL) + lane + 64 * s] = row.idx[s];
-            xch[((wave - 1) * 2 + 1) * (64 * SL) + lane + 64 * s] = __float_as_int(row.dist[s]);
-        }
-    }
-    __syncthreads();
-    if (wave == 0) {
-        for (int w = 0; w < 3; ++w) {
-#pragma unroll
-            for (int s = 0; s < SL; ++s) {
-                const int c = xch[(w * 2 + 0) * (64 * SL) + lane + 64 * s];
-                const float d = __int_as_float(xch[(w * 2 + 1) * (64 * SL) + lane + 64 * s]);
-                row.merge(lane + 64 * s < K && c >= 0, c, d);
+        for (int u = 0; u < kWgMaxSteps; ++u) {
+            const int at = 64 * wave + 256 * u + lane;
+            c[u] = -1;
+            if (at < n_marked) {
+                const uint32_t e = marked[at];
+                const float lb = __uint_as_float(e & 0xffff0000u);
+                if (lb > prev && !(lb > lim)) c[u] = old_idx[(size_t)srow[e & 255u] * K + ((e >> 8) & 255u)];
             }
         }
+#pragma unroll
+        for (int u = 0; u < kWgMaxSteps; ++u) {
+            if (64 * wave + 256 * u >= n_marked) break;
+            bool fresh = c[u] >= 0 && c[u] < N && c[u] != p;
+            if (ballot64(fresh) == 0) continue;
+            // the shared last slot may have fallen since the ids were requested
+            const int at = 64 * wave + 256 * u + lane;
+            const float tau_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
+            if (fresh && __uint_as_float(marked[at] & 0xffff0000u) > tau_now) fresh = false;
+            if (fresh && *reinterpret_cast<volatile int*>(&n_set_s) < kWgTable / 4 * 3) {
+                fresh = set_insert(table, kWgTable - 1, c[u], false);
+                if (fresh) atomicAdd(&n_set_s, 1);
+            }
+            const uint64_t fm = ballot64(fresh);
+            if (fresh) ids[have + mask_prefix(fm)] = c[u];        // have < 64 here: at most 127 entries
+            have += __popcll(fm);
+            if (have >= 64) run_batch();
+        }
+        prev = thr;
+    }
+    if (have > 0) run_batch();
+
+    // ---- 3. one row out of four: wavefronts 0 and 1 take the rows of 2 and 3, then 0 takes the row of 1
+    auto put_row = [&](int at) {
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            xch[(at * 2 + 0) * (64 * SL) + lane + 64 * s] = row.idx[s];
+            xch[(at * 2 + 1) * (64 * SL) + lane + 64 * s] = __float_as_int(row.dist[s]);
+        }
+    };
+    auto take_row = [&](int at) {
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            const int c = xch[(at * 2 + 0) * (64 * SL) + lane + 64 * s];
+            const float d = __int_as_float(xch[(at * 2 + 1) * (64 * SL) + lane + 64 * s]);
+            row.merge(lane + 64 * s < K && c >= 0, c, d);
+        }
+    };
+    if (wave >= 2) put_row(wave - 2);
+    __syncthreads();
+    if (wave < 2) take_row(wave);
+    if (wave == 1) put_row(2);
+    __syncthreads();
+    if (wave == 0) {
+        take_row(2);
         if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
     }
 }
 
-// ints of LDS the workgroup-per-point merge needs for a set of `table` entries
-int merge_wg_ints(int table, int dpad, int K, int sl)
+// marks per point the workgroup-per-point merge can take with the LDS of a compute unit shared by two workgroups
+int merge_wg_cap(int dpad, int K, int sl)
 {
-    const int region = std::max(table / 4 * 3, 4 * kWgTile + 6 * 64 * sl);
-    return (table + ((K + 3) & ~3) + dpad + region + 3) / 4 * 4;
+    const int budget = 78 * 1024 / 4;
+    const int fixed = kWgTable + 2 * ((K + 3) & ~3) + dpad + 4 * kWgTile + 6 * 64 * sl + 4 * 128;
+    return std::min(std::min(budget - fixed, K * K), kWgMaxCap);
+}
+
+int merge_wg_ints(int cap, int dpad, int K, int sl)
+{
+    return (kWgTable + 2 * ((K + 3) & ~3) + dpad + cap + 4 * kWgTile + 6 * 64 * sl + 4 * 128 + 3) / 4 * 4;
 }
 
 template <int SL>
-int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
-                    int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in, int n_in, int* todo_out,
-                    int* n_out, hipStream_t stream)
+int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int cap,
+                    int dpad, const int* fwd2rev, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
+                    int* todo_out, int* n_out, hipStream_t stream)
 {
-    const size_t lds = (size_t)merge_wg_ints(table, dpad, K, SL) * sizeof(int);
+    const size_t lds = (size_t)merge_wg_ints(cap, dpad, K, SL) * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge_wg<SL>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
     hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3((unsigned)n_work), dim3(256), lds, stream, points, N, D, K, old_idx,
-                       knn_idx, knn_dist, table, dpad, fwd2rev, pass, todo_in, n_in, todo_out, n_out);
+                       knn_idx, knn_dist, cap, dpad, fwd2rev, pass, bounds, todo_in, n_in, todo_out, n_out);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -634,6 +733,18 @@ int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, cons
 
 }  // namespace
 
+bool explore_merge_uses_bounds(int D, int K)
+{
+    const int dpad = bf16_valid(D);
+    const int lds_ints = 150 * 1024 / 4;
+    const int sl = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
+    const int want = std::max(next_pow2(K * K + K + 2), next_pow2(4 * K + 66));
+    int big_waves = 4;
+    while (big_waves > 1 && merge_wave_ints(want, dpad, K) > lds_ints / big_waves) big_waves >>= 1;
+    return big_waves < 4 && merge_wg_cap(dpad, K, sl) >= kWgMinCap;
+}
+
+
 // One exploration pass.  old_idx is scratch of N*K ints (receives the snapshot).
 // bf may be null (or hold null rows): every candidate then gets the exact distance.
 // ws may be null; with a workspace and a bfloat16 copy for the join (bf_join, may be centred; bf must not be)
@@ -697,26 +808,24 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         // fewer than four wavefronts per workgroup would leave the compute units nearly empty: such sets get one
         // workgroup per point instead
         const bool per_wg = big_waves < 4;
-        if (per_wg) {
-            big_table = want;
-            while (big_table > small_table && merge_wg_ints(big_table, dpad, K, sl) > lds_ints) big_table >>= 1;
-        } else {
+        const int wg_cap = merge_wg_cap(dpad, K, sl);
+        if (!per_wg)
             while (big_table > small_table && merge_wave_ints(big_table, dpad, K) > lds_ints / big_waves) big_table >>= 1;
-        }
-        if (big_table > small_table) {
+        if (per_wg ? wg_cap >= kWgMinCap : big_table > small_table) {
+            const uint16_t* bounds = explore_ws_bounds(ws);
             int rc = 0;
             if (!per_wg)
                 rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass,
                                     listA, n_todo, listB, listB + N, stream);
             else if (sl == 1)
-                rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
-                                        listB, listB + N, stream);
+                rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                                        n_todo, listB, listB + N, stream);
             else if (sl == 2)
-                rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
-                                        listB, listB + N, stream);
+                rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                                        n_todo, listB, listB + N, stream);
             else
-                rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass, listA, n_todo,
-                                        listB, listB + N, stream);
+                rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                                        n_todo, listB, listB + N, stream);
             if (rc)
                 return 1;
             RSFK_HIP(hipMemcpyAsync(host_n, listB + N, sizeof(int), hipMemcpyDeviceToHost, stream));

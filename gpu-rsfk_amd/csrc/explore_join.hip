@@ -7,15 +7,22 @@
 // of a 32 x 32 tile come from one chain of matrix-core instructions on the bfloat16
 // copy of the points (v_mfma_f32_32x32x16_bf16: Gram matrix G, d~ = n_p + n_c - 2 G).
 //
-// d~ is only used to discard: with the error bound of bucket_knn_screen.hip (bfloat16
-// rounding via Cauchy-Schwarz, accumulation errors relative to n_p + n_c) a pair is
-// dropped when the exact fp32 distance provably is not below the last slot of row p.
+// d~ is only used to discard.  With S = n_p + n_c (norms of the bfloat16 rows), u = 2^-8:
+//   rounding to bfloat16:   |d(real) - d~(real)| <= 2u sqrt(d~ Q) + u^2 Q,  Q = 2 S  (Cauchy-Schwarz)
+//   Gram matrix and norms:  |d~(computed) - d~(real)| <= E1 = (D' + 16) 2^-21 S
+//   fp32 chain:             result >= d(real) (1 - gamma),  gamma = (D + 8) 2^-22
+// so L = (d~ - E1 - 1.01 (2u sqrt((d~ + E1) Q) + u^2 Q)) (1 - gamma) is a lower bound of the exact fp32
+// distance, and a pair is dropped when L is above the last slot of row p.
 // The outcome is one bit per (entry of the graph, neighbour slot): pass[j] for entry j
 // of the reversed graph (p lists q) has bit n set iff neighbour n of q may enter row p.
 // The exploration kernel of point p finds its entries through fwd2rev, gathers the
 // few ids whose bit is set (a few per cent), computes their exact distances and
 // merges them.  Nothing is decided here that the exact arithmetic would decide
 // otherwise; no atomics on shared counters, no buffer that can overflow.
+//
+// For the merge kernel that works through a point's candidates in the order of their
+// bounds (explore.hip: rows with many candidates), L itself is kept for every marked
+// pair, rounded down to a bfloat16 number (16 bits per pair of the join).
 //
 // Steps: in-degree count -> exclusive scan -> fill R (compressed rows) and the map
 // from graph entries to their place in R -> join.
@@ -35,6 +42,7 @@ struct ExploreWorkspace {
     int* deg = nullptr;        // N: in-degree (counted, then consumed by the fill)
     int* totals = nullptr;     // per scan block
     uint32_t* pass = nullptr;  // N*K*MW
+    uint16_t* bounds = nullptr; // N*K*32*MW lower bounds of the marked pairs (bfloat16, rounded down), or null
     int* todo = nullptr;       // two lists of N+1 ints: points left over by a launch; entry N = their number
     int* host_count = nullptr; // pinned
     int n_blocks = 0;
@@ -138,11 +146,11 @@ __global__ void k_fill_rev(const int* __restrict__ old_idx, size_t total, int N,
 }
 
 // One wavefront per q.  Per-wavefront LDS (ints): cq[KP] | pid[32] | pn[32] | ptau[32], KP = K rounded up to 32.
-template <int WAVES>
+template <int WAVES, bool BOUNDS>
 __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N, int K, const int* __restrict__ old_idx,
                                                               const float* __restrict__ knn_dist,
                                                               const int* __restrict__ offs, const int* __restrict__ rev,
-                                                              uint32_t* __restrict__ pass, int KP, int bpitch, int ksteps,
+                                                              uint32_t* __restrict__ pass, uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
                                                               float kappa, float one_minus_gamma, int wave_lds_ints)
 {
     extern __shared__ __align__(16) int lds_join[];
@@ -212,7 +220,13 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
                 const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);
                 const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;
                 const bool skip = lower > ptau[m];        // false if anything is NaN; a tie at the last slot may still enter (smaller index)
-                const uint64_t bm = ballot64(cid >= 0 && !skip);
+                const bool marked = cid >= 0 && !skip;
+                const uint64_t bm = ballot64(marked);
+                if (BOUNDS && marked && m < np) {
+                    // a bound below zero (or NaN) says nothing: 0.  Dropping the low half of a positive float rounds down.
+                    const uint32_t lb = lower > 0.0f ? __float_as_uint(lower) >> 16 : 0u;
+                    bounds[((size_t)r0 + pt0 + m) * (size_t)KP + ct * 32 + (lane & 31)] = (uint16_t)lb;
+                }
                 const int m_lo = 8 * (i >> 2) + (i & 3);
                 if (lane == m_lo) mine = (uint32_t)bm;
                 if (lane == m_lo + 4) mine = (uint32_t)(bm >> 32);
@@ -238,7 +252,7 @@ size_t explore_ws_bytes(int N, int K)
     return (size_t)N * ((size_t)K * 4 * (2 + mw) + 24) + 4096;
 }
 
-int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
+int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
 {
     *out = nullptr;
     auto* w = new ExploreWorkspace();
@@ -256,6 +270,11 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
         set_last_error("exploration workspace: out of device memory");
         return 1;
     }
+    if (with_bounds) {
+        // 2 bytes per pair of the join; without them the merge still works, in the order of the marks
+        void* b = nullptr;
+        if (ws_alloc(&b, (size_t)N * K * w->MW * 32 * sizeof(uint16_t)) == 0) w->bounds = static_cast<uint16_t*>(b);
+    }
     *out = w;
     return 0;
 }
@@ -263,7 +282,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass, w->todo};
+    void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass, w->todo, w->bounds};
     for (void* b : bufs)
         ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
@@ -272,6 +291,7 @@ void explore_ws_free(ExploreWorkspace* w)
 
 const int* explore_ws_fwd2rev(const ExploreWorkspace* w) { return w->fwd2rev; }
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w) { return w->pass; }
+const uint16_t* explore_ws_bounds(const ExploreWorkspace* w) { return w->bounds; }
 int* explore_ws_todo(ExploreWorkspace* w, int which) { return w->todo + (size_t)which * ((size_t)w->N + 1); }
 int* explore_ws_host_count(ExploreWorkspace* w) { return w->host_count; }
 
@@ -303,9 +323,14 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21
     const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
     RSFK_CHECK(one_minus_gamma > 0.5f, "exploration join: D too large");
-    hipLaunchKernelGGL(k_explore_join<kWaves>, dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds, stream,
-                       bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, KP, bf16_pitch(D), ksteps, kappa,
-                       one_minus_gamma, wave_ints);
+    if (w->bounds)
+        hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
+                           stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
+                           kappa, one_minus_gamma, wave_ints);
+    else
+        hipLaunchKernelGGL((k_explore_join<kWaves, false>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
+                           stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
+                           kappa, one_minus_gamma, wave_ints);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

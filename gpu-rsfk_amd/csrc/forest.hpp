@@ -64,16 +64,20 @@ void release_copy_buffers();
 struct ExploreWorkspace;
 bool explore_join_enabled(int N, int K);
 size_t explore_ws_bytes(int N, int K);
-int explore_ws_alloc(ExploreWorkspace** out, int N, int K);
+int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds = false);
 void explore_ws_free(ExploreWorkspace* w);
 const int* explore_ws_fwd2rev(const ExploreWorkspace* w);
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w);
+const uint16_t* explore_ws_bounds(const ExploreWorkspace* w);
 int* explore_ws_todo(ExploreWorkspace* w, int which);
 int* explore_ws_host_count(ExploreWorkspace* w);
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
                         const float* knn_dist, hipStream_t stream);
 
 // explore.hip
+// true when rows of K neighbours of D-dimensional points get the merge kernel that takes a point's candidates in the
+// order of their lower bounds (the workspace should then be allocated with room for the bounds)
+bool explore_merge_uses_bounds(int D, int K);
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
