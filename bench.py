@@ -233,7 +233,9 @@ def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
     kernel = (("k_bucket_knn_small<64> (buckets <= 64" + ("" if first is None else "; trees 0..%d" % (first - 1) if first > 0 else "; no tree")
                + ")" + ("" if first is None else " / k_bucket_knn_screen (later trees: pair matrix bounded on the matrix cores)")
                + " + k_bucket_knn_small<72> (65..72)") if small
-              else "k_bucket_knn (64 x 64 tiles of the pair matrix)" + ("" if mx <= 72 or K > 64 else " + k_bucket_knn_small for the buckets up to 72 points"))
+              else ("k_bucket_knn_rows (a bucket's points resident in LDS, every K-NN row touched once)"
+                    if K <= 64 and mx <= 64 * min(4, (40960 - 1024) // (64 * (4 * (((D + 3) & ~3) + (4 if (((D + 3) >> 2) & 1) == 0 else 0)) + 4)))
+                    else "k_bucket_knn (64 x 64 tiles of the pair matrix)") + ("" if mx <= 72 or K > 64 else " + k_bucket_knn_small for the buckets up to 72 points"))
     if gram is not None:
         kernel += "; k_bucket_knn_gram from tree %s on (RSFK_GRAM_FROM)" % gram
     if alg_flops / alg_bytes > balance:

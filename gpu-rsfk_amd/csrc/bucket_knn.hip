@@ -283,6 +283,15 @@ int largest_bucket(const int* sizes, int n, hipStream_t stream, int* out)
 
 }  // namespace
 
+// Largest bucket that goes to the kernel that keeps a bucket's points in LDS (0: none); RSFK_BUCKET_ROWS=0 switches
+// it off.
+static int resident_rows_cap(int D, int K)
+{
+    const char* e = std::getenv("RSFK_BUCKET_ROWS");
+    if (e && e[0] == '0') return 0;
+    return bucket_rows_cap(D, K);
+}
+
 int bucket_gram_from()
 {
     // Off unless asked for: on the shapes measured so far (bucket sizes 33..256, D 32..784, K 32 and 90) the direct
@@ -322,6 +331,15 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
             return 1;
         if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
         skip_upto = medium_bucket_cap();
+        const int rows_cap = resident_rows_cap(D, K);
+        if (rows_cap > skip_upto) {
+            // buckets whose points fit into LDS whole: every K-NN row is touched once
+            if (launch_bucket_knn_rows(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto + 1,
+                                       max_bucket >= 0 ? std::min(max_bucket, rows_cap) : rows_cap, false, true, knn_idx, knn_dist, stream))
+                return 1;
+            if (max_bucket >= 0 && max_bucket <= rows_cap) return 0;
+            skip_upto = rows_cap;
+        }
     }
     return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream);
 }
@@ -330,10 +348,11 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  rows_sorted: every K-NN row is
 // known to be sorted by distance.  screen: the small buckets go to the kernel that bounds the pair matrix on the matrix
 // cores first (needs sorted rows, K <= 64).  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
-// kinds touch different rows, so the two parts of one tree may run side by side).
+// kinds touch different rows, so the two parts of one tree may run side by side).  young_rows: the rows may be new or
+// far from done (first trees of a build).
 int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part)
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part, bool young_rows)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
@@ -373,6 +392,15 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
             return 1;
         if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
         skip_upto = medium_bucket_cap();
+        const int rows_cap = resident_rows_cap(D, K);
+        if (rows_cap > skip_upto) {
+            if (launch_bucket_knn_rows(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto + 1,
+                                       max_bucket >= 0 ? std::min(max_bucket, rows_cap) : rows_cap, rows_sorted, young_rows, knn_idx,
+                                       knn_dist, stream))
+                return 1;
+            if (max_bucket >= 0 && max_bucket <= rows_cap) return 0;
+            skip_upto = rows_cap;
+        }
     }
     return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream,
                           rows_sorted);

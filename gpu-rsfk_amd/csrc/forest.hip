@@ -165,6 +165,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         for (auto& e : ev)
             if (e.create()) return 1;
         const int gram_from = bucket_gram_from();
+        constexpr int kYoungTrees = 2;          // trees of a build whose bucket step still finds rows that are far from done
         SideStream sync;
         if (std::getenv("RSFK_KNN_ONE_STREAM") == nullptr && sync.open()) return 1;
         int rc = 0;
@@ -191,11 +192,11 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 const bool gram = t0 + j >= gram_from;
                 rc = launch_bucket_knn_tree(d_points, t0 + j >= screen_from, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
-                                            d_idx, d_dist, stream, split ? 1 : 0);
+                                            d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees);
                 if (!rc && split) {
                     rc = launch_bucket_knn_tree(d_points, false, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
-                                                stats[5 * j + 2], d_idx, d_dist, sync.side, 2);
+                                                stats[5 * j + 2], d_idx, d_dist, sync.side, 2, t0 + j < kYoungTrees);
                     (void)hipEventRecord(sync.big, sync.side);
                 }
                 big_pending = split;

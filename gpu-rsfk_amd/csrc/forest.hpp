@@ -38,7 +38,7 @@ int bucket_gram_from();
 
 int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0);
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0, bool young_rows = true);
 
 // bucket_knn_screen.hip
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);
@@ -46,6 +46,12 @@ int launch_bucket_knn_screen(const float* points, int D, int K, const int* ids, 
                              int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream);
 // trees from this index on send their buckets of up to 64 points to that kernel (RSFK_BUCKET_SCREEN)
 int bucket_screen_from(int D, int K);
+
+// bucket_knn_rows.hip
+int bucket_rows_cap(int D, int K);
+int launch_bucket_knn_rows(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
+                           int stride, int min_size, int max_size, bool rows_sorted, bool young_rows, int* knn_idx,
+                           float* knn_dist, hipStream_t stream);
 
 // bucket_knn_small.hip
 int small_bucket_cap();
