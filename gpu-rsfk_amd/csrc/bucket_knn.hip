@@ -33,6 +33,7 @@ constexpr int kTile = 64;          // points per tile side
 constexpr int kDC = 32;            // dimensions staged per step
 constexpr int kDCP = kDC + 4;      // LDS row pitch in floats: 9 x 16 B, odd => conflict-free b128 reads
 constexpr int kDistPitch = kTile + 1;
+constexpr int kStripBuckets = 4096;  // launches over at most this many buckets split them into strips of 64 members
 
 // ---------------------------------------------------------------------------
 // general kernel
@@ -51,45 +52,62 @@ struct BucketKnnLds {
     int flag_b[kTile];
 };
 
-// Stage rows ids[0..rows) x dims [d0, d0+32) into dst (zero filled outside).
-__device__ __forceinline__ void stage_rows(float* __restrict__ dst, const int* __restrict__ ids, int rows,
-                                           const float* __restrict__ points, int D, int d0, bool vec_ok)
-{
-    const int t = threadIdx.x;
-    const int r = t >> 2;            // 0..63
-    const int seg = (t & 3) * 8;     // 0,8,16,24
+// A thread's share (8 values of one row) of the rows ids[0..rows) x dims [d0, d0+32) on its way from memory to LDS:
+// requested into registers first, so that the next 32 dimensions travel while these are being used.
+struct StagedRows {
     float v[8];
+
+    __device__ __forceinline__ void request(const int* __restrict__ ids, int rows, const float* __restrict__ points, int D,
+                                            int d0, bool vec_ok)
+    {
+        const int t = threadIdx.x;
+        const int r = t >> 2;            // 0..63
+        const int seg = (t & 3) * 8;     // 0,8,16,24
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = 0.0f;
-    if (r < rows) {
-        const float* src = points + (size_t)ids[r] * (size_t)D + d0 + seg;
-        const int left = D - d0 - seg;
-        if (vec_ok && left >= 8) {
-            const float4 q0 = *reinterpret_cast<const float4*>(src);
-            const float4 q1 = *reinterpret_cast<const float4*>(src + 4);
-            v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w;
-            v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
-        } else {
+        for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+        if (r < rows && d0 + seg < D) {
+            const float* src = points + (size_t)ids[r] * (size_t)D + d0 + seg;
+            const int left = D - d0 - seg;
+            if (vec_ok && left >= 8) {
+                const float4 q0 = *reinterpret_cast<const float4*>(src);
+                const float4 q1 = *reinterpret_cast<const float4*>(src + 4);
+                v[0] = q0.x; v[1] = q0.y; v[2] = q0.z; v[3] = q0.w;
+                v[4] = q1.x; v[5] = q1.y; v[6] = q1.z; v[7] = q1.w;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) if (e < left) v[e] = src[e];
+                for (int e = 0; e < 8; ++e) if (e < left) v[e] = src[e];
+            }
         }
     }
-    float4* d4 = reinterpret_cast<float4*>(dst + r * kDCP + seg);
-    d4[0] = make_float4(v[0], v[1], v[2], v[3]);
-    d4[1] = make_float4(v[4], v[5], v[6], v[7]);
-}
 
-template <int SL>
+    // (zero filled outside the rows and beyond D)
+    __device__ __forceinline__ void commit(float* __restrict__ dst) const
+    {
+        const int t = threadIdx.x;
+        float4* d4 = reinterpret_cast<float4*>(dst + (t >> 2) * kDCP + (t & 3) * 8);
+        d4[0] = make_float4(v[0], v[1], v[2], v[3]);
+        d4[1] = make_float4(v[4], v[5], v[6], v[7]);
+    }
+};
+
+// STRIP = false: a workgroup per bucket walks the tiles (I, J >= I) of the upper triangle and updates the rows of
+// both tiles.  STRIP = true: a workgroup per 64 members of a bucket (workgroup w: tile w % max_tiles of bucket
+// w / max_tiles) walks all tiles J and updates only its own rows -- every pair is computed from both ends, but a launch
+// over few buckets has max_tiles times as many workgroups, each with half the merges: for grids that would
+// otherwise leave most of the device idle.
+template <int SL, bool STRIP>
 __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ points, int D, int K,
                                                      const int* __restrict__ ids, const int* __restrict__ starts,
                                                      const int* __restrict__ sizes, int stride, int skip_upto,
                                                      int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                     int rows_sorted)
+                                                     int rows_sorted, int max_tiles)
 {
     __shared__ BucketKnnLds L;
-    const int bkt = blockIdx.x;
+    const int bkt = STRIP ? blockIdx.x / max_tiles : blockIdx.x;
     const int s = sizes[bkt];
     if (s < 2 || s <= skip_upto) return;
+    const int I_first = STRIP ? (int)blockIdx.x - bkt * max_tiles : 0;
+    if (I_first * kTile >= s) return;
     const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -98,9 +116,9 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const int nt = (s + kTile - 1) / kTile;
 
-    for (int I = 0; I < nt; ++I) {
+    for (int I = I_first; I < (STRIP ? I_first + 1 : nt); ++I) {
         const int rows = min(kTile, s - I * kTile);
-        for (int J = I; J < nt; ++J) {
+        for (int J = STRIP ? 0 : I; J < nt; ++J) {
             const int cols = min(kTile, s - J * kTile);
             const bool diag = (I == J);
             __syncthreads();   // previous tile's LDS fully consumed
@@ -123,10 +141,17 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
 #pragma unroll
                 for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
             __syncthreads();
+            StagedRows sa, sb;
+            sa.request(L.ida, rows, points, D, 0, vec_ok);
+            if (!diag) sb.request(L.idb, cols, points, D, 0, vec_ok);
             for (int d0 = 0; d0 < D; d0 += kDC) {
-                stage_rows(L.a, L.ida, rows, points, D, d0, vec_ok);
-                if (!diag) stage_rows(L.b, L.idb, cols, points, D, d0, vec_ok);
+                sa.commit(L.a);
+                if (!diag) sb.commit(L.b);
                 __syncthreads();
+                if (d0 + kDC < D) {
+                    sa.request(L.ida, rows, points, D, d0 + kDC, vec_ok);
+                    if (!diag) sb.request(L.idb, cols, points, D, d0 + kDC, vec_ok);
+                }
                 const float* B = diag ? L.a : L.b;
 #pragma unroll 2
                 for (int dd = 0; dd < kDC; dd += 4) {
@@ -170,7 +195,7 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
             __syncthreads();
             // Rows of tile I take the columns of tile J as candidates, then (off the diagonal) the columns of tile J
             // the rows of tile I.  A wavefront walks its rows that have a candidate, the next one's row in flight.
-            for (int side = 0; side < (diag ? 1 : 2); ++side) {
+            for (int side = 0; side < ((diag || STRIP) ? 1 : 2); ++side) {
                 const int n_mine = side == 0 ? rows : cols, n_other = side == 0 ? cols : rows;
                 const int* id_mine = side == 0 ? L.ida : L.idb;
                 const int* id_other = side == 0 ? L.idb : L.ida;
@@ -228,20 +253,29 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
 namespace {
 
 int launch_general(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
-                   int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted = false)
+                   int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted = false,
+                   int max_bucket = -1)
 {
     if (n_buckets <= 0) return 0;
-    dim3 grid((unsigned)n_buckets), block(256);
     const int rs = rows_sorted ? 1 : 0;
-    if (K <= 64)
-        hipLaunchKernelGGL(k_bucket_knn<1>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
-                           knn_dist, rs);
-    else if (K <= 128)
-        hipLaunchKernelGGL(k_bucket_knn<2>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
-                           knn_dist, rs);
-    else
-        hipLaunchKernelGGL(k_bucket_knn<4>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, skip_upto, knn_idx,
-                           knn_dist, rs);
+    // few buckets (and their largest size known): a workgroup per 64 members instead of one per bucket
+    const int max_tiles = max_bucket > 0 ? (max_bucket + kTile - 1) / kTile : 0;
+    const char* env = std::getenv("RSFK_BUCKET_STRIP");        // 0 / 1 overrides the choice (the results are the same)
+    const bool strip = max_tiles > 1 && (env && *env ? env[0] == '1' : n_buckets <= kStripBuckets);
+    dim3 grid((unsigned)n_buckets * (unsigned)(strip ? max_tiles : 1)), block(256);
+#define RSFK_GENERAL_CASE(SLV)                                                                                              \
+    do {                                                                                                                    \
+        if (strip)                                                                                                          \
+            hipLaunchKernelGGL((k_bucket_knn<SLV, true>), grid, block, 0, stream, points, D, K, ids, starts, sizes, stride,  \
+                               skip_upto, knn_idx, knn_dist, rs, max_tiles);                                                \
+        else                                                                                                                \
+            hipLaunchKernelGGL((k_bucket_knn<SLV, false>), grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, \
+                               skip_upto, knn_idx, knn_dist, rs, 1);                                                        \
+    } while (0)
+    if (K <= 64) RSFK_GENERAL_CASE(1);
+    else if (K <= 128) RSFK_GENERAL_CASE(2);
+    else RSFK_GENERAL_CASE(4);
+#undef RSFK_GENERAL_CASE
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -341,7 +375,8 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
             skip_upto = rows_cap;
         }
     }
-    return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream);
+    return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream, false,
+                          max_bucket);
 }
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
@@ -379,7 +414,8 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
             if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
-        } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted)) {
+        } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted,
+                                  kBucketSplit)) {
             return 1;
         }
     }
@@ -403,7 +439,7 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
         }
     }
     return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream,
-                          rows_sorted);
+                          rows_sorted, max_bucket);
 }
 
 }  // namespace rsfk

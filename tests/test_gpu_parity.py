@@ -86,12 +86,19 @@ def test_tree_edge_cases(gpu, orc, rng):
     (1200, 1, 4, 5, 10), (2500, 3, 1, 2, 4), (2000, 130, 64, 65, 130), (1500, 20, 65, 66, 140),
     (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
 ])
-@pytest.mark.parametrize("kernel", ["direct", "gram", "screen"])
+@pytest.mark.parametrize("kernel", ["direct", "direct_per_bucket", "gram", "screen"])
 def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
     """kernel: "direct" = fp32 chains for every pair; "gram" = the kernel that bounds the pair matrix on the matrix
     cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0); "screen" = the same
     idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=0; other buckets, and K > 64,
-    take the direct kernels)."""
+    take the direct kernels); "direct_per_bucket" = the tiled direct kernel with a workgroup per bucket, as launches
+    over many buckets run it (RSFK_BUCKET_STRIP=0; with the few buckets of a test it otherwise takes a workgroup per 64
+    members), and without the kernel that keeps a bucket's points in LDS (RSFK_BUCKET_ROWS=0)."""
+    if kernel == "direct_per_bucket":
+        if MAX <= 72 and K <= 64:
+            pytest.skip("no bucket of this shape reaches the tiled kernel")
+        monkeypatch.setenv("RSFK_BUCKET_STRIP", "0")
+        monkeypatch.setenv("RSFK_BUCKET_ROWS", "0")
     if kernel == "gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     if kernel == "screen":
