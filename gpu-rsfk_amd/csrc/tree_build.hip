@@ -31,6 +31,7 @@
 #include "rsfk_common.hpp"
 #include "wave64.hpp"
 #include "bf16.hpp"
+#include "tree_sweep.hpp"
 #include <vector>
 #include <algorithm>
 #include <cstdlib>
@@ -280,20 +281,23 @@ __device__ __forceinline__ void resolve_exact(const int* list, int n, const floa
 constexpr int kSideBatch = 4;        // points per group and call of the screen in the wide phase
 constexpr int kTailBatch = 2;        // ... in the tail kernel
 
-// Append a child node either to the next wide level or to the tail queue.
-__device__ __forceinline__ void emit_node(const TreeNode& c, const TreeParams& P, TreeNode* next, int next_cap,
-                                          TreeNode* tail, int tail_cap, LevelCounters* ctr)
+// Append a child node either to the next wide level or to the tail queue.  Returns its place in the queue of the next
+// wide level, or -1.
+__device__ __forceinline__ int emit_node(const TreeNode& c, const TreeParams& P, TreeNode* next, int next_cap,
+                                         TreeNode* tail, int tail_cap, LevelCounters* ctr)
 {
     const bool forced = c.depth >= P.MAX_DEPTH - 1;
     if (!c.leaf && !forced && c.count > P.small) {
         const int at = atomicAdd(&ctr->n_next, 1);
-        if (at < next_cap) next[at] = c; else ctr->overflow = 1;
-    } else {
-        TreeNode t = c;
-        if (forced) t.leaf = 1;
-        const int at = atomicAdd(&ctr->n_tail, 1);
-        if (at < tail_cap) tail[at] = t; else ctr->overflow = 1;
+        if (at < next_cap) { next[at] = c; return at; }
+        ctr->overflow = 1;
+        return -1;
     }
+    TreeNode t = c;
+    if (forced) t.leaf = 1;
+    const int at = atomicAdd(&ctr->n_tail, 1);
+    if (at < tail_cap) tail[at] = t; else ctr->overflow = 1;
+    return -1;
 }
 
 // The split / min-size-merge / leaf rules for a node whose left side has `a`
@@ -375,7 +379,7 @@ __global__ void k_init_perm(int* __restrict__ perm, int N, int B)
 }
 
 __global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr, TreeParams P, int B, int seed0,
-                             int* n_rec)
+                             int* n_rec, int* pmap)
 {
     const int t = blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= B) return;
@@ -385,7 +389,8 @@ __global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr
     r.rec = 0; r.pad_ = 0;
     r.key = root_key(seed0 + t);
     // the root is never a leaf (src/kernels/build_tree_init.cu:79) unless the depth limit forces it
-    emit_node(r, P, nodes, B, tail, B, ctr);
+    const int at = emit_node(r, P, nodes, B, tail, B, ctr);
+    if (pmap) pmap[t * pm::kPaths] = at;      // path 0 of level 0 = the root, if it is split at all
 }
 
 // chunk_base[i] = number of chunks of nodes [0,i); one workgroup.
@@ -542,7 +547,8 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
                                                     const int* __restrict__ chunk2node, const int* __restrict__ chunk_left,
                                                     TreeNode* __restrict__ next, int next_cap,
                                                     TreeNode* __restrict__ tail, int tail_cap, LevelCounters* ctr,
-                                                    TreeRec* __restrict__ recs, int* __restrict__ n_rec, int rec_cap)
+                                                    TreeRec* __restrict__ recs, int* __restrict__ n_rec, int rec_cap,
+                                                    int2* __restrict__ child)
 {
     __shared__ int red[2][kBlock / 64];
     __shared__ int wcnt[kBlock / 64];
@@ -604,8 +610,58 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
             index_split(recs + (size_t)nd.tree * rec_cap, n_rec + nd.tree, rec_cap, nd.rec, src[nd.dstart + r1] & kIdMask,
                         src[nd.dstart + r2] & kIdMask, nc, c0.rec, c1.rec, ctr);
         }
-        emit_node(c0, P, next, next_cap, tail, tail_cap, ctr);
-        if (nc == 2) emit_node(c1, P, next, next_cap, tail, tail_cap, ctr);
+        const int at0 = emit_node(c0, P, next, next_cap, tail, tail_cap, ctr);
+        const int at1 = nc == 2 ? emit_node(c1, P, next, next_cap, tail, tail_cap, ctr) : at0;
+        // where the members of either side are at the next level (a node with one child keeps them together)
+        if (child) child[ni] = make_int2(at0, at1);
+    }
+}
+
+// What k_side leaves behind, from sides that are already known (one bit per point of the tree, pm::k_pm_sweep and
+// pm::k_pm_resolve): bit 31 of the permutation entries of a chunk and the number of its left members.
+__global__ __launch_bounds__(kBlock) void k_pm_mark(TreeParams P, int* __restrict__ perm0, int* __restrict__ perm1,
+                                                    const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
+                                                    const int* __restrict__ chunk2node, int* __restrict__ chunk_left,
+                                                    const uint32_t* __restrict__ sidebits, int W)
+{
+    __shared__ int part[kBlock / 64];
+    const int c = blockIdx.x;
+    const int ni = chunk2node[c];
+    const TreeNode nd = nodes[ni];
+    const int k = c - chunk_base[ni];
+    int* perm = (nd.buf ? perm1 : perm0) + (size_t)nd.tree * (size_t)P.N;
+    const uint32_t* bits = sidebits + (size_t)nd.tree * (size_t)W;
+    const int pos0 = nd.start + k * P.chunk;
+    const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
+    int lefts = 0;
+    for (int r0 = pos0; r0 < pos1; r0 += 4 * kBlock) {
+        int id[4];
+        uint32_t w[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int pos = r0 + u * kBlock + (int)threadIdx.x;
+            id[u] = pos < pos1 ? (perm[pos] & kIdMask) : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) w[u] = id[u] >= 0 ? bits[id[u] >> 5] : 0u;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int pos = r0 + u * kBlock + (int)threadIdx.x;
+            if (id[u] >= 0) {
+                const bool right = (w[u] >> (id[u] & 31)) & 1u;
+                perm[pos] = right ? (id[u] | (int)0x80000000) : id[u];
+                lefts += right ? 0 : 1;
+            }
+        }
+    }
+    lefts = wave_sum_i(lefts);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = lefts;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int all = 0;
+#pragma unroll
+        for (int i = 0; i < kBlock / 64; ++i) all += part[i];
+        chunk_left[c] = all;
     }
 }
 
@@ -893,12 +949,24 @@ struct TreeBatchWorkspace {
     // events around the kernels of a wide level (hyperplanes | side test | scatter) and around the tail kernel
     hipEvent_t ev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     float phase_s[4] = {0.f, 0.f, 0.f, 0.f};   // of the last batch: side tests, hyperplanes, scatter, tail kernel
+    // side tests of the first levels taken point by point (tree_sweep.hpp); allocated when D allows it
+    int pm_ks = 0;                       // 32-dimension steps of a row as matrix-core operands (1, 2, 4, 8), 0 = not available
+    int pm_W = 0;                        // tiles of 32 points (even)
+    int pm_Bs = 0;                       // B rounded up to 16
+    uint8_t* pm_path = nullptr;          // 32 W x Bs
+    uint32_t* pm_side = nullptr;         // B x W
+    uint32_t* pm_undec = nullptr;        // B x W
+    int* pm_map[2] = {nullptr, nullptr}; // B x pm::kPaths, this level's and the next one's
+    pm::PlaneQ* pm_sc = nullptr;         // B x pm::kPaths
+    int8_t* pm_aq = nullptr;             // B x pm::kMaxGroups x 32 x 32 pm_ks
+    int2* pm_child = nullptr;            // node_cap
 };
 
 static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
-                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec, w.planes};
+                   w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec, w.planes,
+                   w.pm_path, w.pm_side, w.pm_undec, w.pm_map[0], w.pm_map[1], w.pm_sc, w.pm_aq, w.pm_child};
     for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
@@ -925,7 +993,7 @@ int tree_small_threshold() { return 1024; }
 size_t tree_ws_bytes(int N, int D, int MIN, int B)
 {
     const size_t lc = (size_t)N / (size_t)std::max(MIN, 1) + 2;
-    return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24 + (size_t)(4 + nvec_len(D)) * 4));
+    return bf16_copy_bytes(N, D) + (size_t)B * ((size_t)N * 8 + (size_t)N * 2 + 512 * 1024 + lc * (8 + sizeof(TreeNode)) + ((size_t)N / 1024 + 2) * (2 * sizeof(TreeNode) + 24 + (size_t)(4 + nvec_len(D)) * 4));
 }
 
 // From now on every build with this workspace also writes the index of each tree (TreeRec records).
@@ -968,6 +1036,19 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     if (dmalloc(&w->leaf_size, (size_t)B * w->leaf_cap)) return 1;
     if (dmalloc(&w->stats, (size_t)B)) return 1;
     if (dmalloc(&w->ctr, (size_t)1)) return 1;
+    if (D <= 256 && N > small && B <= 64) {
+        w->pm_ks = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : 8;
+        w->pm_W = 2 * ((N + 63) / 64);                     // an even number of 32-point tiles
+        w->pm_Bs = (B + 15) & ~15;
+        if (dmalloc(&w->pm_path, (size_t)w->pm_Bs * w->pm_W * 32)) return 1;
+        if (dmalloc(&w->pm_side, (size_t)w->pm_Bs * w->pm_W)) return 1;
+        if (dmalloc(&w->pm_undec, (size_t)w->pm_Bs * w->pm_W)) return 1;
+        if (dmalloc(&w->pm_map[0], (size_t)B * pm::kPaths)) return 1;
+        if (dmalloc(&w->pm_map[1], (size_t)B * pm::kPaths)) return 1;
+        if (dmalloc(&w->pm_sc, (size_t)B * pm::kPaths)) return 1;
+        if (dmalloc(&w->pm_aq, (size_t)B * pm::kMaxGroups * 32 * 32 * w->pm_ks)) return 1;
+        if (dmalloc(&w->pm_child, (size_t)w->node_cap)) return 1;
+    }
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_ctr), sizeof(LevelCounters)));
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stats), sizeof(TreeStats) * (size_t)B));
     for (hipEvent_t& e : w->ev) RSFK_HIP(hipEventCreate(&e));
@@ -1007,8 +1088,16 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     std::memcpy(w->h_stats, init.data(), sizeof(TreeStats) * (size_t)nb);
     RSFK_HIP(hipMemcpyAsync(w->stats, w->h_stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyHostToDevice, stream));
     RSFK_HIP(hipMemsetAsync(w->ctr, 0, sizeof(LevelCounters), stream));
+    // Levels whose side tests are taken point by point (needs the 8-bit copy).  RSFK_PM_LEVELS overrides (0 = none).
+    // The sweep multiplies every tile of points with every block of 16 hyperplanes of a tree, so its cost doubles
+    // per level from the fifth on; measured, the seventh level is the last one it takes faster than k_side.
+    int pm_levels = 0;
+    if (q8 && w->pm_ks) {
+        pm_levels = pm::kMaxLevels - 1;
+        if (const char* e = std::getenv("RSFK_PM_LEVELS")) pm_levels = std::max(0, std::min(pm::kMaxLevels, std::atoi(e)));
+    }
     hipLaunchKernelGGL(k_init_roots, dim3((nb + 63) / 64), dim3(64), 0, stream, w->nodes[0], w->tail, w->ctr, P, nb, seed0,
-                       w->n_rec);
+                       w->n_rec, pm_levels > 0 ? w->pm_map[0] : nullptr);
     RSFK_HIP(hipGetLastError());
 
     int cur = 0;
@@ -1038,6 +1127,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         level_timed = false;
     };
     // wide levels
+    int level = 0;
     while (true) {
         // one trip to the host per level: the chunk table of the level is made first (from the node count on the
         // device), then both counts come back together
@@ -1058,6 +1148,28 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
         hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
         (void)hipEventRecord(w->ev[1], stream);
+        const bool swept = level < pm_levels;
+        if (swept) {
+            // the sides of every point in all trees of the batch, then their marks in the permutations
+            const int n_paths = 1 << level, ks = w->pm_ks, W = w->pm_W;
+            const int rec = 4 + nvec_len(D);
+            hipLaunchKernelGGL(pm::k_pm_planes, dim3((unsigned)((nb * n_paths + 3) / 4)), dim3(256), 0, stream, w->planes, rec, D,
+                               32 * ks, w->pm_map[level & 1], n_paths, nb, w->pm_sc, w->pm_aq);
+            const dim3 sgrid((unsigned)((W + 7) / 8));          // two tiles per wavefront, four wavefronts
+#define RSFK_SWEEP_LAUNCH(KS)                                                                                                \
+            hipLaunchKernelGGL((pm::k_pm_sweep<KS>), sgrid, dim3(256), 0, stream, q8, N, D, nb, w->pm_Bs, level, W, w->pm_path, \
+                               w->pm_side, w->pm_undec, w->pm_aq, w->pm_sc)
+            if (ks == 1) RSFK_SWEEP_LAUNCH(1);
+            else if (ks == 2) RSFK_SWEEP_LAUNCH(2);
+            else if (ks == 4) RSFK_SWEEP_LAUNCH(4);
+            else RSFK_SWEEP_LAUNCH(8);
+#undef RSFK_SWEEP_LAUNCH
+            const size_t words = (size_t)nb * W;
+            hipLaunchKernelGGL(pm::k_pm_resolve, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, points, D, W,
+                               w->pm_Bs, words, w->pm_path, w->pm_sc, w->planes, rec, w->pm_side, w->pm_undec);
+            hipLaunchKernelGGL(k_pm_mark, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
+                               w->chunk_base, w->chunk2node, w->chunk_left, w->pm_side, W);
+        } else {
         // lanes per point in the 8-bit screen: a lane takes 16 coordinates per step
         const int q8_pieces = q8_padded(D) >> 4;
 #define RSFK_SIDE_LAUNCH(Q, L)                                                                                              \
@@ -1068,14 +1180,22 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         else if (q8_pieces <= 4) RSFK_SIDE_LAUNCH(true, 4);
         else RSFK_SIDE_LAUNCH(true, 8);
 #undef RSFK_SIDE_LAUNCH
+        }
         (void)hipEventRecord(w->ev[2], stream);
+        const bool map_next = level + 1 < pm_levels;
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
-                           w->recs, w->n_rec, w->rec_cap);
+                           w->recs, w->n_rec, w->rec_cap, map_next ? w->pm_child : nullptr);
+        if (map_next) {
+            const int n_paths = 1 << level;
+            hipLaunchKernelGGL(pm::k_pm_next_map, dim3((unsigned)((nb * n_paths + 255) / 256)), dim3(256), 0, stream,
+                               w->pm_map[level & 1], w->pm_map[(level + 1) & 1], w->pm_child, n_paths, nb);
+        }
         (void)hipEventRecord(w->ev[3], stream);
         level_timed = true;
         RSFK_HIP(hipGetLastError());
         cur ^= 1;
+        ++level;
     }
     // tail
     const int n_tail = w->h_ctr->n_tail;
