@@ -303,11 +303,19 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
 }
 
 // Exploration of the points whose candidates the join has marked (explore_join.hip): entry (p, k) of
-// the graph has the mask of neighbour slots at pass[fwd2rev[p K + k]].  One wavefront per point: gather
+// the graph has the mask of neighbour slots at pass[p K + k] (entries without a valid neighbour have none).  One wavefront per point: gather
 // the marked ids, drop repeats and ids the row holds (hash set), exact distances, merge.  Points with
 // more marks than the LDS of this launch takes are appended to todo_out (for a launch with more LDS
 // per wavefront, or for the general kernel).  todo_in: the points to work on, or null for all.
 // Per-wavefront LDS (ints): tile[64*20] | xrow[dpad] | table[table_size] | srow[K] | marked[3/4 table_size].
+// Number of entry (p, k) of the graph snapshot, p K + k, or -1 when the slot holds no valid neighbour (the join writes
+// nothing for such an entry).
+__device__ __forceinline__ int graph_entry(const int* __restrict__ old_idx, int N, int K, int p, int k)
+{
+    const int q = old_idx[(size_t)p * K + k];
+    return q >= 0 && q < N ? p * K + k : -1;
+}
+
 constexpr int kMergeChunk = 16;
 constexpr int kMergeTile = 64 * (kMergeChunk + 4);
 
@@ -316,7 +324,6 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
                                                                const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                                float* __restrict__ knn_dist, int table_size,
                                                                int wave_lds_ints, int dpad,
-                                                               const int* __restrict__ fwd2rev,
                                                                const uint32_t* __restrict__ pass,
                                                                const int* __restrict__ todo_in, int n_in,
                                                                int* __restrict__ todo_out, int* __restrict__ n_out)
@@ -329,7 +336,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     const int MW = (K + 31) >> 5;
     int bits = 0;
     for (int k = lane; k < K; k += 64) {
-        const int j = fwd2rev[(size_t)p * K + k];
+        const int j = graph_entry(old_idx, N, K, p, k);
         if (j >= 0)
             for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
     }
@@ -370,7 +377,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     int n_marked = 0;                                     // wave-uniform
     for (int k0 = 0; k0 < K; k0 += 64) {
         const int k = k0 + lane;
-        const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
+        const int j = k < K ? graph_entry(old_idx, N, K, p, k) : -1;
         int mine = 0;
         if (j >= 0)
             for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
@@ -462,7 +469,7 @@ template <int SL>
 __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restrict__ points, int N, int D, int K,
                                                           const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                           float* __restrict__ knn_dist, int cap, int dpad,
-                                                          const int* __restrict__ fwd2rev, const uint32_t* __restrict__ pass,
+                                                          const uint32_t* __restrict__ pass,
                                                           const uint16_t* __restrict__ bounds,
                                                           const int* __restrict__ todo_in, int n_in,
                                                           int* __restrict__ todo_out, int* __restrict__ n_out)
@@ -478,7 +485,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     const int MW = (K + 31) >> 5, KP = MW * 32;
     int* table = lds_w;
     int* srow = table + kWgTable;
-    int* jrow = srow + ((K + 3) & ~3);                            // place of graph entry (p, k) in the reversed graph
+    int* jrow = srow + ((K + 3) & ~3);                            // number of graph entry (p, k), -1 without a valid neighbour
     float* xrow = reinterpret_cast<float*>(jrow + ((K + 3) & ~3));
     uint32_t* marked = reinterpret_cast<uint32_t*>(xrow + dpad);
     int* tiles = reinterpret_cast<int*>(marked + cap);
@@ -494,7 +501,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
 
     // ---- 1. the marked pairs of the point; thread k takes neighbour k (K <= 256)
     const int k = threadIdx.x;
-    const int j = k < K ? fwd2rev[(size_t)p * K + k] : -1;
+    const int j = k < K ? graph_entry(old_idx, N, K, p, k) : -1;
     if (k < K) {
         srow[k] = old_idx[(size_t)p * K + k];
         jrow[k] = j;
@@ -660,7 +667,7 @@ int merge_wg_ints(int cap, int dpad, int K, int sl)
 
 template <int SL>
 int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int cap,
-                    int dpad, const int* fwd2rev, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
+                    int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
                     int* todo_out, int* n_out, hipStream_t stream)
 {
     const size_t lds = (size_t)merge_wg_ints(cap, dpad, K, SL) * sizeof(int);
@@ -668,7 +675,7 @@ int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
     hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3((unsigned)n_work), dim3(256), lds, stream, points, N, D, K, old_idx,
-                       knn_idx, knn_dist, cap, dpad, fwd2rev, pass, bounds, todo_in, n_in, todo_out, n_out);
+                       knn_idx, knn_dist, cap, dpad, pass, bounds, todo_in, n_in, todo_out, n_out);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -682,7 +689,7 @@ int next_pow2(int v)
 
 template <int SL, int WAVES>
 int launch_merge(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
-                 int wave_ints, int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in, int n_in,
+                 int wave_ints, int dpad, const uint32_t* pass, const int* todo_in, int n_in,
                  int* todo_out, int* n_out, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
@@ -691,7 +698,7 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
     const int n_work = todo_in ? n_in : N;
     dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, fwd2rev, pass, todo_in, n_in, todo_out, n_out);
+                       knn_dist, table, wave_ints, dpad, pass, todo_in, n_in, todo_out, n_out);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -700,13 +707,13 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
 int merge_wave_ints(int table, int dpad, int K) { return (kMergeTile + dpad + table + K + table / 4 * 3 + 3) / 4 * 4; }
 
 int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
-                   float* knn_dist, int table, int dpad, const int* fwd2rev, const uint32_t* pass, const int* todo_in,
+                   float* knn_dist, int table, int dpad, const uint32_t* pass, const int* todo_in,
                    int n_in, int* todo_out, int* n_out, hipStream_t stream)
 {
     const int wi = merge_wave_ints(table, dpad, K);
 #define RSFK_MERGE_CASE(SLV, WV)                                                                                        \
     if (sl == SLV && waves == WV)                                                                                       \
-        return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, fwd2rev, pass,       \
+        return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, pass,       \
                                      todo_in, n_in, todo_out, n_out, stream);
     RSFK_MERGE_CASE(1, 4) RSFK_MERGE_CASE(1, 2) RSFK_MERGE_CASE(1, 1)
     RSFK_MERGE_CASE(2, 4) RSFK_MERGE_CASE(2, 2) RSFK_MERGE_CASE(2, 1)
@@ -790,12 +797,11 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         // The points it cannot take come back in a list and get a second launch with the largest set that
         // fits; what is left after that goes to the general kernel below.
         if (launch_explore_join(ws, *bf_join, N, D, K, old_idx, knn_dist, stream)) return 1;
-        const int* f2r = explore_ws_fwd2rev(ws);
         const uint32_t* pass = explore_ws_pass(ws);
         int* listA = explore_ws_todo(ws, 0);
         int* listB = explore_ws_todo(ws, 1);
         int* host_n = explore_ws_host_count(ws);
-        if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, f2r, pass, nullptr, 0,
+        if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, pass, nullptr, 0,
                            listA, listA + N, stream))
             return 1;
         RSFK_HIP(hipMemcpyAsync(host_n, listA + N, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -815,16 +821,16 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
             const uint16_t* bounds = explore_ws_bounds(ws);
             int rc = 0;
             if (!per_wg)
-                rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, f2r, pass,
+                rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, pass,
                                     listA, n_todo, listB, listB + N, stream);
             else if (sl == 1)
-                rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
                                         n_todo, listB, listB + N, stream);
             else if (sl == 2)
-                rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
                                         n_todo, listB, listB + N, stream);
             else
-                rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, f2r, pass, bounds, listA,
+                rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
                                         n_todo, listB, listB + N, stream);
             if (rc)
                 return 1;

@@ -13,10 +13,11 @@
 //   fp32 chain:             result >= d(real) (1 - gamma),  gamma = (D + 8) 2^-22
 // so L = (d~ - E1 - 1.01 (2u sqrt((d~ + E1) Q) + u^2 Q)) (1 - gamma) is a lower bound of the exact fp32
 // distance, and a pair is dropped when L is above the last slot of row p.
-// The outcome is one bit per (entry of the graph, neighbour slot): pass[j] for entry j
-// of the reversed graph (p lists q) has bit n set iff neighbour n of q may enter row p.
-// The exploration kernel of point p finds its entries through fwd2rev, gathers the
-// few ids whose bit is set (a few per cent), computes their exact distances and
+// The outcome is one bit per (entry of the graph, neighbour slot): pass[p K + k] for the
+// entry (p, k) = q has bit n set iff neighbour n of q may enter row p (an element of R(q)
+// is the number p K + k of the entry, so the join knows where to write and the merge
+// kernel of p reads its K words in one piece).  The exploration kernel of point p gathers
+// the few ids whose bit is set (a few per cent), computes their exact distances and
 // merges them.  Nothing is decided here that the exact arithmetic would decide
 // otherwise; no atomics on shared counters, no buffer that can overflow.
 //
@@ -24,8 +25,7 @@
 // bounds (explore.hip: rows with many candidates), L itself is kept for every marked
 // pair, rounded down to a bfloat16 number (16 bits per pair of the join).
 //
-// Steps: in-degree count -> exclusive scan -> fill R (compressed rows) and the map
-// from graph entries to their place in R -> join.
+// Steps: R in compressed rows (counting sort of the graph entries by neighbour, see k_bin_count) -> join.
 #include "rsfk_common.hpp"
 #include "wave64.hpp"
 #include "forest.hpp"
@@ -36,24 +36,43 @@ namespace rsfk {
 
 struct ExploreWorkspace {
     int N = 0, K = 0, MW = 0;  // MW = 32-bit words per entry of pass
-    int* rev = nullptr;        // N*K: R lists, compressed rows
-    int* fwd2rev = nullptr;    // N*K: entry (p, k) of the graph -> its place in rev (-1: no valid neighbour there)
+    int shift = 0;             // a bin of the reversed-graph builder = 2^shift consecutive points
+    int n_bins = 0;
+    int n_parts = 0;           // workgroups of the two passes over the graph; each owns a contiguous range of entries
+    int per_part = 0;          // entries per such range
+    uint32_t div_m = 0;        // e / K == (div_m * e) >> div_s for 0 <= e < 2^31
+    int div_s = 0;
+    int* rev = nullptr;        // N*K: R lists in compressed rows; an element is the number p K + k of a graph entry
     int* offs = nullptr;       // N+1: start of R(q)
-    int* deg = nullptr;        // N: in-degree (counted, then consumed by the fill)
-    int* totals = nullptr;     // per scan block
-    uint32_t* pass = nullptr;  // N*K*MW
+    int* bin_e = nullptr;      // N*K: entry numbers grouped by the bin of the neighbour they hold
+    uint16_t* bin_q = nullptr; // N*K: that neighbour minus the first point of its bin
+    int* bin_size = nullptr;   // n_bins
+    int* bin_start = nullptr;  // n_bins + 1
+    int* part_off = nullptr;   // n_parts x n_bins: where the entries of a part start inside a bin
+    uint32_t* pass = nullptr;  // N*K*MW, indexed by entry number
     uint16_t* bounds = nullptr; // N*K*32*MW lower bounds of the marked pairs (bfloat16, rounded down), or null
     int* todo = nullptr;       // two lists of N+1 ints: points left over by a launch; entry N = their number
     int* host_count = nullptr; // pinned
-    int n_blocks = 0;
 };
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-constexpr int kScanBlock = 1024;            // elements per workgroup of the scan (256 threads x 4)
 constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16
+constexpr int kMaxBins = 8192;
+constexpr int kMaxShift = 13;
+constexpr int kRowsBlock = 512;             // threads of k_bin_rows
+
+// Bins of the reversed-graph builder for N points: false if N is too large for it.
+bool rev_bins(int N, int* shift, int* n_bins)
+{
+    int s = 10;
+    while (s < kMaxShift && (((N - 1) >> s) + 1) > kMaxBins / 2) ++s;
+    *shift = s;
+    *n_bins = N > 0 ? ((N - 1) >> s) + 1 : 1;
+    return *n_bins <= kMaxBins;
+}
 
 __global__ void k_zero(int* a, int n, int* counter0, int* counter1)
 {
@@ -62,96 +81,136 @@ __global__ void k_zero(int* a, int n, int* counter0, int* counter1)
     if (i == 0) { *counter0 = 0; *counter1 = 0; }
 }
 
-__global__ void k_degree(const int* __restrict__ old_idx, size_t total, int N, int* __restrict__ deg)
+// exclusive scan of one value per thread over the workgroup (blockDim.x a multiple of 64, at most 1024); returns the
+// total in *total.  lds: one int per wavefront.
+__device__ __forceinline__ int block_excl_scan(int v, int* total, int* lds)
 {
-    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
-        const int q = old_idx[e];
-        if (q >= 0 && q < N) atomicAdd(&deg[q], 1);
-    }
-}
-
-// exclusive scan of 256 values, one per thread; returns the block total in *total
-__device__ __forceinline__ int block_scan_256(int v, int* total, int* lds4)
-{
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     int incl = v;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
         const int t = __shfl_up(incl, o, 64);
         if (lane >= o) incl += t;
     }
-    if (lane == 63) lds4[wave] = incl;
+    if (lane == 63) lds[wave] = incl;
     __syncthreads();
     int woff = 0, tot = 0;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) { const int x = lds4[w]; if (w < wave) woff += x; tot += x; }
+    for (int w = 0; w < waves; ++w) { const int x = lds[w]; if (w < wave) woff += x; tot += x; }
     __syncthreads();
     *total = tot;
     return woff + incl - v;
 }
 
-__global__ __launch_bounds__(256) void k_scan_blocks(const int* __restrict__ deg, int N, int* __restrict__ offs,
-                                                     int* __restrict__ totals)
+// The reversed graph R(q) = {entries (p, k) of the graph that hold q}, in compressed rows, without an atomic operation
+// on device memory per entry (device-wide atomics are carried out at the memory side of the fabric, about 27 G of them
+// a second: 2.8 ms for the 32 M entries of a 1 M x 32 graph, counting and placing).  Counting sort in two levels:
+// the points are cut into bins of 2^shift, (1) every part of the graph counts its entries per bin in LDS and reserves
+// its share of each bin with one atomic per bin, (2) the entries are moved to their bins -- entry number and neighbour
+// minus the start of the bin -- (3) one workgroup per bin counts its neighbours in LDS, scans, writes the row offsets
+// and places the entries.  The order of the entries inside R(q) is arbitrary; nothing downstream depends on it.
+__global__ __launch_bounds__(256) void k_bin_count(const int* __restrict__ old_idx, int total, int per_part, int N, int shift,
+                                                   int n_bins, int* __restrict__ bin_size, int* __restrict__ part_off)
 {
-    __shared__ int lds4[4];
-    const int i0 = blockIdx.x * kScanBlock + threadIdx.x * 4;
-    int v[4];
+    extern __shared__ int hist[];
+    for (int b = threadIdx.x; b < n_bins; b += 256) hist[b] = 0;
+    __syncthreads();
+    const int e0 = blockIdx.x * per_part, e1 = min(total, e0 + per_part);
+    for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
+        int q[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) v[j] = i0 + j < N ? deg[i0 + j] : 0;
-    const int mine = v[0] + v[1] + v[2] + v[3];
-    int tot;
-    int run = block_scan_256(mine, &tot, lds4);
+        for (int u = 0; u < 4; ++u) q[u] = e + 256 * u < e1 ? old_idx[e + 256 * u] : -1;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        if (i0 + j < N) offs[i0 + j] = run;
-        run += v[j];
+        for (int u = 0; u < 4; ++u)
+            if (q[u] >= 0 && q[u] < N) atomicAdd(&hist[q[u] >> shift], 1);
     }
-    if (threadIdx.x == 0) totals[blockIdx.x] = tot;
+    __syncthreads();
+    for (int b = threadIdx.x; b < n_bins; b += 256) {
+        const int c = hist[b];
+        part_off[(size_t)blockIdx.x * n_bins + b] = c ? atomicAdd(&bin_size[b], c) : 0;
+    }
 }
 
-// exclusive scan of the block totals in place, one workgroup; also writes the grand total to *last
-__global__ __launch_bounds__(256) void k_scan_totals(int* __restrict__ totals, int n_blocks, int* __restrict__ last)
+// bin_start = exclusive scan of bin_size (one workgroup); the number of valid entries goes to bin_start[n_bins] and *last
+__global__ __launch_bounds__(256) void k_bin_scan(const int* __restrict__ bin_size, int n_bins, int* __restrict__ bin_start,
+                                                  int* __restrict__ last)
 {
     __shared__ int lds4[4];
     int carry = 0;
-    for (int b0 = 0; b0 < n_blocks; b0 += 256) {
+    for (int b0 = 0; b0 < n_bins; b0 += 256) {
         const int i = b0 + threadIdx.x;
-        const int v = i < n_blocks ? totals[i] : 0;
+        const int v = i < n_bins ? bin_size[i] : 0;
         int tot;
-        const int ex = block_scan_256(v, &tot, lds4);
-        if (i < n_blocks) totals[i] = carry + ex;
+        const int ex = block_excl_scan(v, &tot, lds4);
+        if (i < n_bins) bin_start[i] = carry + ex;
         carry += tot;
     }
-    if (threadIdx.x == 0) *last = carry;
+    if (threadIdx.x == 0) { bin_start[n_bins] = carry; *last = carry; }
 }
 
-__global__ __launch_bounds__(256) void k_scan_add(int* __restrict__ offs, int N, const int* __restrict__ totals)
+__global__ __launch_bounds__(256) void k_bin_scatter(const int* __restrict__ old_idx, int total, int per_part, int N, int shift,
+                                                     int n_bins, const int* __restrict__ bin_start,
+                                                     const int* __restrict__ part_off, int* __restrict__ bin_e,
+                                                     uint16_t* __restrict__ bin_q)
 {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < N) offs[i] += totals[i / kScanBlock];
-}
-
-__global__ void k_fill_rev(const int* __restrict__ old_idx, size_t total, int N, int K, int* __restrict__ deg,
-                           const int* __restrict__ offs, int* __restrict__ rev, int* __restrict__ fwd2rev)
-{
-    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
-        const int q = old_idx[e];
-        int j = -1;
-        if (q >= 0 && q < N) {
-            j = offs[q] + atomicSub(&deg[q], 1) - 1;
-            rev[j] = (int)(e / (size_t)K);
+    extern __shared__ int cursor[];
+    for (int b = threadIdx.x; b < n_bins; b += 256) cursor[b] = bin_start[b] + part_off[(size_t)blockIdx.x * n_bins + b];
+    __syncthreads();
+    const int low = (1 << shift) - 1;
+    const int e0 = blockIdx.x * per_part, e1 = min(total, e0 + per_part);
+    for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
+        int q[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) q[u] = e + 256 * u < e1 ? old_idx[e + 256 * u] : -1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (q[u] >= 0 && q[u] < N) {
+                const int at = atomicAdd(&cursor[q[u] >> shift], 1);
+                bin_e[at] = e + 256 * u;
+                bin_q[at] = (uint16_t)(q[u] & low);
+            }
         }
-        fwd2rev[e] = j;
     }
 }
 
-// One wavefront per q.  Per-wavefront LDS (ints): cq[KP] | pid[32] | pn[32] | ptau[32], KP = K rounded up to 32.
+// One workgroup per bin.  LDS: one counter per point of the bin.
+__global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int* __restrict__ bin_e, const uint16_t* __restrict__ bin_q,
+                                                         const int* __restrict__ bin_start, int shift, int N,
+                                                         int* __restrict__ offs, int* __restrict__ rev)
+{
+    extern __shared__ int cnt[];
+    __shared__ int wave_lds[kRowsBlock / 64];
+    const int R = 1 << shift;
+    const int b = blockIdx.x;
+    const int s0 = bin_start[b], s1 = bin_start[b + 1];
+    const int q0 = b << shift;
+    for (int i = threadIdx.x; i < R; i += kRowsBlock) cnt[i] = 0;
+    __syncthreads();
+    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) atomicAdd(&cnt[bin_q[i]], 1);
+    __syncthreads();
+    int carry = 0;
+    for (int c0 = 0; c0 < R; c0 += kRowsBlock) {
+        const int v = cnt[c0 + threadIdx.x];
+        int tot;
+        const int ex = block_excl_scan(v, &tot, wave_lds);
+        cnt[c0 + threadIdx.x] = carry + ex;
+        if (q0 + c0 + (int)threadIdx.x < N) offs[q0 + c0 + threadIdx.x] = s0 + carry + ex;
+        carry += tot;
+    }
+    __syncthreads();
+    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) {
+        const int at = atomicAdd(&cnt[bin_q[i]], 1);
+        rev[s0 + at] = bin_e[i];
+    }
+}
+
+// One wavefront per q.  Per-wavefront LDS (ints): cq[KP] | pid[32] | pn[32] | ptau[32] | pe[32], KP = K rounded up to 32.
 template <int WAVES, bool BOUNDS>
 __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N, int K, const int* __restrict__ old_idx,
                                                               const float* __restrict__ knn_dist,
                                                               const int* __restrict__ offs, const int* __restrict__ rev,
                                                               uint32_t* __restrict__ pass, uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
-                                                              float kappa, float one_minus_gamma, int wave_lds_ints)
+                                                              float kappa, float one_minus_gamma, int wave_lds_ints,
+                                                              uint32_t div_m, int div_s)
 {
     extern __shared__ __align__(16) int lds_join[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -163,6 +222,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
     int* pid = cq + KP;
     float* pn = reinterpret_cast<float*>(pid + 32);
     float* ptau = pn + 32;
+    int* pe = reinterpret_cast<int*>(ptau + 32);
     const int MW = KP >> 5;
 
     for (int k = lane; k < KP; k += 64) {
@@ -174,9 +234,12 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
     for (int pt0 = 0; pt0 < R; pt0 += 32) {
         const int np = min(32, R - pt0);
         wave_lds_sync();                                  // reads of the previous tile are done (and cq is written)
+        int my_e = -1;                                    // lanes 0..31: the graph entry (p, k) with q = neighbour k of p
         if (lane < 32) {
-            const int p = lane < np ? rev[(size_t)r0 + pt0 + lane] : -1;
+            my_e = lane < np ? rev[(size_t)r0 + pt0 + lane] : -1;
+            const int p = my_e >= 0 ? (int)(((uint64_t)div_m * (uint64_t)(uint32_t)my_e) >> div_s) : -1;
             pid[lane] = p;
+            pe[lane] = my_e;
             pn[lane] = p >= 0 ? bf.norms[p] : 0.0f;
             ptau[lane] = p >= 0 ? knn_dist[(size_t)p * K + (K - 1)] : 0.0f;
         }
@@ -225,31 +288,33 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
                 if (BOUNDS && marked && m < np) {
                     // a bound below zero (or NaN) says nothing: 0.  Dropping the low half of a positive float rounds down.
                     const uint32_t lb = lower > 0.0f ? __float_as_uint(lower) >> 16 : 0u;
-                    bounds[((size_t)r0 + pt0 + m) * (size_t)KP + ct * 32 + (lane & 31)] = (uint16_t)lb;
+                    bounds[(size_t)pe[m] * (size_t)KP + ct * 32 + (lane & 31)] = (uint16_t)lb;
                 }
                 const int m_lo = 8 * (i >> 2) + (i & 3);
                 if (lane == m_lo) mine = (uint32_t)bm;
                 if (lane == m_lo + 4) mine = (uint32_t)(bm >> 32);
             }
-            if (lane < np) pass[((size_t)r0 + pt0 + lane) * MW + ct] = mine;
+            if (lane < np) pass[(size_t)my_e * MW + ct] = mine;
         }
     }
 }
 
 }  // namespace
 
-// The join is used unless RSFK_EXPLORE_JOIN=0 is set or the graph has 2^31 or more entries.
+// The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has 2^31 or more entries or N is beyond what the
+// builder of the reversed graph takes (8192 bins of 2^13 points).
 bool explore_join_enabled(int N, int K)
 {
     const char* env = std::getenv("RSFK_EXPLORE_JOIN");
     if (env && env[0] == '0') return false;
-    return (size_t)N * (size_t)K < ((size_t)1 << 31);
+    int shift, n_bins;
+    return (size_t)N * (size_t)K < ((size_t)1 << 31) && rev_bins(N, &shift, &n_bins);
 }
 
 size_t explore_ws_bytes(int N, int K)
 {
     const size_t mw = (size_t)((K + 31) / 32);
-    return (size_t)N * ((size_t)K * 4 * (2 + mw) + 24) + 4096;
+    return (size_t)N * ((size_t)K * (10 + 4 * mw) + 24) + ((size_t)20 << 20);
 }
 
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
@@ -259,11 +324,23 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     w->N = N;
     w->K = K;
     w->MW = (K + 31) / 32;
-    w->n_blocks = (N + kScanBlock - 1) / kScanBlock;
+    if (!rev_bins(N, &w->shift, &w->n_bins) || (size_t)N * (size_t)K >= ((size_t)1 << 31)) {
+        delete w;
+        set_last_error("exploration workspace: graph too large for the join");
+        return 1;
+    }
+    const size_t total = (size_t)N * (size_t)K;
+    w->n_parts = (int)std::min<size_t>(512, std::max<size_t>(1, (total + 8191) / 8192));
+    w->per_part = (int)(((total + w->n_parts - 1) / w->n_parts + 1023) / 1024 * 1024);
+    int l = 0;
+    while ((1 << l) < K) ++l;
+    w->div_s = 31 + l;
+    w->div_m = (uint32_t)((((uint64_t)1 << w->div_s) + (uint64_t)K - 1) / (uint64_t)K);
     auto dm = [](void* p, size_t n) { return ws_alloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)) ? hipErrorOutOfMemory : hipSuccess; };
-    if (dm(&w->rev, (size_t)N * K) != hipSuccess || dm(&w->fwd2rev, (size_t)N * K) != hipSuccess ||
-        dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->deg, (size_t)N) != hipSuccess ||
-        dm(&w->totals, (size_t)w->n_blocks + 1) != hipSuccess || dm(&w->pass, (size_t)N * K * w->MW) != hipSuccess ||
+    if (dm(&w->rev, total) != hipSuccess || dm(&w->bin_e, total) != hipSuccess || dm(&w->bin_q, (total + 1) / 2) != hipSuccess ||
+        dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->bin_size, (size_t)w->n_bins) != hipSuccess ||
+        dm(&w->bin_start, (size_t)w->n_bins + 1) != hipSuccess ||
+        dm(&w->part_off, (size_t)w->n_parts * (size_t)w->n_bins) != hipSuccess || dm(&w->pass, total * w->MW) != hipSuccess ||
         dm(&w->todo, 2 * ((size_t)N + 1)) != hipSuccess ||
         hipHostMalloc(reinterpret_cast<void**>(&w->host_count), sizeof(int)) != hipSuccess) {
         explore_ws_free(w);
@@ -273,7 +350,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     if (with_bounds) {
         // 2 bytes per pair of the join; without them the merge still works, in the order of the marks
         void* b = nullptr;
-        if (ws_alloc(&b, (size_t)N * K * w->MW * 32 * sizeof(uint16_t)) == 0) w->bounds = static_cast<uint16_t*>(b);
+        if (ws_alloc(&b, total * w->MW * 32 * sizeof(uint16_t)) == 0) w->bounds = static_cast<uint16_t*>(b);
     }
     *out = w;
     return 0;
@@ -282,41 +359,42 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->fwd2rev, w->offs, w->deg, w->totals, w->pass, w->todo, w->bounds};
+    void* bufs[] = {w->rev, w->bin_e, w->bin_q, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->todo, w->bounds};
     for (void* b : bufs)
         ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
     delete w;
 }
 
-const int* explore_ws_fwd2rev(const ExploreWorkspace* w) { return w->fwd2rev; }
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w) { return w->pass; }
 const uint16_t* explore_ws_bounds(const ExploreWorkspace* w) { return w->bounds; }
 int* explore_ws_todo(ExploreWorkspace* w, int which) { return w->todo + (size_t)which * ((size_t)w->N + 1); }
 int* explore_ws_host_count(ExploreWorkspace* w) { return w->host_count; }
 
-// Fill pass and fwd2rev from the snapshot old_idx and the current last slots of knn_dist (rows sorted by distance).
+// Fill pass (and bounds) from the snapshot old_idx and the current last slots of knn_dist (rows sorted by distance).
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
                         const float* knn_dist, hipStream_t stream)
 {
     RSFK_CHECK(w && w->N == N && w->K == K, "exploration join: workspace does not match");
     RSFK_CHECK(K >= 1 && K <= 256, "exploration join: K must be in 1..256");
     RSFK_CHECK((size_t)N * (size_t)K < ((size_t)1 << 31), "exploration join: N*K must be below 2^31");
-    const size_t total = (size_t)N * (size_t)K;
-    const int nb = w->n_blocks;
-    const unsigned wide = (unsigned)std::min<size_t>((total + 255) / 256, 65536);
-    hipLaunchKernelGGL(k_zero, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, w->deg, N, w->todo + N, w->todo + 2 * (size_t)N + 1);
-    hipLaunchKernelGGL(k_degree, dim3(wide), dim3(256), 0, stream, old_idx, total, N, w->deg);
-    hipLaunchKernelGGL(k_scan_blocks, dim3((unsigned)nb), dim3(256), 0, stream, w->deg, N, w->offs, w->totals);
-    hipLaunchKernelGGL(k_scan_totals, dim3(1), dim3(256), 0, stream, w->totals, nb, w->offs + N);
-    hipLaunchKernelGGL(k_scan_add, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, w->offs, N, w->totals);
-    hipLaunchKernelGGL(k_fill_rev, dim3(wide), dim3(256), 0, stream, old_idx, total, N, K, w->deg, w->offs, w->rev,
-                       w->fwd2rev);
+    const int total = (int)((size_t)N * (size_t)K);
+    const int nbins = w->n_bins;
+    const size_t bin_lds = (size_t)nbins * sizeof(int);
+    hipLaunchKernelGGL(k_zero, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, w->bin_size, nbins, w->todo + N,
+                       w->todo + 2 * (size_t)N + 1);
+    hipLaunchKernelGGL(k_bin_count, dim3((unsigned)w->n_parts), dim3(256), bin_lds, stream, old_idx, total, w->per_part, N,
+                       w->shift, nbins, w->bin_size, w->part_off);
+    hipLaunchKernelGGL(k_bin_scan, dim3(1), dim3(256), 0, stream, w->bin_size, nbins, w->bin_start, w->offs + N);
+    hipLaunchKernelGGL(k_bin_scatter, dim3((unsigned)w->n_parts), dim3(256), bin_lds, stream, old_idx, total, w->per_part, N,
+                       w->shift, nbins, w->bin_start, w->part_off, w->bin_e, w->bin_q);
+    hipLaunchKernelGGL(k_bin_rows, dim3((unsigned)nbins), dim3(kRowsBlock), sizeof(int) << w->shift, stream, w->bin_e, w->bin_q,
+                       w->bin_start, w->shift, N, w->offs, w->rev);
     RSFK_HIP(hipGetLastError());
 
     constexpr int kWaves = 4;
     const int KP = (K + 31) & ~31;
-    const int wave_ints = (KP + 96 + 3) & ~3;
+    const int wave_ints = (KP + 128 + 3) & ~3;
     const size_t lds = (size_t)kWaves * (size_t)wave_ints * sizeof(int);
     const int ksteps = (bf16_valid(D) + 15) / 16;
     RSFK_CHECK(ksteps * 16 <= bf16_pitch(D), "exploration join: bfloat16 rows too short");
@@ -326,11 +404,11 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     if (w->bounds)
         hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
-                           kappa, one_minus_gamma, wave_ints);
+                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
     else
         hipLaunchKernelGGL((k_explore_join<kWaves, false>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
-                           kappa, one_minus_gamma, wave_ints);
+                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

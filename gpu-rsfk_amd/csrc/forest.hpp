@@ -72,7 +72,6 @@ bool explore_join_enabled(int N, int K);
 size_t explore_ws_bytes(int N, int K);
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds = false);
 void explore_ws_free(ExploreWorkspace* w);
-const int* explore_ws_fwd2rev(const ExploreWorkspace* w);
 const uint32_t* explore_ws_pass(const ExploreWorkspace* w);
 const uint16_t* explore_ws_bounds(const ExploreWorkspace* w);
 int* explore_ws_todo(ExploreWorkspace* w, int which);
