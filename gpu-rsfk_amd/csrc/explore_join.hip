@@ -50,6 +50,7 @@ struct ExploreWorkspace {
     int* bin_start = nullptr;  // n_bins + 1
     int* part_off = nullptr;   // n_parts x n_bins: where the entries of a part start inside a bin
     uint32_t* pass = nullptr;  // N*K*MW, indexed by entry number
+    float2* norm_tau = nullptr; // N: norm of the bfloat16 row and last slot of the K-NN row of a point, side by side
     uint16_t* bounds = nullptr; // N*K*32*MW lower bounds of the marked pairs (bfloat16, rounded down), or null
     int* todo = nullptr;       // two lists of N+1 ints: points left over by a launch; entry N = their number
     int* host_count = nullptr; // pinned
@@ -203,10 +204,18 @@ __global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int* __restrict__
     }
 }
 
+// What the join needs of a point besides its row, in one 8-byte record (one gather instead of two).
+__global__ void k_norm_tau(const float* __restrict__ norms, const float* __restrict__ knn_dist, int N, int K,
+                           float2* __restrict__ out)
+{
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < N) out[p] = make_float2(norms[p], knn_dist[(size_t)p * K + (K - 1)]);
+}
+
 // One wavefront per q.  Per-wavefront LDS (ints): cq[KP] | pid[32] | pn[32] | ptau[32] | pe[32], KP = K rounded up to 32.
 template <int WAVES, bool BOUNDS>
 __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N, int K, const int* __restrict__ old_idx,
-                                                              const float* __restrict__ knn_dist,
+                                                              const float2* __restrict__ norm_tau,
                                                               const int* __restrict__ offs, const int* __restrict__ rev,
                                                               uint32_t* __restrict__ pass, uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
                                                               float kappa, float one_minus_gamma, int wave_lds_ints,
@@ -240,8 +249,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
             const int p = my_e >= 0 ? (int)(((uint64_t)div_m * (uint64_t)(uint32_t)my_e) >> div_s) : -1;
             pid[lane] = p;
             pe[lane] = my_e;
-            pn[lane] = p >= 0 ? bf.norms[p] : 0.0f;
-            ptau[lane] = p >= 0 ? knn_dist[(size_t)p * K + (K - 1)] : 0.0f;
+            const float2 nt = p >= 0 ? norm_tau[p] : make_float2(0.0f, 0.0f);
+            pn[lane] = nt.x;
+            ptau[lane] = nt.y;
         }
         wave_lds_sync();
 
@@ -251,7 +261,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
         for (int ct = 0; ct < MW; ++ct) {
             const int cid = cq[ct * 32 + (lane & 31)];
             const uint16_t* rb = bf.rows + (size_t)(cid >= 0 ? cid : q) * (size_t)bpitch + 8 * (lane >> 5);
-            const float cn = cid >= 0 ? bf.norms[cid] : 0.0f;
+            const float cn = cid >= 0 ? norm_tau[cid].x : 0.0f;
             f32x16 g;
 #pragma unroll
             for (int i = 0; i < 16; ++i) g[i] = 0.0f;
@@ -314,7 +324,7 @@ bool explore_join_enabled(int N, int K)
 size_t explore_ws_bytes(int N, int K)
 {
     const size_t mw = (size_t)((K + 31) / 32);
-    return (size_t)N * ((size_t)K * (10 + 4 * mw) + 24) + ((size_t)20 << 20);
+    return (size_t)N * ((size_t)K * (10 + 4 * mw) + 32) + ((size_t)20 << 20);
 }
 
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
@@ -340,7 +350,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     if (dm(&w->rev, total) != hipSuccess || dm(&w->bin_e, total) != hipSuccess || dm(&w->bin_q, (total + 1) / 2) != hipSuccess ||
         dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->bin_size, (size_t)w->n_bins) != hipSuccess ||
         dm(&w->bin_start, (size_t)w->n_bins + 1) != hipSuccess ||
-        dm(&w->part_off, (size_t)w->n_parts * (size_t)w->n_bins) != hipSuccess || dm(&w->pass, total * w->MW) != hipSuccess ||
+        dm(&w->part_off, (size_t)w->n_parts * (size_t)w->n_bins) != hipSuccess || dm(&w->pass, total * w->MW) != hipSuccess || dm(&w->norm_tau, 2 * (size_t)N) != hipSuccess ||
         dm(&w->todo, 2 * ((size_t)N + 1)) != hipSuccess ||
         hipHostMalloc(reinterpret_cast<void**>(&w->host_count), sizeof(int)) != hipSuccess) {
         explore_ws_free(w);
@@ -359,7 +369,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->bin_e, w->bin_q, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->todo, w->bounds};
+    void* bufs[] = {w->rev, w->bin_e, w->bin_q, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->norm_tau, w->todo, w->bounds};
     for (void* b : bufs)
         ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
@@ -390,6 +400,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
                        w->shift, nbins, w->bin_start, w->part_off, w->bin_e, w->bin_q);
     hipLaunchKernelGGL(k_bin_rows, dim3((unsigned)nbins), dim3(kRowsBlock), sizeof(int) << w->shift, stream, w->bin_e, w->bin_q,
                        w->bin_start, w->shift, N, w->offs, w->rev);
+    hipLaunchKernelGGL(k_norm_tau, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, bf.norms, knn_dist, N, K, w->norm_tau);
     RSFK_HIP(hipGetLastError());
 
     constexpr int kWaves = 4;
@@ -403,11 +414,11 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     RSFK_CHECK(one_minus_gamma > 0.5f, "exploration join: D too large");
     if (w->bounds)
         hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
-                           stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
+                           stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
                            kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
     else
         hipLaunchKernelGGL((k_explore_join<kWaves, false>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
-                           stream, bf, N, K, old_idx, knn_dist, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
+                           stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
                            kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
     RSFK_HIP(hipGetLastError());
     return 0;
