@@ -309,6 +309,97 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
     }
 }
 
+// The join for rows of at most 32 neighbours and points of at most 128 dimensions (KS = steps of 16 dimensions, fixed
+// at compile time: 2, 4 or 8).  One word of marks per graph entry; the rows of the neighbours of q are loaded once
+// and stay in registers for all tiles of R(q); the norm and last slot of the points of a tile travel while their rows
+// are fetched.  A wavefront then has three dependent trips to memory per q (row offsets and neighbours | their rows
+// and the elements of R(q) | the rows of those points) instead of five, and short rows leave room for twice the
+// wavefronts per SIMD.  The bound is that of k_explore_join, term by term.
+template <int WAVES, int KS>
+__global__ __launch_bounds__(64 * WAVES) void k_explore_join_short(Bf16Copy bf, int N, int K, const int* __restrict__ old_idx,
+                                                                    const float2* __restrict__ norm_tau,
+                                                                    const int* __restrict__ offs, const int* __restrict__ rev,
+                                                                    uint32_t* __restrict__ pass, int bpitch, int ksteps,
+                                                                    float kappa, float one_minus_gamma, uint32_t div_m, int div_s)
+{
+    __shared__ int pid_s[WAVES][32];
+    __shared__ float pn_s[WAVES][32], ptau_s[WAVES][32];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int q = blockIdx.x * WAVES + wave;
+    if (q >= N) return;                                   // whole wavefront leaves together
+    const int r0 = offs[q], R = offs[q + 1] - r0;
+    const int col = lane & 31, hi = lane >> 5;
+    int cid = col < K ? old_idx[(size_t)q * K + col] : -1;
+    if (R <= 0) return;
+    if (cid < 0 || cid >= N) cid = -1;
+    const uint16_t* rb = bf.rows + (size_t)(cid >= 0 ? cid : q) * (size_t)bpitch + 8 * hi;
+    bf16x8 b[KS];
+#pragma unroll
+    for (int u = 0; u < KS; ++u) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b[u][i] = (__bf16)0.0f;
+        if (u < ksteps) b[u] = *reinterpret_cast<const bf16x8*>(rb + 16 * u);
+    }
+    const float cn = cid >= 0 ? norm_tau[cid].x : 0.0f;
+    const int mbase = 4 * hi;
+    int* pid = pid_s[wave];
+    float* pn = pn_s[wave];
+    float* ptau = ptau_s[wave];
+
+    for (int pt0 = 0; pt0 < R; pt0 += 32) {
+        const int np = min(32, R - pt0);
+        int my_e = -1;                                    // lanes 0..31: the graph entry (p, k) with q = neighbour k of p
+        float2 nt = make_float2(0.0f, 0.0f);
+        if (lane < 32) {
+            my_e = lane < np ? rev[(size_t)r0 + pt0 + lane] : -1;
+            const int p = my_e >= 0 ? (int)(((uint64_t)div_m * (uint64_t)(uint32_t)my_e) >> div_s) : -1;
+            pid[lane] = p;
+            if (p >= 0) nt = norm_tau[p];
+        }
+        wave_lds_sync();
+        const int pm = pid[col];
+        const uint16_t* ra = bf.rows + (size_t)(pm >= 0 ? pm : q) * (size_t)bpitch + 8 * hi;
+        bf16x8 a[KS];
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[u][i] = (__bf16)0.0f;
+            if (u < ksteps) a[u] = *reinterpret_cast<const bf16x8*>(ra + 16 * u);
+        }
+        f32x16 g;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) g[i] = 0.0f;
+#pragma unroll
+        for (int u = 0; u < KS; ++u) g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[u], b[u], g, 0, 0, 0);
+        if (lane < 32) {
+            pn[lane] = nt.x;
+            ptau[lane] = nt.y;
+        }
+        wave_lds_sync();
+        // Accumulator i of lane l: point m = 4 (l / 32) + 8 (i / 4) + i % 4 of the tile, column = neighbour l % 32.
+        uint32_t mine = 0;                                // mask of the point this lane stores (lanes 0..31)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = mbase + 8 * (i >> 2) + (i & 3);
+            const float S = pn[m] + cn;
+            const float dt = __builtin_fmaf(-2.0f, g[i], S);
+            const float e1 = kappa * S;
+            const float dhi = fmaxf(dt + e1, 0.0f);
+            const float Q = 2.0001f * S;
+            const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);
+            const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;
+            const bool skip = lower > ptau[m];            // false if anything is NaN; a tie at the last slot may still enter
+            const uint64_t bm = ballot64(cid >= 0 && !skip);
+            const int m_lo = 8 * (i >> 2) + (i & 3);
+            if (lane == m_lo) mine = (uint32_t)bm;
+            if (lane == m_lo + 4) mine = (uint32_t)(bm >> 32);
+            if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // four at a time: all sixteen at once take too many registers
+        }
+        if (lane < np) pass[(size_t)my_e] = mine;
+        wave_lds_sync();                                  // the tile's LDS values are read before the next tile writes them
+    }
+}
+
 }  // namespace
 
 // The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has 2^31 or more entries or N is beyond what the
@@ -412,7 +503,16 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     const float kappa = (float)(ksteps * 16 + 16) * (1.0f / 2097152.0f);            // (Dp + 16) 2^-21
     const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
     RSFK_CHECK(one_minus_gamma > 0.5f, "exploration join: D too large");
-    if (w->bounds)
+    if (!w->bounds && KP == 32 && ksteps <= 8) {
+        const dim3 grid((unsigned)((N + kWaves - 1) / kWaves)), block(64 * kWaves);
+#define RSFK_JOIN_SHORT(KSV)                                                                                                \
+        hipLaunchKernelGGL((k_explore_join_short<kWaves, KSV>), grid, block, 0, stream, bf, N, K, old_idx, w->norm_tau, w->offs, \
+                           w->rev, w->pass, bf16_pitch(D), ksteps, kappa, one_minus_gamma, w->div_m, w->div_s)
+        if (ksteps <= 2) RSFK_JOIN_SHORT(2);
+        else if (ksteps <= 4) RSFK_JOIN_SHORT(4);
+        else RSFK_JOIN_SHORT(8);
+#undef RSFK_JOIN_SHORT
+    } else if (w->bounds)
         hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
                            kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
