@@ -113,4 +113,39 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
     row.merge(lane < n && finished, my_c, acc);          // unfinished sums are all above the last slot
 }
 
+// The same without the tile: lane l reads the row of candidate l itself, 32 dimensions (eight 16-byte pieces) per
+// step, and runs its chain from registers; the point's coordinates come from L.xrow (every lane reads the same
+// word).  For short rows: no LDS besides xrow, no synchronisation inside the batch.
+template <int SL>
+__device__ __forceinline__ void exact_direct(const ExploreLds& L, const int* list, int n, const float* __restrict__ points,
+                                             int D, bool vec_ok, KnnRow<SL>& row, float tau_cap = INFINITY)
+{
+    const int lane = lane_id();
+    const int my_c = lane < n ? list[lane] : -1;
+    const float* rp = points + (size_t)(my_c >= 0 ? my_c : 0) * (size_t)D;
+    float acc = 0.0f;
+    const float tau0 = fminf(row.tau, tau_cap);
+    bool finished = true;
+    for (int d0 = 0; d0 < D; d0 += 32) {
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            v[i] = my_c >= 0 ? load_piece(rp, d0 + 4 * i, D, vec_ok) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (d0 + 4 * i < D) {                         // (wave-uniform; xrow is zero beyond D like the pieces)
+                const float4 x = *reinterpret_cast<const float4*>(&L.xrow[d0 + 4 * i]);
+                float df;
+                df = v[i].x - x.x; acc = __builtin_fmaf(df, df, acc);
+                df = v[i].y - x.y; acc = __builtin_fmaf(df, df, acc);
+                df = v[i].z - x.z; acc = __builtin_fmaf(df, df, acc);
+                df = v[i].w - x.w; acc = __builtin_fmaf(df, df, acc);
+            }
+        }
+        // partial sums only grow: once all of them are above the row maximum nothing can enter
+        if (ballot64(lane < n && acc <= tau0) == 0) { finished = false; break; }
+    }
+    row.merge(lane < n && finished, my_c, acc);          // unfinished sums are all above the last slot
+}
+
 }  // namespace rsfk

@@ -318,12 +318,25 @@ __device__ __forceinline__ int graph_entry(const int* __restrict__ old_idx, int 
 
 constexpr int kMergeChunk = 16;
 constexpr int kMergeTile = 64 * (kMergeChunk + 4);
+// Rows of at most this many (padded) dimensions are read by the lane that runs their chain, 32 dimensions at a time,
+// without the transposing tile in LDS (exact_direct): the LDS of a wavefront shrinks by the tile.
+__host__ __device__ inline int merge_tile_ints(int dpad, int direct_max) { return dpad <= direct_max ? 0 : kMergeTile; }
+int merge_direct_max()
+{
+    static const int v = [] {
+        // measured: 1M x 100 merge 4.4 -> 3.4 ms, 10M x 32 43 -> 27 ms; 1M x 256 slower (eight steps, each a trip)
+        const char* e = std::getenv("RSFK_MERGE_DIRECT");
+        return e ? std::atoi(e) : 128;
+    }();
+    return v;
+}
+
 
 template <int SL, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __restrict__ points, int N, int D, int K,
                                                                const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                                float* __restrict__ knn_dist, int table_size,
-                                                               int wave_lds_ints, int dpad,
+                                                               int wave_lds_ints, int dpad, int direct_max,
                                                                const uint32_t* __restrict__ pass,
                                                                const int* __restrict__ todo_in, int n_in,
                                                                int* __restrict__ todo_out, int* __restrict__ n_out)
@@ -349,9 +362,10 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     int* base = lds_m + (size_t)wave * (size_t)wave_lds_ints;
     ExploreLds L;
     L.tile = reinterpret_cast<float*>(base);
-    L.xrow = reinterpret_cast<float*>(base + kMergeTile);
+    const int tile_ints = merge_tile_ints(dpad, direct_max);
+    L.xrow = reinterpret_cast<float*>(base + tile_ints);
     L.queue2 = nullptr;
-    L.table = base + kMergeTile + dpad;
+    L.table = base + tile_ints + dpad;
     L.srow = L.table + table_size;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
@@ -418,7 +432,8 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     wave_lds_sync();
     for (int off = 0; off < U; off += 64) {
         wave_lds_sync();
-        exact_batch<SL, kMergeChunk>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+        if (tile_ints == 0) exact_direct<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+        else exact_batch<SL, kMergeChunk>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
     }
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
@@ -698,13 +713,16 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
     const int n_work = todo_in ? n_in : N;
     dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, pass, todo_in, n_in, todo_out, n_out);
+                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, todo_in, n_in, todo_out, n_out);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
 
 // ints of LDS a wavefront of the merge kernel needs for a set of `table` entries
-int merge_wave_ints(int table, int dpad, int K) { return (kMergeTile + dpad + table + K + table / 4 * 3 + 3) / 4 * 4; }
+int merge_wave_ints(int table, int dpad, int K)
+{
+    return (merge_tile_ints(dpad, merge_direct_max()) + dpad + table + K + table / 4 * 3 + 3) / 4 * 4;
+}
 
 int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
                    float* knn_dist, int table, int dpad, const uint32_t* pass, const int* todo_in,
