@@ -44,8 +44,8 @@ struct ExploreWorkspace {
     int div_s = 0;
     int* rev = nullptr;        // N*K: R lists in compressed rows; an element is the number p K + k of a graph entry
     int* offs = nullptr;       // N+1: start of R(q)
-    int* bin_e = nullptr;      // N*K: entry numbers grouped by the bin of the neighbour they hold
-    uint16_t* bin_q = nullptr; // N*K: that neighbour minus the first point of its bin
+    int2* bin_eq = nullptr;    // N*K: (entry number, neighbour minus the first point of its bin), grouped by the bin of
+                               // the neighbour; one 8-byte store per entry
     int* bin_size = nullptr;   // n_bins
     int* bin_start = nullptr;  // n_bins + 1
     int* part_off = nullptr;   // n_parts x n_bins: where the entries of a part start inside a bin
@@ -61,15 +61,18 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16
-constexpr int kMaxBins = 8192;
+constexpr int kMaxBins = 6144;
 constexpr int kMaxShift = 13;
 constexpr int kRowsBlock = 512;             // threads of k_bin_rows
 
 // Bins of the reversed-graph builder for N points: false if N is too large for it.
 bool rev_bins(int N, int* shift, int* n_bins)
 {
-    int s = 10;
-    while (s < kMaxShift && (((N - 1) >> s) + 1) > kMaxBins / 2) ++s;
+    // measured: small bins make the placement of k_bin_rows local (1M points: 0.25 ms with bins of 256 points, 0.62 ms
+    // with 1024), many bins make the runs k_bin_scatter writes short (0.49 against 0.36 ms)
+    int s = 8;
+    if (const char* e = std::getenv("RSFK_REV_SHIFT")) s = std::max(8, std::min(kMaxShift, std::atoi(e)));
+    while (s < kMaxShift && (((N - 1) >> s) + 1) > kMaxBins) ++s;
     *shift = s;
     *n_bins = N > 0 ? ((N - 1) >> s) + 1 : 1;
     return *n_bins <= kMaxBins;
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(256) void k_bin_count(const int* __restrict__ old_i
     extern __shared__ int hist[];
     for (int b = threadIdx.x; b < n_bins; b += 256) hist[b] = 0;
     __syncthreads();
-    const int e0 = blockIdx.x * per_part, e1 = min(total, e0 + per_part);
+    const int e0 = blockIdx.x * per_part, e1 = (int)min((long long)total, (long long)e0 + per_part);
     for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
         int q[4];
 #pragma unroll
@@ -150,14 +153,13 @@ __global__ __launch_bounds__(256) void k_bin_scan(const int* __restrict__ bin_si
 
 __global__ __launch_bounds__(256) void k_bin_scatter(const int* __restrict__ old_idx, int total, int per_part, int N, int shift,
                                                      int n_bins, const int* __restrict__ bin_start,
-                                                     const int* __restrict__ part_off, int* __restrict__ bin_e,
-                                                     uint16_t* __restrict__ bin_q)
+                                                     const int* __restrict__ part_off, int2* __restrict__ bin_eq)
 {
     extern __shared__ int cursor[];
     for (int b = threadIdx.x; b < n_bins; b += 256) cursor[b] = bin_start[b] + part_off[(size_t)blockIdx.x * n_bins + b];
     __syncthreads();
     const int low = (1 << shift) - 1;
-    const int e0 = blockIdx.x * per_part, e1 = min(total, e0 + per_part);
+    const int e0 = blockIdx.x * per_part, e1 = (int)min((long long)total, (long long)e0 + per_part);
     for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
         int q[4];
 #pragma unroll
@@ -166,15 +168,14 @@ __global__ __launch_bounds__(256) void k_bin_scatter(const int* __restrict__ old
         for (int u = 0; u < 4; ++u) {
             if (q[u] >= 0 && q[u] < N) {
                 const int at = atomicAdd(&cursor[q[u] >> shift], 1);
-                bin_e[at] = e + 256 * u;
-                bin_q[at] = (uint16_t)(q[u] & low);
+                bin_eq[at] = make_int2(e + 256 * u, q[u] & low);
             }
         }
     }
 }
 
 // One workgroup per bin.  LDS: one counter per point of the bin.
-__global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int* __restrict__ bin_e, const uint16_t* __restrict__ bin_q,
+__global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int2* __restrict__ bin_eq,
                                                          const int* __restrict__ bin_start, int shift, int N,
                                                          int* __restrict__ offs, int* __restrict__ rev)
 {
@@ -186,21 +187,26 @@ __global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int* __restrict__
     const int q0 = b << shift;
     for (int i = threadIdx.x; i < R; i += kRowsBlock) cnt[i] = 0;
     __syncthreads();
-    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) atomicAdd(&cnt[bin_q[i]], 1);
+    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) atomicAdd(&cnt[bin_eq[i].y], 1);
     __syncthreads();
     int carry = 0;
     for (int c0 = 0; c0 < R; c0 += kRowsBlock) {
-        const int v = cnt[c0 + threadIdx.x];
+        const int c = c0 + (int)threadIdx.x;
+        const bool in = c < R;                            // (a bin may have fewer points than the workgroup has threads)
+        const int v = in ? cnt[c] : 0;
         int tot;
         const int ex = block_excl_scan(v, &tot, wave_lds);
-        cnt[c0 + threadIdx.x] = carry + ex;
-        if (q0 + c0 + (int)threadIdx.x < N) offs[q0 + c0 + threadIdx.x] = s0 + carry + ex;
+        if (in) {
+            cnt[c] = carry + ex;
+            if (q0 + c < N) offs[q0 + c] = s0 + carry + ex;
+        }
         carry += tot;
     }
     __syncthreads();
     for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) {
-        const int at = atomicAdd(&cnt[bin_q[i]], 1);
-        rev[s0 + at] = bin_e[i];
+        const int2 eq = bin_eq[i];
+        const int at = atomicAdd(&cnt[eq.y], 1);
+        rev[s0 + at] = eq.x;
     }
 }
 
@@ -403,7 +409,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join_short(Bf16Copy bf, 
 }  // namespace
 
 // The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has 2^31 or more entries or N is beyond what the
-// builder of the reversed graph takes (8192 bins of 2^13 points).
+// builder of the reversed graph takes (6144 bins of 2^13 points).
 bool explore_join_enabled(int N, int K)
 {
     const char* env = std::getenv("RSFK_EXPLORE_JOIN");
@@ -415,7 +421,7 @@ bool explore_join_enabled(int N, int K)
 size_t explore_ws_bytes(int N, int K)
 {
     const size_t mw = (size_t)((K + 31) / 32);
-    return (size_t)N * ((size_t)K * (10 + 4 * mw) + 32) + ((size_t)20 << 20);
+    return (size_t)N * ((size_t)K * (12 + 4 * mw) + 32) + ((size_t)20 << 20);
 }
 
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
@@ -438,7 +444,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     w->div_s = 31 + l;
     w->div_m = (uint32_t)((((uint64_t)1 << w->div_s) + (uint64_t)K - 1) / (uint64_t)K);
     auto dm = [](void* p, size_t n) { return ws_alloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)) ? hipErrorOutOfMemory : hipSuccess; };
-    if (dm(&w->rev, total) != hipSuccess || dm(&w->bin_e, total) != hipSuccess || dm(&w->bin_q, (total + 1) / 2) != hipSuccess ||
+    if (dm(&w->rev, total) != hipSuccess || dm(&w->bin_eq, 2 * total) != hipSuccess ||
         dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->bin_size, (size_t)w->n_bins) != hipSuccess ||
         dm(&w->bin_start, (size_t)w->n_bins + 1) != hipSuccess ||
         dm(&w->part_off, (size_t)w->n_parts * (size_t)w->n_bins) != hipSuccess || dm(&w->pass, total * w->MW) != hipSuccess || dm(&w->norm_tau, 2 * (size_t)N) != hipSuccess ||
@@ -460,7 +466,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->bin_e, w->bin_q, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->norm_tau, w->todo, w->bounds};
+    void* bufs[] = {w->rev, w->bin_eq, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->norm_tau, w->todo, w->bounds};
     for (void* b : bufs)
         ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
@@ -488,8 +494,8 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
                        w->shift, nbins, w->bin_size, w->part_off);
     hipLaunchKernelGGL(k_bin_scan, dim3(1), dim3(256), 0, stream, w->bin_size, nbins, w->bin_start, w->offs + N);
     hipLaunchKernelGGL(k_bin_scatter, dim3((unsigned)w->n_parts), dim3(256), bin_lds, stream, old_idx, total, w->per_part, N,
-                       w->shift, nbins, w->bin_start, w->part_off, w->bin_e, w->bin_q);
-    hipLaunchKernelGGL(k_bin_rows, dim3((unsigned)nbins), dim3(kRowsBlock), sizeof(int) << w->shift, stream, w->bin_e, w->bin_q,
+                       w->shift, nbins, w->bin_start, w->part_off, w->bin_eq);
+    hipLaunchKernelGGL(k_bin_rows, dim3((unsigned)nbins), dim3(kRowsBlock), sizeof(int) << w->shift, stream, w->bin_eq,
                        w->bin_start, w->shift, N, w->offs, w->rev);
     hipLaunchKernelGGL(k_norm_tau, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, bf.norms, knn_dist, N, K, w->norm_tau);
     RSFK_HIP(hipGetLastError());
