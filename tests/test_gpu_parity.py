@@ -117,6 +117,26 @@ def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX
         assert rows_have_no_duplicates(gi)
 
 
+@pytest.mark.parametrize("N,D,K,MIN,MAX", [
+    (4000, 32, 32, 64, 256), (3000, 48, 20, 80, 200), (2500, 16, 64, 70, 250), (3000, 64, 8, 65, 128),
+    (2600, 32, 5, 30, 256),
+])
+def test_bucket_knn_resident_rows_matches_oracle(gpu, orc, rng, N, D, K, MIN, MAX):
+    """Buckets of 73..256 low-dimensional points go to the kernel that keeps a bucket's points in LDS.  Three trees on
+    the same rows of normally distributed points: in the second and third most candidates are above the last slot of
+    the row they are offered to, and many of the others are points the row already holds."""
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    oi, od = orc.init_lists(N, K)
+    gi, gd = orc.init_lists(N, K)
+    for seed in (3, 4, 5):
+        _say("bucket_knn resident rows", N, D, K, MIN, MAX, seed)
+        perm, ls, lz, _ = orc.build_tree(X, MIN, MAX, 5000, seed)
+        orc.bucket_knn(X, K, perm, lz, oi, od, starts=ls)
+        gpu.bucket_knn(X, K, perm, lz, gi, gd, starts=ls)
+        assert_knn_equal(gi, gd, oi, od)
+        assert rows_have_no_duplicates(gi)
+
+
 def test_bucket_knn_single_bucket_is_exact_knn(gpu, rng):
     """One bucket holding every point: the kernel must return exact K-NN."""
     for N, D, K in [(300, 8, 16), (700, 20, 32)]:
