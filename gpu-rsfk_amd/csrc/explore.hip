@@ -772,6 +772,14 @@ bool explore_merge_uses_bounds(int D, int K)
 
 // One exploration pass.  old_idx is scratch of N*K ints (receives the snapshot).
 // bf may be null (or hold null rows): every candidate then gets the exact distance.
+// Rows short enough for the LDS of the merge kernels: the exploration then takes its candidates from the join, and
+// the general kernel (the only user of the uncentred copy) only sees what the merge kernels hand back.
+bool explore_merge_fits(int D, int K)
+{
+    const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
+    return 4 * merge_wave_ints(small_table, bf16_valid(D), K) <= 150 * 1024 / 4;
+}
+
 // ws may be null; with a workspace and a bfloat16 copy for the join (bf_join, may be centred; bf must not be)
 // the candidates come from the join over the reversed graph (explore_join.hip), which needs rows sorted by
 // distance.
@@ -784,8 +792,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
     const int dpad = bf16_valid(D);
     const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
     // (rows too long for the LDS of the merge kernel: every point enumerates its own candidates)
-    const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr &&
-                      4 * merge_wave_ints(small_table, dpad, K) <= 150 * 1024 / 4;
+    const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr && explore_merge_fits(D, K);
     if (join && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
     const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set

@@ -63,6 +63,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr float kU = 1.0f / 256.0f;         // unit roundoff of bfloat16
 constexpr int kMaxBins = 6144;
 constexpr int kMaxShift = 13;
+// entry numbers are ints, and the passes over the graph look 768 entries ahead of the one they test
+constexpr size_t kMaxEntries = ((size_t)1 << 31) - 4096;
 constexpr int kRowsBlock = 512;             // threads of k_bin_rows
 
 // Bins of the reversed-graph builder for N points: false if N is too large for it.
@@ -118,7 +120,8 @@ __global__ __launch_bounds__(256) void k_bin_count(const int* __restrict__ old_i
     extern __shared__ int hist[];
     for (int b = threadIdx.x; b < n_bins; b += 256) hist[b] = 0;
     __syncthreads();
-    const int e0 = blockIdx.x * per_part, e1 = (int)min((long long)total, (long long)e0 + per_part);
+    const long long first = (long long)blockIdx.x * per_part;
+    const int e0 = (int)min((long long)total, first), e1 = (int)min((long long)total, first + per_part);
     for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
         int q[4];
 #pragma unroll
@@ -159,7 +162,8 @@ __global__ __launch_bounds__(256) void k_bin_scatter(const int* __restrict__ old
     for (int b = threadIdx.x; b < n_bins; b += 256) cursor[b] = bin_start[b] + part_off[(size_t)blockIdx.x * n_bins + b];
     __syncthreads();
     const int low = (1 << shift) - 1;
-    const int e0 = blockIdx.x * per_part, e1 = (int)min((long long)total, (long long)e0 + per_part);
+    const long long first = (long long)blockIdx.x * per_part;
+    const int e0 = (int)min((long long)total, first), e1 = (int)min((long long)total, first + per_part);
     for (int e = e0 + (int)threadIdx.x; e < e1; e += 1024) {
         int q[4];
 #pragma unroll
@@ -408,14 +412,14 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join_short(Bf16Copy bf, 
 
 }  // namespace
 
-// The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has 2^31 or more entries or N is beyond what the
+// The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has about 2^31 or more entries or N is beyond what the
 // builder of the reversed graph takes (6144 bins of 2^13 points).
 bool explore_join_enabled(int N, int K)
 {
     const char* env = std::getenv("RSFK_EXPLORE_JOIN");
     if (env && env[0] == '0') return false;
     int shift, n_bins;
-    return (size_t)N * (size_t)K < ((size_t)1 << 31) && rev_bins(N, &shift, &n_bins);
+    return (size_t)N * (size_t)K < kMaxEntries && rev_bins(N, &shift, &n_bins);
 }
 
 size_t explore_ws_bytes(int N, int K)
@@ -431,7 +435,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     w->N = N;
     w->K = K;
     w->MW = (K + 31) / 32;
-    if (!rev_bins(N, &w->shift, &w->n_bins) || (size_t)N * (size_t)K >= ((size_t)1 << 31)) {
+    if (!rev_bins(N, &w->shift, &w->n_bins) || (size_t)N * (size_t)K >= kMaxEntries) {
         delete w;
         set_last_error("exploration workspace: graph too large for the join");
         return 1;
@@ -484,7 +488,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 {
     RSFK_CHECK(w && w->N == N && w->K == K, "exploration join: workspace does not match");
     RSFK_CHECK(K >= 1 && K <= 256, "exploration join: K must be in 1..256");
-    RSFK_CHECK((size_t)N * (size_t)K < ((size_t)1 << 31), "exploration join: N*K must be below 2^31");
+    RSFK_CHECK((size_t)N * (size_t)K < kMaxEntries, "exploration join: N*K must be below 2^31 - 4096");
     const int total = (int)((size_t)N * (size_t)K);
     const int nbins = w->n_bins;
     const size_t bin_lds = (size_t)nbins * sizeof(int);

@@ -143,15 +143,18 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
     if (n_trees == 0 && nnef <= 0) return 0;          // nothing to do: no copies are made, nothing is queued
     const double t_forest0 = now_s();
-    Bf16Guard bf;
-    if (bf16_copy_alloc(&bf.c, N, D)) return 1;
-    if (bf16_copy_fill(bf.c, d_points, N, D, stream)) return 1;
-
     const int screen_from = bucket_screen_from(D, K);
 
     Q8Guard q8;
     const uint8_t* q8_rows = nullptr;
     if (n_trees > 0 && make_tree_screen(q8, d_points, N, D, verbose, stream, &q8_rows)) return 1;
+    // The uncentred bfloat16 copy screens the side tests when the 8-bit copy does not, and the general exploration
+    // kernel; with the 8-bit screen and the join nobody needs it (the few points the merge kernels may hand back to
+    // the general kernel are then worked on without a screen).
+    const bool join_explores = nnef > 0 && explore_join_enabled(N, K) && explore_merge_fits(D, K);
+    const bool plain_copy = (n_trees > 0 && q8_rows == nullptr) || (nnef > 0 && !join_explores);
+    Bf16Guard bf;
+    if (plain_copy && (bf16_copy_alloc(&bf.c, N, D) || bf16_copy_fill(bf.c, d_points, N, D, stream))) return 1;
 
     if (n_trees > 0) {
         // the bucket kernels read a row's maximum from its last slot: rows the caller passed in unsorted are put
@@ -244,7 +247,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             if (bf16_copy_alloc(&bfc.c, N, D, true) || bf16_copy_fill(bfc.c, d_points, N, D, stream)) return 1;
         }
         for (int it = 0; it < nnef; ++it) {
-            if (launch_explore(d_points, &bf.c, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream))
+            if (launch_explore(d_points, plain_copy ? &bf.c : nullptr, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream))
                 return 1;
         }
         RSFK_HIP(hipStreamSynchronize(stream));

@@ -69,6 +69,7 @@ void release_copy_buffers();
 // explore_join.hip
 struct ExploreWorkspace;
 bool explore_join_enabled(int N, int K);
+bool explore_merge_fits(int D, int K);
 size_t explore_ws_bytes(int N, int K);
 int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds = false);
 void explore_ws_free(ExploreWorkspace* w);
