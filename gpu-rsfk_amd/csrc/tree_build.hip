@@ -716,8 +716,10 @@ constexpr int kMaxGroup = 16;        // nodes of one level of a subtree worked o
 // fewer, G) at a time -- their hyperplanes are made together (one wavefront each), all their points are tested in
 // one sweep, and each node is partitioned by one wavefront -- so the number of dependent trips to memory per
 // subtree is a few per level instead of a few per node.
-template <bool Q8>
-__global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ points,
+// TB = threads per workgroup: 256, or 1024 for launches over so few subtrees that workgroups of 256 would leave
+// most of the device idle (the phases of a level then have four times the lanes).
+template <bool Q8, int TB>
+__global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
                                                  const uint16_t* __restrict__ pb16, const uint8_t* __restrict__ q8, TreeParams P,
                                                  const int* __restrict__ perm0, const int* __restrict__ perm1,
                                                  int* __restrict__ perm_out,
@@ -753,7 +755,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     if (tk.leaf) {
         // already a bucket (any size): move it to the output buffer and record it
         if (src != dst)
-            for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = src[tk.start + i] & kIdMask;
+            for (int i = tid; i < tk.count; i += TB) dst[tk.start + i] = src[tk.start + i] & kIdMask;
         if (tid == 0) {
             emit_leaf(tk.tree, tk.start, tk.count, tk.depth, leaf_cap, leaf_start, leaf_size, stats, ctr);
             if (recs_all) index_bucket(recs_all + (size_t)tk.tree * rec_cap, rec_cap, tk.rec, tk.start, tk.count, ctr);
@@ -762,7 +764,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     }
     TreeRec* recs = recs_all ? recs_all + (size_t)tk.tree * rec_cap : nullptr;
     int* n_rec = recs_all ? n_rec_all + tk.tree : nullptr;
-    for (int i = tid; i < tk.count; i += kBlock) seg[i] = src[tk.start + i] & kIdMask;
+    for (int i = tid; i < tk.count; i += TB) seg[i] = src[tk.start + i] & kIdMask;
     if (tid == 0) {
         SmallNode r;
         r.start = 0; r.count = tk.count; r.dstart = tk.dstart - tk.start; r.dcount = tk.dcount;
@@ -804,26 +806,27 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                 pre_s[nb] = run;
             }
             __syncthreads();
-            for (int j = wave; j < nb; j += kBlock / 64) {
+            for (int j = wave; j < nb; j += TB / 64) {
                 make_hyperplane_wave(points + (size_t)pair_s[j][0] * P.D, points + (size_t)pair_s[j][1] * P.D, P.D,
                                      nvec + (size_t)j * Dv, hp_s[j]);
                 if (lane == 0) b_s[j] = hp_s[j][0];       // written by this lane just above
             }
             for (int j = 0; j < nb; ++j) {
                 const int c = pre_s[j + 1] - pre_s[j];
-                for (int t = tid; t < c; t += kBlock) fmap[pre_s[j] + t] = (unsigned char)j;
+                for (int t = tid; t < c; t += TB) fmap[pre_s[j] + t] = (unsigned char)j;
             }
             __syncthreads();
             // side of every point of the group's nodes
             const int total = pre_s[nb];
-            const int iters = (total + kGroups - 1) / kGroups;
+            constexpr int kTailGroups = TB / 8;
+            const int iters = (total + kTailGroups - 1) / kTailGroups;
             for (int it = 0; it < iters; it += kTailBatch) {
                 int id[kTailBatch], jj[kTailBatch], pos[kTailBatch];
                 float bb[kTailBatch], h1[kTailBatch], h2[kTailBatch];
                 bool valid[kTailBatch], right[kTailBatch], redo[kTailBatch];
 #pragma unroll
                 for (int u = 0; u < kTailBatch; ++u) {
-                    const int f = (it + u) * kGroups + grp;
+                    const int f = (it + u) * kTailGroups + grp;
                     valid[u] = f < total;
                     jj[u] = valid[u] ? fmap[f] : 0;
                     pos[u] = valid[u] ? start_s[jj[u]] + f - pre_s[jj[u]] : 0;
@@ -846,7 +849,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
                           [&](int pos, bool right) { if (right) seg[pos] |= (int)0x80000000; });
             __syncthreads();
             // stable partition, one wavefront per node: seg -> tmp -> seg
-            for (int j = wave; j < nb; j += kBlock / 64) {
+            for (int j = wave; j < nb; j += TB / 64) {
                 const int st = start_s[j], cnt = pre_s[j + 1] - pre_s[j];
                 int a = 0;
                 for (int r0 = 0; r0 < cnt; r0 += 64) a += __popcll(ballot64(r0 + lane < cnt && seg[st + r0 + lane] >= 0));
@@ -896,7 +899,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
         SmallNode* t = cur; cur = nxt; nxt = t;
         __syncthreads();
     }
-    for (int i = tid; i < tk.count; i += kBlock) dst[tk.start + i] = seg[i];
+    for (int i = tid; i < tk.count; i += TB) dst[tk.start + i] = seg[i];
     if (tid == 0) {
         TreeStats* st = stats + tk.tree;
         base_s[0] = kind_s[0] ? atomicAdd(&st->n_leaves, kind_s[0]) : 0;
@@ -907,7 +910,7 @@ __global__ __launch_bounds__(kBlock) void k_tail(const float* __restrict__ point
     }
     __syncthreads();
     const int nrec = min(nrec_s, node_cap);
-    for (int i = tid; i < nrec; i += kBlock) {
+    for (int i = tid; i < nrec; i += TB) {
         const int2 r = lrec[i];
         const int count = r.y & 0xffff, rank = r.y >> 16;
         store_leaf(tk.tree, r.x, count, base_s[count > kBucketSplit ? 1 : 0] + rank, leaf_cap, leaf_start, leaf_size, ctr);
@@ -1211,19 +1214,23 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         const bool tail_q8 = q8 != nullptr && std::getenv("RSFK_TAIL_BF16") == nullptr;
         (void)hipEventRecord(w->ev[4], stream);
-        if (tail_q8) {
-            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds));
-            hipLaunchKernelGGL(k_tail<true>, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, q8, P, w->perm[0], w->perm[1],
-                               w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr,
-                               w->recs, w->n_rec, w->rec_cap);
-        } else {
-            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds));
-            hipLaunchKernelGGL(k_tail<false>, dim3(n_tail), dim3(kBlock), lds, stream, points, pb16, q8, P, w->perm[0], w->perm[1],
-                               w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start, w->leaf_size, w->stats, w->ctr,
-                               w->recs, w->n_rec, w->rec_cap);
-        }
+        // few subtrees (small inputs, few trees): workgroups of 1024 threads, so that a subtree's levels take less time
+        // (70,000 x 784, 10 trees: 1.24 -> 1.00 ms per tree).  RSFK_TAIL_BLOCK=256 / 1024 overrides.
+        bool wide_wg = n_tail < 8 * 256;
+        if (const char* e = std::getenv("RSFK_TAIL_BLOCK")) wide_wg = std::atoi(e) >= 1024;
+#define RSFK_TAIL_LAUNCH(Q, T)                                                                                             \
+        do {                                                                                                               \
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail<Q, T>),                                      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                          \
+            hipLaunchKernelGGL((k_tail<Q, T>), dim3(n_tail), dim3(T), lds, stream, points, pb16, q8, P, w->perm[0],         \
+                               w->perm[1], w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start,            \
+                               w->leaf_size, w->stats, w->ctr, w->recs, w->n_rec, w->rec_cap);                             \
+        } while (0)
+        if (tail_q8 && wide_wg) RSFK_TAIL_LAUNCH(true, 1024);
+        else if (tail_q8) RSFK_TAIL_LAUNCH(true, 256);
+        else if (wide_wg) RSFK_TAIL_LAUNCH(false, 1024);
+        else RSFK_TAIL_LAUNCH(false, 256);
+#undef RSFK_TAIL_LAUNCH
         (void)hipEventRecord(w->ev[5], stream);
         RSFK_HIP(hipGetLastError());
     }

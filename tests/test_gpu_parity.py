@@ -31,11 +31,16 @@ def _say(*a):
     (5000, 32, 33, 66, "u"), (30000, 100, 33, 66, "u"), (60000, 3, 64, 256, "n"),      # wide phase, several levels
     (20000, 33, 17, 34, "n"), (8000, 784, 91, 182, "sparse"),
 ])
-@pytest.mark.parametrize("screen", ["auto", "q8", "bf16"])
+@pytest.mark.parametrize("screen", ["auto", "q8", "bf16", "q8-256"])
 def test_tree_partition_is_identical(gpu, orc, rng, monkeypatch, N, D, MIN, MAX, dist, screen):
     """screen: which low-precision copy the side tests are screened on (RSFK_TREE_SCREEN; "auto" chooses from the
-    data).  The partition must be the one of the fp32 arithmetic whatever the screen."""
-    if screen != "auto":
+    data).  The partition must be the one of the fp32 arithmetic whatever the screen.  "q8-256": the 8-bit screen with
+    the subtrees below the wide levels finished by workgroups of 256 threads, as launches over many subtrees have it
+    (RSFK_TAIL_BLOCK; the few subtrees of a test otherwise get workgroups of 1024)."""
+    if screen == "q8-256":
+        monkeypatch.setenv("RSFK_TREE_SCREEN", "q8")
+        monkeypatch.setenv("RSFK_TAIL_BLOCK", "256")
+    elif screen != "auto":
         monkeypatch.setenv("RSFK_TREE_SCREEN", screen)
     if dist == "u":
         X = rng.random((N, D), dtype=np.float32)
