@@ -67,6 +67,16 @@ constexpr int kMaxShift = 13;
 constexpr size_t kMaxEntries = ((size_t)1 << 31) - 4096;
 constexpr int kRowsBlock = 512;             // threads of k_bin_rows
 
+// RSFK_JOIN_WG=0: the wavefront-per-q join also where the workgroup-per-q one applies.
+bool join_wg_on()
+{
+    static const bool on = [] {
+        const char* e = std::getenv("RSFK_JOIN_WG");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 // Bins of the reversed-graph builder for N points: false if N is too large for it.
 bool rev_bins(int N, int* shift, int* n_bins)
 {
@@ -410,6 +420,147 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join_short(Bf16Copy bf, 
     }
 }
 
+// The join with one workgroup (four wavefronts) per q, for rows of more than 32 neighbours.  k_explore_join loads the rows of a tile of R(q) again for every group of 32 neighbours and the rows of
+// the neighbours again for every tile of R(q): at K = 90 (three groups, three tiles) every row three times.  Here 96
+// points of R(q) and all neighbours of q pass through LDS together, 64 dimensions at a time (the next 64 are requested
+// while these are used), and the wavefronts share the pairs (tile of R(q), group of neighbours) among them, each
+// keeping the accumulators of its pairs: every row is read once per 96 points of R(q).  Bound and outputs are those
+// of k_explore_join.  NPW = pairs per wavefront (3: K <= 128, 6: K <= 256).
+constexpr int kJwP = 96;                    // points of R(q) worked on together (three tiles)
+constexpr int kJwRowBytes = 144;            // 64 bfloat16 values + 16 bytes: rows start in different banks
+
+template <bool BOUNDS, int NPW>
+__global__ __launch_bounds__(256) void k_explore_join_wg(Bf16Copy bf, int N, int K, const int* __restrict__ old_idx,
+                                                         const float2* __restrict__ norm_tau, const int* __restrict__ offs,
+                                                         const int* __restrict__ rev, uint32_t* __restrict__ pass,
+                                                         uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
+                                                         float kappa, float one_minus_gamma, uint32_t div_m, int div_s)
+{
+    constexpr int kPieces = (kJwP + (NPW == 3 ? 128 : 256)) * 8 / 256;      // 16-byte pieces a thread stages per step
+    extern __shared__ __align__(16) unsigned char lds_jw[];
+    unsigned char* rowsb = lds_jw;                                         // kJwP + KP rows of 144 bytes
+    int* cq = reinterpret_cast<int*>(rowsb + (size_t)(kJwP + KP) * kJwRowBytes);
+    float* cn = reinterpret_cast<float*>(cq + KP);
+    int* pid = reinterpret_cast<int*>(cn + KP);
+    int* pe = pid + kJwP;
+    float* pn = reinterpret_cast<float*>(pe + kJwP);
+    float* ptau = pn + kJwP;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 31, h = lane >> 5;
+    const int q = blockIdx.x;
+    const int r0 = offs[q], R = offs[q + 1] - r0;
+    if (R <= 0) return;                                                    // the whole workgroup leaves together
+    const int MW = KP >> 5;
+    const int nrows = kJwP + KP;
+    for (int k = tid; k < KP; k += 256) {
+        int c = k < K ? old_idx[(size_t)q * K + k] : -1;
+        if (c < 0 || c >= N) c = -1;
+        cq[k] = c;
+        cn[k] = c >= 0 ? norm_tau[c].x : 0.0f;
+    }
+    for (int pg = 0; pg < R; pg += kJwP) {
+        const int npg = min(kJwP, R - pg);
+        const int npairs = ((npg + 31) >> 5) * MW;
+        __syncthreads();                                                   // the previous group is done with the LDS
+        if (tid < kJwP) {
+            const int e = tid < npg ? rev[(size_t)r0 + pg + tid] : -1;
+            const int p = e >= 0 ? (int)(((uint64_t)div_m * (uint64_t)(uint32_t)e) >> div_s) : -1;
+            const float2 nt = p >= 0 ? norm_tau[p] : make_float2(0.0f, 0.0f);
+            pid[tid] = p;
+            pe[tid] = e;
+            pn[tid] = nt.x;
+            ptau[tid] = nt.y;
+        }
+        __syncthreads();
+        f32x16 acc[NPW];
+#pragma unroll
+        for (int i = 0; i < NPW; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) acc[i][j] = 0.0f;
+        // pieces this thread stages: piece i = tid + 256 j of the (row, 16-byte piece) grid
+        uint4 pre[kPieces];
+        auto request = [&](int c0) {
+#pragma unroll
+            for (int j = 0; j < kPieces; ++j) {
+                const int i = tid + 256 * j;
+                pre[j] = make_uint4(0u, 0u, 0u, 0u);
+                if (i < nrows * 8) {
+                    const int r = i >> 3, pc = i & 7;
+                    const int id = r < kJwP ? pid[r] : cq[r - kJwP];
+                    const int el = c0 * 16 + pc * 8;
+                    if (id >= 0 && el < ksteps * 16)
+                        pre[j] = *reinterpret_cast<const uint4*>(bf.rows + (size_t)id * (size_t)bpitch + el);
+                }
+            }
+        };
+        request(0);
+        for (int c0 = 0; c0 < ksteps; c0 += 4) {
+            if (c0 > 0) __syncthreads();                                   // the previous step's values have been used
+#pragma unroll
+            for (int j = 0; j < kPieces; ++j) {
+                const int i = tid + 256 * j;
+                if (i < nrows * 8) *reinterpret_cast<uint4*>(rowsb + (size_t)(i >> 3) * kJwRowBytes + (i & 7) * 16) = pre[j];
+            }
+            __syncthreads();
+            if (c0 + 4 < ksteps) request(c0 + 4);
+#pragma unroll
+            for (int i = 0; i < NPW; ++i) {
+                const int pair = wave + 4 * i;
+                if (pair < npairs) {
+                    const int pt = pair / MW, ct = pair - pt * MW;
+                    const unsigned char* ra = rowsb + (size_t)(pt * 32 + n) * kJwRowBytes + h * 16;
+                    const unsigned char* rb = rowsb + (size_t)(kJwP + ct * 32 + n) * kJwRowBytes + h * 16;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        if (c0 + u < ksteps) {
+                            const bf16x8 a = *reinterpret_cast<const bf16x8*>(ra + 32 * u);
+                            const bf16x8 b = *reinterpret_cast<const bf16x8*>(rb + 32 * u);
+                            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[i], 0, 0, 0);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);                         // one pair after the other (registers)
+            }
+        }
+        // Accumulator j of lane l: point 4 (l / 32) + 8 (j / 4) + j % 4 of the tile, column = neighbour l % 32 of the group.
+#pragma unroll
+        for (int i = 0; i < NPW; ++i) {
+            const int pair = wave + 4 * i;
+            if (pair < npairs) {
+                const int pt = pair / MW, ct = pair - pt * MW;
+                const int col = ct * 32 + n;
+                const int cid = cq[col];
+                const float cnv = cn[col];
+                uint32_t mine = 0;
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int m = pt * 32 + 4 * h + 8 * (j >> 2) + (j & 3);
+                    const float S = pn[m] + cnv;
+                    const float dt = __builtin_fmaf(-2.0f, acc[i][j], S);
+                    const float e1 = kappa * S;
+                    const float dhi = fmaxf(dt + e1, 0.0f);
+                    const float Q = 2.0001f * S;
+                    const float ebf = 1.01f * (2.0f * kU * __builtin_sqrtf(dhi * Q) + kU * kU * Q);
+                    const float lower = (dt - e1 - ebf) * one_minus_gamma - 1e-30f;
+                    const bool skip = lower > ptau[m];            // false if anything is NaN; a tie at the last slot may still enter
+                    const bool marked = cid >= 0 && !skip;
+                    const uint64_t bm = ballot64(marked);
+                    if (BOUNDS && marked && m < npg) {
+                        // a bound below zero (or NaN) says nothing: 0.  Dropping the low half of a positive float rounds down.
+                        const uint32_t lb = lower > 0.0f ? __float_as_uint(lower) >> 16 : 0u;
+                        bounds[(size_t)pe[m] * (size_t)KP + col] = (uint16_t)lb;
+                    }
+                    const int m_lo = 8 * (j >> 2) + (j & 3);
+                    if (lane == m_lo) mine = (uint32_t)bm;
+                    if (lane == m_lo + 4) mine = (uint32_t)(bm >> 32);
+                    if ((j & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // four at a time (registers)
+                }
+                if (lane < 32 && pt * 32 + lane < npg) pass[(size_t)pe[pt * 32 + lane] * MW + ct] = mine;
+            }
+        }
+    }
+}
+
 }  // namespace
 
 // The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has about 2^31 or more entries or N is beyond what the
@@ -522,6 +673,23 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
         else if (ksteps <= 4) RSFK_JOIN_SHORT(4);
         else RSFK_JOIN_SHORT(8);
 #undef RSFK_JOIN_SHORT
+    } else if (KP > 32 && join_wg_on()) {
+        // one workgroup per q: every row once per 96 points of R(q).  (Rows of at most 32 neighbours have one pair per
+        // tile of R(q): too little for four wavefronts; 1M x 256, K = 32: 8.1 ms against 12.6.)
+        const size_t lds_wg = (size_t)(kJwP + KP) * kJwRowBytes + (size_t)KP * 8 + (size_t)kJwP * 16;
+#define RSFK_JOIN_WG(BV, NV)                                                                                                \
+        do {                                                                                                               \
+            RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_join_wg<BV, NV>),                         \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_wg));                       \
+            hipLaunchKernelGGL((k_explore_join_wg<BV, NV>), dim3((unsigned)N), dim3(256), lds_wg, stream, bf, N, K, old_idx,  \
+                               w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps, kappa,           \
+                               one_minus_gamma, w->div_m, w->div_s);                                                       \
+        } while (0)
+        if (w->bounds && KP <= 128) RSFK_JOIN_WG(true, 3);
+        else if (w->bounds) RSFK_JOIN_WG(true, 6);
+        else if (KP <= 128) RSFK_JOIN_WG(false, 3);
+        else RSFK_JOIN_WG(false, 6);
+#undef RSFK_JOIN_WG
     } else if (w->bounds)
         hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
