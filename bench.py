@@ -215,6 +215,28 @@ CONFIGS = {
 FP32_PEAK_TFLOPS = 157.3
 
 
+def gather_probe(dX, N, D, reps=5):
+    """Rate of rsfk_probe_gather_device over all rows of dX in a random order (HIP events on the launching stream)."""
+    import torch
+    from gpu_rsfk import capi
+    ids = torch.randperm(N, device=dX.device, dtype=torch.int64).to(torch.int32)
+    sums = torch.empty(4096, dtype=torch.float32, device=dX.device)
+    stream = torch.cuda.current_stream()
+    times = []
+    for rep in range(reps + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        capi._check(capi.lib().rsfk_probe_gather_device(dX.data_ptr(), N, D, ids.data_ptr(), N, sums.data_ptr(),
+                                                       stream.cuda_stream))
+        e1.record(stream)
+        e1.synchronize()
+        if rep > 0:
+            times.append(e0.elapsed_time(e1) * 1e-3)
+    t = float(np.median(times))
+    return {"row_bytes": 4 * D, "rows": N, "seconds": round(t, 7), "GB/s": round(4.0 * D * N / t / 1e9, 1),
+            "note": "rows of the point matrix read once in a random order and nothing else"}
+
+
 def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
     """Roofline object of the bucket K-NN step of one tree (one step of the forest loop = one tree's launches).
 
@@ -354,6 +376,16 @@ def main():
     expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
     leaves = fls[0].data["Total Leaves"] if fls and T > 0 else []
     roofline = bucket_roofline(N, D, K, T, mn, mx, knn_s, leaves)
+    # what the device delivers when scattered rows of 4 D bytes are only read: every row of the matrix once, in a random
+    # order, by rsfk_probe_gather_device (one wavefront per row, nothing computed); the bucket kernels gather the same
+    # rows in the order of a tree's permutation and cannot be faster than this on their N 4 D bytes
+    try:
+        roofline["gather_probe"] = gather_probe(dX, N, D)
+        if roofline.get("bound") == "hbm" and roofline["gather_probe"]["GB/s"] > 0:
+            # the same achieved rate against what scattered rows of this size reach on the device
+            roofline["frac_of_gather_rate"] = round(roofline["achieved"] / roofline["gather_probe"]["GB/s"], 4)
+    except Exception as e:           # the probe is an aid: the line is valid without it
+        roofline["gather_probe"] = {"error": str(e)}
 
     # CPU baseline: the oracle (a port of the reference algorithm, OpenMP) on the same workload -- whole with
     # --cpu-full, else on its first rows, as many as about 30 s of CPU time cover (the rate per point of a smaller

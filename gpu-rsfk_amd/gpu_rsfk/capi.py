@@ -31,6 +31,7 @@ SYMBOLS = {
     "rsfk_explore_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _f32, _ci]),
     "rsfk_last_error": (ctypes.c_char_p, []),
     "rsfk_device_count": (_ci, []),
+    "rsfk_probe_gather_device": (_ci, [_vp, _ci, _ci, _vp, ctypes.c_longlong, _vp, _vp]),
     "rsfk_release_workspace": (None, []),
 }
 

@@ -176,6 +176,14 @@ void rsfk_release_workspace(void);
 /* number of HIP devices visible to the library (0 when there is none) */
 int rsfk_device_count(void);
 
+/* Measurement aid, no counterpart in the reference: reads the rows ids[0..n_ids) of the device matrix points
+ * (N x D floats) the way the bucket kernels gather them -- one wavefront per row, 16-byte pieces -- and adds them
+ * up into sums (one float per workgroup launched, at least 4096 floats).  bench.py times it to report the rate at
+ * which this device delivers scattered rows of 4 D bytes, next to the rate of the bucket K-NN kernel.  stream: a
+ * hipStream_t or null.  Returns 0, or nonzero with the reason in rsfk_last_error(). */
+int rsfk_probe_gather_device(const float* d_points, int N, int D, const int* d_ids, long long n_ids, float* d_sums,
+                             void* stream);
+
 #ifdef __cplusplus
 }
 #endif
