@@ -551,7 +551,6 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
                                                     int2* __restrict__ child)
 {
     __shared__ int red[2][kBlock / 64];
-    __shared__ int wcnt[kBlock / 64];
     const int c = blockIdx.x;
     const int ni = chunk2node[c];
     const TreeNode nd = nodes[ni];
@@ -581,24 +580,40 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
     const int pos0 = nd.start + k * P.chunk;
     const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
     int lbase = before;                                   // lefts of the node before the current round
-    for (int r0 = pos0; r0 < pos1; r0 += kBlock) {
-        const int pos = r0 + tid;
-        const bool valid = pos < pos1;
-        const int v = valid ? src[pos] : 0;
-        const bool right = v < 0;
-        const bool isl = valid && !right;
-        const uint64_t m = ballot64(isl);
-        if (lane == 0) wcnt[wave] = __popcll(m);
-        __syncthreads();
-        int woff = 0, tot = 0;
+    // rounds of four entries per thread (entry u of a thread at r0 + u kBlock + tid: loads and stores stay coalesced,
+    // four loads in flight, one exchange of the wavefronts' counts per round)
+    constexpr int kPer = 4;
+    __shared__ int wcnt4[kPer][kBlock / 64];
+    for (int r0 = pos0; r0 < pos1; r0 += kPer * kBlock) {
+        int v[kPer];
+        uint64_t m[kPer];
 #pragma unroll
-        for (int w = 0; w < kBlock / 64; ++w) { const int x = wcnt[w]; if (w < wave) woff += x; tot += x; }
-        const int lrank = lbase + woff + mask_prefix(m);  // lefts of the node before this position
-        if (valid) {
-            const int dest = right ? nd.start + all + (pos - nd.start) - lrank : nd.start + lrank;
-            dst[dest] = v & kIdMask;
+        for (int u = 0; u < kPer; ++u) {
+            const int pos = r0 + u * kBlock + tid;
+            v[u] = pos < pos1 ? src[pos] : -1;            // (beyond the chunk: counts as a right one, is not stored)
         }
-        lbase += tot;
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            m[u] = ballot64(v[u] >= 0);
+            if (lane == 0) wcnt4[u][wave] = __popcll(m[u]);
+        }
+        __syncthreads();
+        int run = lbase;                                  // lefts before entry (u, wavefront 0)
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            int woff = 0, tot = 0;
+#pragma unroll
+            for (int w = 0; w < kBlock / 64; ++w) { const int x = wcnt4[u][w]; if (w < wave) woff += x; tot += x; }
+            const int pos = r0 + u * kBlock + tid;
+            if (pos < pos1) {
+                const int lrank = run + woff + mask_prefix(m[u]);      // lefts of the node before this position
+                const bool right = v[u] < 0;
+                const int dest = right ? nd.start + all + (pos - nd.start) - lrank : nd.start + lrank;
+                dst[dest] = v[u] & kIdMask;
+            }
+            run += tot;
+        }
+        lbase = run;
         __syncthreads();
     }
     if (k == 0 && tid == 0) {
