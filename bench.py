@@ -237,6 +237,37 @@ def gather_probe(dX, N, D, reps=5):
             "note": "rows of the point matrix read once in a random order and nothing else"}
 
 
+PROFILE_FILES = {"c2": "knng_build_c2_uniform_1M_d100_k32.md", "c3": "knng_build_c3_gmm64_1M_d256_k32.md",
+                 "c4": "knng_build_c4_sparse_70k_d784_k90.md", "c5": "knng_build_c5_normal_10M_d32_k32.md"}
+FETCH_SCALE = 1.92          # FETCH_SIZE reads 0.52 of the bytes a copy kernel of known size loads; WRITE_SIZE matches
+
+
+def profiled_traffic(config, steps_profiled=2):
+    """HBM bytes per tree of the bucket K-NN kernels from the tracked rocprofv3 summary of this workload
+    (profiles/: FETCH_SIZE and WRITE_SIZE in KiB per launch, launches of two builds), or None.  The counters cannot be
+    collected inside this run; the summary is of the same command (bench.py --config <c>) and says how it was made."""
+    fn = PROFILE_FILES.get(config)
+    path = os.path.join(ROOT, "profiles", fn) if fn else None
+    if not path or not os.path.exists(path):
+        return None
+    launches, kib = {}, {}
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) == 7 and cells[0].startswith("k_bucket_knn"):
+            try:
+                if "." in cells[2]:                       # trace table: launches, total ms, ...
+                    launches[cells[0]] = int(cells[1])
+                else:                                     # counter table: FETCH KiB, WRITE KiB per launch
+                    kib[cells[0]] = (float(cells[1]), float(cells[2]))
+            except ValueError:
+                pass
+    total = 0.0
+    for k, n in launches.items():
+        if k in kib:
+            total += n * (kib[k][0] * FETCH_SCALE + kib[k][1]) * 1024.0
+    return total / steps_profiled if total > 0 else None
+
+
 def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
     """Roofline object of the bucket K-NN step of one tree (one step of the forest loop = one tree's launches).
 
@@ -376,6 +407,14 @@ def main():
     expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
     leaves = fls[0].data["Total Leaves"] if fls and T > 0 else []
     roofline = bucket_roofline(N, D, K, T, mn, mx, knn_s, leaves)
+    cfg_name = next((name for name, c in CONFIGS.items()
+                     if (args.workload, N, D, K, T, mn, mx, args.explore) == c), None)
+    per_build = profiled_traffic(cfg_name) if T > 0 and cfg_name else None
+    if per_build:
+        roofline["traffic"] = round(per_build / T)
+        roofline["note"] = ("traffic: HBM bytes per tree of the bucket K-NN kernels from the tracked rocprofv3 summary of this "
+                            "command (profiles/%s: FETCH_SIZE x %.2f + WRITE_SIZE, all bucket kernels of a build / trees)"
+                            % (PROFILE_FILES[cfg_name], FETCH_SCALE))
     # what the device delivers when scattered rows of 4 D bytes are only read: every row of the matrix once, in a random
     # order, by rsfk_probe_gather_device (one wavefront per row, nothing computed); the bucket kernels gather the same
     # rows in the order of a tree's permutation and cannot be faster than this on their N 4 D bytes
