@@ -36,6 +36,61 @@ constexpr int kMaxChunk = 64;               // dimensions staged at once
 // CAP = largest bucket, THREADS = workgroup size, SPACING = LDS rows between members 2t and 2t+1: the 2x2 block
 // (a, b) reads rows a, a + SPACING, b, b + SPACING -- consecutive a (consecutive threads) give conflict-free 16-byte
 // reads (the pitch is an odd number of 16-byte units).
+// Does the row in the registers of the wavefront (slot k in lane k) hold nothing but, possibly, the point itself in
+// slot 0?  Empty slots are (-1, +inf).
+__device__ __forceinline__ bool fresh_row(int ri, float rd, int self_id, int K)
+{
+    const int lane = lane_id();
+    const bool empty = ri == -1 && rd == INFINITY;
+    const bool fine = lane >= K || empty || (lane == 0 && ri == self_id);
+    return ballot64(!fine) == 0;
+}
+
+// dv[v] of lane l: distance of candidate l + 64 v of a fresh row (the point itself included, with the distance its row
+// holds), +inf where there is none; n candidates in all.  When no two finite distances are equal, the place of a
+// candidate in the row ordered by (distance, index) is the number of finite distances below its own: dv[v] is
+// replaced by that number (as an integer; -1 for a candidate that is not finite) and the result is true.  With equal
+// distances the result is false and dv is unchanged.
+template <int CL>
+__device__ __forceinline__ bool place_by_rank(float (&dv)[CL], int n)
+{
+    int rank[CL];
+#pragma unroll
+    for (int v = 0; v < CL; ++v) rank[v] = 0;
+#pragma unroll
+    for (int u = 0; u < CL; ++u) {
+        const int nu = min(kWave, n - kWave * u);
+        // four at a time (lanes past the last candidate hold +inf and count for nothing)
+        for (int j = 0; j < nu; j += 4) {
+            float dj[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) dj[x] = read_lane_f(dv[u], j + x);
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int v = 0; v < CL; ++v) rank[v] += dj[x] < dv[v] ? 1 : 0;
+        }
+    }
+    // equal distances give equal numbers: all numbers of the finite candidates must differ
+    uint32_t seen[4] = {0u, 0u, 0u, 0u};                 // bit r of the 128-bit set: some candidate has number r
+    int n_finite = 0;
+#pragma unroll
+    for (int v = 0; v < CL; ++v) {
+        const bool fin = dv[v] < INFINITY;
+        n_finite += __popcll(ballot64(fin));
+#pragma unroll
+        for (int w = 0; w < 2 * CL; ++w) seen[w] |= (fin && (rank[v] >> 5) == w) ? (1u << (rank[v] & 31)) : 0u;
+        if (!fin) rank[v] = -1;
+    }
+    int n_seen = 0;
+#pragma unroll
+    for (int w = 0; w < 2 * CL; ++w) n_seen += __popc(wave_or_u32(seen[w]));
+    if (n_seen != n_finite) return false;
+#pragma unroll
+    for (int v = 0; v < CL; ++v) dv[v] = __int_as_float(rank[v]);
+    return true;
+}
+
 template <int CAP, int THREADS, int SPACING>
 struct SmallCfg {
     static constexpr int kWaves = THREADS / 64;
@@ -200,13 +255,8 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
     const int my_id2 = (kCap > 64 && 64 + lane < kCap) ? lids[64 + lane] : -1;      // second round of candidates
     // bit u: member wave + kWaves u has a candidate
     const int fm = wave + kWaves * lane;
-    uint32_t active = (uint32_t)ballot64(lane < 32 && fm < kCap && flag[fm < kCap ? fm : 0] != 0);
-    auto next_member = [&]() {
-        if (active == 0) return -1;
-        const int u = __ffs(active) - 1;
-        active &= active - 1;
-        return wave + kWaves * u;
-    };
+    const bool has_cand = lane < 32 && fm < kCap && flag[fm < kCap ? fm : 0] != 0;
+    uint32_t active = (uint32_t)ballot64(has_cand);
     auto load_row = [&](int i, int& ri, float& rd) {
         ri = -2;
         rd = INFINITY;
@@ -216,47 +266,90 @@ __global__ __launch_bounds__(THREADS, 4) void k_bucket_knn_small(const float* __
             rd = knn_dist[at];
         }
     };
-    constexpr int kAhead = 4;
-    int cur_i[kAhead], cur_ri[kAhead], nxt_i[kAhead], nxt_ri[kAhead];
-    float cur_rd[kAhead], nxt_rd[kAhead];
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
-        cur_i[u] = next_member();
-        load_row(cur_i[u], cur_ri[u], cur_rd[u]);
-    }
-    while (cur_i[0] >= 0) {
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            nxt_i[u] = next_member();
-            load_row(nxt_i[u], nxt_ri[u], nxt_rd[u]);
-        }
+    // handle(i, ri, rd) for the members of the set, in ascending order
+    auto walk = [&](uint32_t members, auto&& handle) {
+        auto next_member = [&]() {
+            if (members == 0) return -1;
+            const int u = __ffs(members) - 1;
+            members &= members - 1;
+            return wave + kWaves * u;
+        };
+        constexpr int kAhead = 4;
+        int cur_i[kAhead], cur_ri[kAhead], nxt_i[kAhead], nxt_ri[kAhead];
+        float cur_rd[kAhead], nxt_rd[kAhead];
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) {
-            const int i = cur_i[u];
-            if (i < 0) break;
-            const float d = dist[i * kDistPitch + lane];
-            KnnRow<1> row;
-            row.idx[0] = cur_ri[u];
-            row.dist[0] = cur_rd[u];
-            row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
-            if (kCap > 64) {
-                const int j2 = 64 + lane;
-                const float d2 = j2 < s ? dist[i * kDistPitch + j2] : INFINITY;
-                const bool okv[2] = {lane < s && lane != i, j2 < s && j2 != i};
-                const int cv[2] = {my_id, my_id2};
-                const float dv[2] = {d, d2};
-                row.template merge<2>(okv, cv, dv);
-            } else {
-                row.merge(lane < s && lane != i, my_id, d);
-            }
-            if (row.changed) {
-                const size_t at = (size_t)lids[i] * (size_t)K;
-                row.store(knn_idx + at, knn_dist + at);
-            }
+            cur_i[u] = next_member();
+            load_row(cur_i[u], cur_ri[u], cur_rd[u]);
         }
+        while (cur_i[0] >= 0) {
 #pragma unroll
-        for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }
+            for (int u = 0; u < kAhead; ++u) {
+                nxt_i[u] = next_member();
+                load_row(nxt_i[u], nxt_ri[u], nxt_rd[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) {
+                if (cur_i[u] < 0) break;
+                handle(cur_i[u], cur_ri[u], cur_rd[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }
+        }
+    };
+
+    // Rows that are not full (last slot at +inf; every row in the first tree of a build) may hold nothing but the
+    // point itself.  Such a row needs no insertions: the place of a candidate is the number of candidates below it.
+    // Rows done that way leave the set; the others (and rows with two candidates at the same distance) are left to
+    // the insertions below.
+    const uint32_t maybe_fresh = (uint32_t)ballot64(has_cand && tau[fm < kCap ? fm : 0] == INFINITY);
+    if (maybe_fresh != 0) {
+        walk(maybe_fresh, [&](int i, int ri, float rd) {
+            if (!fresh_row(ri, rd, lids[i], K)) return;
+            const float self_d = read_lane_i(ri, 0) >= 0 ? read_lane_f(rd, 0) : INFINITY;
+            constexpr int CL = kCap > 64 ? 2 : 1;
+            const int j2 = 64 + lane;
+            float cd[CL], place[CL];
+            cd[0] = lane == i ? self_d : (lane < s ? dist[i * kDistPitch + lane] : INFINITY);
+            if (CL > 1) cd[CL - 1] = j2 == i ? self_d : (j2 < s ? dist[i * kDistPitch + j2] : INFINITY);
+#pragma unroll
+            for (int v = 0; v < CL; ++v) place[v] = cd[v];
+            if (!place_by_rank<CL>(place, s)) return;
+            const size_t at = (size_t)lids[i] * (size_t)K;
+            const int cv[2] = {my_id, my_id2};
+#pragma unroll
+            for (int v = 0; v < CL; ++v) {
+                const int slot = __float_as_int(place[v]);
+                if (slot >= 0 && slot < K) {
+                    knn_idx[at + slot] = cv[v];
+                    knn_dist[at + slot] = cd[v];
+                }
+            }
+            active &= ~(1u << ((i - wave) / kWaves));
+        });
     }
+
+    walk(active, [&](int i, int ri, float rd) {
+        const float d = dist[i * kDistPitch + lane];
+        KnnRow<1> row;
+        row.idx[0] = ri;
+        row.dist[0] = rd;
+        row.init_from_regs(K);                   // rows that arrive unsorted are rebuilt here
+        if (kCap > 64) {
+            const int j2 = 64 + lane;
+            const float d2 = j2 < s ? dist[i * kDistPitch + j2] : INFINITY;
+            const bool okv[2] = {lane < s && lane != i, j2 < s && j2 != i};
+            const int cv[2] = {my_id, my_id2};
+            const float dv[2] = {d, d2};
+            row.template merge<2>(okv, cv, dv);
+        } else {
+            row.merge(lane < s && lane != i, my_id, d);
+        }
+        if (row.changed) {
+            const size_t at = (size_t)lids[i] * (size_t)K;
+            row.store(knn_idx + at, knn_dist + at);
+        }
+    });
 }
 
 }  // namespace

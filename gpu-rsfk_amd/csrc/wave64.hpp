@@ -111,6 +111,17 @@ __device__ __forceinline__ int wave_sum_i(int v)
     return read_lane_i(v, 0) + read_lane_i(v, 16) + read_lane_i(v, 32) + read_lane_i(v, 48);
 }
 
+// bitwise or over all 64 lanes, returned in every lane (wave-uniform value)
+__device__ __forceinline__ uint32_t wave_or_u32(uint32_t x)
+{
+    int v = (int)x;
+    v |= dpp_i<kDppXor1>(v);
+    v |= dpp_i<kDppXor2>(v);
+    v |= dpp_i<kDppHalfMirror>(v);
+    v |= dpp_i<kDppMirror>(v);
+    return (uint32_t)(read_lane_i(v, 0) | read_lane_i(v, 16) | read_lane_i(v, 32) | read_lane_i(v, 48));
+}
+
 // exclusive prefix sum over the lanes of the wavefront
 __device__ __forceinline__ int wave_excl_scan_i(int v)
 {

@@ -142,6 +142,47 @@ def test_bucket_knn_resident_rows_matches_oracle(gpu, orc, rng, N, D, K, MIN, MA
         assert rows_have_no_duplicates(gi)
 
 
+@pytest.mark.parametrize("K", [20, 64])
+@pytest.mark.parametrize("data", ["continuous", "grid", "mixed"])
+@pytest.mark.parametrize("start", ["self", "empty", "self_far", "other"])
+def test_bucket_knn_rows_that_start_new(gpu, orc, rng, start, data, K):
+    """A row that holds at most the point itself is filled by counting, for every candidate, the candidates below it;
+    two candidates at the same distance send the row to the insertions instead.  Rows start with the point itself,
+    empty, with the point itself at a distance that is not 0, or with one other point (then they are not new); the points
+    are continuous (no equal distances), on a small grid (nothing but equal distances and duplicates) or both.  Buckets
+    of up to 72 points, so that both shapes of the small-bucket kernel run; with K = 64 the first tree does not fill
+    the rows and the second finds rows that are neither new nor full."""
+    N, D = 3000, 6
+    X = rng.random((N, D), dtype=np.float32)
+    if data == "grid":
+        X = rng.integers(0, 3, (N, D)).astype(np.float32)
+    elif data == "mixed":
+        some = rng.random(N) < 0.05
+        X[some] = rng.integers(0, 2, (int(some.sum()), D)).astype(np.float32)
+    oi = np.full((N, K), -1, np.int32)
+    od = np.full((N, K), np.inf, np.float32)
+    if start in ("self", "self_far"):
+        oi[:, 0] = np.arange(N)
+        od[:, 0] = 0.0 if start == "self" else 0.3
+    elif start == "other":
+        # the point's partner in the pairs (0, 1), (2, 3), ... at its distance (a row must not hold a wrong distance:
+        # an index could then leave the row and come back with another one, and the result would depend on the order)
+        ti, td = orc.init_lists(N, 2)
+        orc.bucket_knn(X, 2, np.arange(N, dtype=np.int32), np.full(N // 2, 2, np.int32), ti, td,
+                       starts=np.arange(0, N, 2, dtype=np.int32))
+        first_is_self = ti[:, 0] == np.arange(N)
+        oi[:, 0] = np.where(first_is_self, ti[:, 1], ti[:, 0])
+        od[:, 0] = np.where(first_is_self, td[:, 1], td[:, 0])
+    gi, gd = oi.copy(), od.copy()
+    for seed in (3, 4):
+        _say("bucket_knn new rows", start, data, K, seed)
+        perm, ls, lz, _ = orc.build_tree(X, 21, 72, 5000, seed)
+        orc.bucket_knn(X, K, perm, lz, oi, od, starts=ls)
+        gpu.bucket_knn(X, K, perm, lz, gi, gd, starts=ls)
+        assert_knn_equal(gi, gd, oi, od)
+        assert rows_have_no_duplicates(gi)
+
+
 def test_bucket_knn_single_bucket_is_exact_knn(gpu, rng):
     """One bucket holding every point: the kernel must return exact K-NN."""
     for N, D, K in [(300, 8, 16), (700, 20, 32)]:
