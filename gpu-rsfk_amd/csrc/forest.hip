@@ -61,21 +61,19 @@ struct DevBuf {
     void* p = nullptr;
     ~DevBuf() { ws_free(p); }
 };
-// second stream (default priority) and the two events that order it against the caller's stream
+// second stream (default priority) and the event that tells the caller's stream when its work is done
 struct SideStream {
     hipStream_t side = nullptr;
-    hipEvent_t start = nullptr, big = nullptr;
+    hipEvent_t big = nullptr;
     int open()
     {
         RSFK_HIP(hipStreamCreateWithFlags(&side, hipStreamNonBlocking));
-        RSFK_HIP(hipEventCreateWithFlags(&start, hipEventDisableTiming));
         RSFK_HIP(hipEventCreateWithFlags(&big, hipEventDisableTiming));
         return 0;
     }
     ~SideStream()
     {
         if (side) { (void)hipStreamSynchronize(side); (void)hipStreamDestroy(side); }
-        if (start) (void)hipEventDestroy(start);
         if (big) (void)hipEventDestroy(big);
     }
 };
@@ -91,23 +89,21 @@ struct Q8Guard {
     Q8Copy c;
     ~Q8Guard() { q8_copy_free(&c); }
 };
-// start / stop events of one tree's K-NN update; released when the owner goes out of scope, on every path
-struct EventPair {
-    hipEvent_t a = nullptr, b = nullptr;
-    EventPair() = default;
-    EventPair(const EventPair&) = delete;
-    EventPair& operator=(const EventPair&) = delete;
-    EventPair(EventPair&& o) noexcept : a(o.a), b(o.b) { o.a = nullptr; o.b = nullptr; }
+// An event with a time stamp; released when the owner goes out of scope, on every path.
+struct TimedEvent {
+    hipEvent_t e = nullptr;
+    TimedEvent() = default;
+    TimedEvent(const TimedEvent&) = delete;
+    TimedEvent& operator=(const TimedEvent&) = delete;
+    TimedEvent(TimedEvent&& o) noexcept : e(o.e) { o.e = nullptr; }
     int create()
     {
-        RSFK_HIP(hipEventCreate(&a));
-        RSFK_HIP(hipEventCreate(&b));
+        RSFK_HIP(hipEventCreate(&e));
         return 0;
     }
-    ~EventPair()
+    ~TimedEvent()
     {
-        if (a) (void)hipEventDestroy(a);
-        if (b) (void)hipEventDestroy(b);
+        if (e) (void)hipEventDestroy(e);
     }
 };
 
@@ -164,7 +160,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         WsGuard ws;
         if (tree_ws_alloc(&ws.w, N, D, MIN, B)) return 1;
         std::vector<int> stats((size_t)5 * B);
-        std::vector<EventPair> ev((size_t)B);
+        // ev[j] is recorded where the K-NN update of tree j of a batch begins (both parts of tree j - 1 are done), ev[nb]
+        // where the last one ends: one event per tree between the launches, not two
+        std::vector<TimedEvent> ev((size_t)B + 1);
         for (auto& e : ev)
             if (e.create()) return 1;
         const int gram_from = bucket_gram_from();
@@ -186,12 +184,8 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 const int n_big = stats[5 * j + 4], n_small = stats[5 * j] - n_big;
                 const bool split = sync.side != nullptr && n_big > 0 && n_small > 0;
                 if (big_pending) (void)hipStreamWaitEvent(stream, sync.big, 0);
-                if (j > 0) (void)hipEventRecord(ev[j - 1].b, stream);          // both parts of the previous tree are done
-                (void)hipEventRecord(ev[j].a, stream);
-                if (split) {
-                    (void)hipEventRecord(sync.start, stream);                    // everything before this tree
-                    (void)hipStreamWaitEvent(sync.side, sync.start, 0);
-                }
+                (void)hipEventRecord(ev[j].e, stream);                         // both parts of the previous tree are done
+                if (split) (void)hipStreamWaitEvent(sync.side, ev[j].e, 0);      // everything before this tree
                 const bool gram = t0 + j >= gram_from;
                 rc = launch_bucket_knn_tree(d_points, t0 + j >= screen_from, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
@@ -205,12 +199,12 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 big_pending = split;
             }
             if (big_pending) (void)hipStreamWaitEvent(stream, sync.big, 0);
-            if (nb > 0) (void)hipEventRecord(ev[nb - 1].b, stream);
+            (void)hipEventRecord(ev[nb].e, stream);
             if (rc) break;
             RSFK_HIP(hipStreamSynchronize(stream));
             for (int j = 0; j < nb; ++j) {
                 float ms = 0.0f;
-                (void)hipEventElapsedTime(&ms, ev[j].a, ev[j].b);
+                (void)hipEventElapsedTime(&ms, ev[j].e, ev[j + 1].e);
                 const int t = t0 + j;
                 if (log_forest) {
                     log_forest[(size_t)0 * n_trees + t] = (float)stats[5 * j + 1];   // Tree Depth
@@ -292,7 +286,7 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
         DevBuf planes;
         if (ws_alloc(&planes.p, sizeof(float) * (size_t)rec_cap * (size_t)ann_plane_pitch(D))) return 1;
         std::vector<int> stats((size_t)5 * B);
-        std::vector<EventPair> ev((size_t)B);
+        std::vector<TimedEvent> ev((size_t)B + 1);          // ev[j]: the search in tree j of a batch begins, ev[nb]: the last ends
         for (auto& e : ev)
             if (e.create()) return 1;
         int rc = 0;
@@ -304,17 +298,17 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
             if (rc) break;
             const double tt = now_s() - tt0;
             for (int j = 0; j < nb && rc == 0; ++j) {
-                (void)hipEventRecord(ev[j].a, stream);
+                (void)hipEventRecord(ev[j].e, stream);
                 rc = launch_ann_tree(d_points, d_queries, NQ, D, K, tree_ws_perm(ws.w, j), tree_ws_recs(ws.w, j),
                                      tree_ws_n_rec(ws.w, j), rec_cap, stats[5 * j + 0], static_cast<int*>(aws.p),
                                      static_cast<float*>(planes.p), d_qidx, d_qdist, stream);
-                (void)hipEventRecord(ev[j].b, stream);
             }
+            (void)hipEventRecord(ev[nb].e, stream);
             if (rc) break;
             RSFK_HIP(hipStreamSynchronize(stream));
             for (int j = 0; j < nb; ++j) {
                 float ms = 0.0f;
-                (void)hipEventElapsedTime(&ms, ev[j].a, ev[j].b);
+                (void)hipEventElapsedTime(&ms, ev[j].e, ev[j + 1].e);
                 const int t = tb0 + j;
                 if (log_forest) {
                     log_forest[(size_t)0 * n_trees + t] = (float)stats[5 * j + 1];   // Tree Depth

@@ -49,7 +49,19 @@ struct LevelCounters {
     int n_tail;        // tail tasks appended so far
     int n_chunks;      // chunks of the current level (written by the scan kernel)
     int overflow;      // set when a queue capacity is exceeded
+    // time spent in the three steps of the wide levels (hyperplanes, side tests, scatter), in ticks of the device's
+    // constant-rate clock: the first thread of a kernel that opens a step closes the one before it
+    long long last_tick;
+    long long phase_ticks[3];
 };
+
+// ended: the step that ends where the calling kernel begins (-1: none, the clock is only started)
+__device__ __forceinline__ void phase_tick(LevelCounters* ctr, int ended)
+{
+    const long long now = (long long)wall_clock64();
+    if (ended >= 0 && ctr->last_tick != 0) ctr->phase_ticks[ended] += now - ctr->last_tick;
+    ctr->last_tick = now;
+}
 
 // ---------------------------------------------------------------------------
 // helpers
@@ -401,7 +413,10 @@ __global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict
     __shared__ int carry_s;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n_nodes = min(ctr->n_next, node_cap);       // nodes of the level, left by the previous level's scatter
-    if (tid == 0) carry_s = 0;
+    if (tid == 0) {
+        carry_s = 0;
+        phase_tick(ctr, 2);
+    }
     __syncthreads();
     for (int base = 0; base < n_nodes; base += 1024) {
         const int i = base + tid;
@@ -426,9 +441,15 @@ __global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict
     if (tid == 0) { chunk_base[n_nodes] = carry_s; ctr->n_chunks = carry_s; }
 }
 
-__global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, int n_chunks, int* __restrict__ chunk2node)
+// (also empties the queue of the level being produced, which the scatter kernel of this level fills)
+__global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, int n_chunks, int* __restrict__ chunk2node,
+                              LevelCounters* ctr)
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c == 0) {
+        phase_tick(ctr, 0);
+        ctr->n_next = 0;
+    }
     if (c >= n_chunks) return;
     int lo = 0, hi = n_nodes - 1;          // last node with chunk_base <= c
     while (lo < hi) {
@@ -444,10 +465,11 @@ __global__ void k_fill_chunks(const int* __restrict__ chunk_base, int n_nodes, i
 __global__ __launch_bounds__(256) void k_level_planes(const float* __restrict__ points, TreeParams P,
                                                       const int* __restrict__ perm0, const int* __restrict__ perm1,
                                                       const TreeNode* __restrict__ nodes, int n_nodes,
-                                                      float* __restrict__ table)
+                                                      float* __restrict__ table, LevelCounters* ctr)
 {
     extern __shared__ __align__(16) float lds_p[];          // per wavefront: 4 + nvec_len(D) floats
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (blockIdx.x == 0 && threadIdx.x == 0) phase_tick(ctr, -1);
     const int ni = blockIdx.x * (blockDim.x >> 6) + wave;
     if (ni >= n_nodes) return;
     const int rec = 4 + nvec_len(P.D);
@@ -552,6 +574,7 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
 {
     __shared__ int red[2][kBlock / 64];
     const int c = blockIdx.x;
+    if (c == 0 && threadIdx.x == 0) phase_tick(ctr, 1);
     const int ni = chunk2node[c];
     const TreeNode nd = nodes[ni];
     const int first = chunk_base[ni];
@@ -965,7 +988,7 @@ struct TreeBatchWorkspace {
     int* n_rec = nullptr;                // B
     int rec_cap = 0;
     // events around the kernels of a wide level (hyperplanes | side test | scatter) and around the tail kernel
-    hipEvent_t ev[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    hipEvent_t ev[2] = {nullptr, nullptr};          // around the tail kernel
     float phase_s[4] = {0.f, 0.f, 0.f, 0.f};   // of the last batch: side tests, hyperplanes, scatter, tail kernel
     // side tests of the first levels taken point by point (tree_sweep.hpp); allocated when D allows it
     int pm_ks = 0;                       // 32-dimension steps of a row as matrix-core operands (1, 2, 4, 8), 0 = not available
@@ -1135,15 +1158,6 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         }
     }
     for (float& v : w->phase_s) v = 0.0f;
-    bool level_timed = false;                 // ev[0..3] bracket the three kernels of the previous level
-    auto add_level_times = [&]() {
-        if (!level_timed) return;
-        float ms = 0.0f;
-        if (hipEventElapsedTime(&ms, w->ev[0], w->ev[1]) == hipSuccess) w->phase_s[1] += ms * 1e-3f;
-        if (hipEventElapsedTime(&ms, w->ev[1], w->ev[2]) == hipSuccess) w->phase_s[0] += ms * 1e-3f;
-        if (hipEventElapsedTime(&ms, w->ev[2], w->ev[3]) == hipSuccess) w->phase_s[2] += ms * 1e-3f;
-        level_timed = false;
-    };
     // wide levels
     int level = 0;
     while (true) {
@@ -1152,20 +1166,18 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], w->node_cap, P.chunk, w->chunk_base, w->ctr);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
-        add_level_times();
         RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
         const int n_nodes = w->h_ctr->n_next;
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
         const int n_chunks = w->h_ctr->n_chunks;
         RSFK_CHECK(n_chunks <= w->chunk_cap, "tree batch: chunk table overflow");
-        (void)hipEventRecord(w->ev[0], stream);
         hipLaunchKernelGGL(k_level_planes, dim3((unsigned)((n_nodes + plane_waves - 1) / plane_waves)), dim3(64 * plane_waves),
-                           plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes);
-        // n_next := 0 for the level being produced
-        RSFK_HIP(hipMemsetAsync(&w->ctr->n_next, 0, sizeof(int), stream));
-        hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks, w->chunk2node);
-        (void)hipEventRecord(w->ev[1], stream);
+                           plane_waves * side_lds, stream, points, P, w->perm[0], w->perm[1], w->nodes[cur], n_nodes, w->planes,
+                           w->ctr);
+        // (also sets n_next := 0 for the level being produced)
+        hipLaunchKernelGGL(k_fill_chunks, dim3((n_chunks + 255) / 256), dim3(256), 0, stream, w->chunk_base, n_nodes, n_chunks,
+                           w->chunk2node, w->ctr);
         const bool swept = level < pm_levels;
         if (swept) {
             // the sides of every point in all trees of the batch, then their marks in the permutations
@@ -1199,7 +1211,6 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         else RSFK_SIDE_LAUNCH(true, 8);
 #undef RSFK_SIDE_LAUNCH
         }
-        (void)hipEventRecord(w->ev[2], stream);
         const bool map_next = level + 1 < pm_levels;
         hipLaunchKernelGGL(k_scatter, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                            w->chunk_base, w->chunk2node, w->chunk_left, w->nodes[cur ^ 1], w->node_cap, w->tail, w->tail_cap, w->ctr,
@@ -1209,8 +1220,6 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
             hipLaunchKernelGGL(pm::k_pm_next_map, dim3((unsigned)((nb * n_paths + 255) / 256)), dim3(256), 0, stream,
                                w->pm_map[level & 1], w->pm_map[(level + 1) & 1], w->pm_child, n_paths, nb);
         }
-        (void)hipEventRecord(w->ev[3], stream);
-        level_timed = true;
         RSFK_HIP(hipGetLastError());
         cur ^= 1;
         ++level;
@@ -1228,7 +1237,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
                            2 * (size_t)node_cap * sizeof(SmallNode) + (size_t)P.small;
         RSFK_CHECK(lds <= 150 * 1024, "tree batch: D too large for the tail kernel's LDS budget");
         const bool tail_q8 = q8 != nullptr && std::getenv("RSFK_TAIL_BF16") == nullptr;
-        (void)hipEventRecord(w->ev[4], stream);
+        (void)hipEventRecord(w->ev[0], stream);
         // few subtrees (small inputs, few trees): workgroups of 1024 threads, so that a subtree's levels take less time
         // (70,000 x 784, 10 trees: 1.24 -> 1.00 ms per tree).  RSFK_TAIL_BLOCK=256 / 1024 overrides.
         bool wide_wg = n_tail < 8 * 256;
@@ -1246,7 +1255,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         else if (wide_wg) RSFK_TAIL_LAUNCH(false, 1024);
         else RSFK_TAIL_LAUNCH(false, 256);
 #undef RSFK_TAIL_LAUNCH
-        (void)hipEventRecord(w->ev[5], stream);
+        (void)hipEventRecord(w->ev[1], stream);
         RSFK_HIP(hipGetLastError());
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
@@ -1254,7 +1263,19 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_HIP(hipStreamSynchronize(stream));
     if (n_tail > 0) {
         float ms = 0.0f;
-        if (hipEventElapsedTime(&ms, w->ev[4], w->ev[5]) == hipSuccess) w->phase_s[3] = ms * 1e-3f;
+        if (hipEventElapsedTime(&ms, w->ev[0], w->ev[1]) == hipSuccess) w->phase_s[3] = ms * 1e-3f;
+    }
+    {
+        // the steps of the wide levels, from the device's clock (events between the kernels of a level would cost
+        // more than some of the kernels)
+        int dev = 0, khz = 0;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) == hipSuccess &&
+            khz > 0) {
+            const float s_per_tick = 1e-3f / (float)khz;
+            w->phase_s[1] = (float)w->h_ctr->phase_ticks[0] * s_per_tick;       // hyperplanes
+            w->phase_s[0] = (float)w->h_ctr->phase_ticks[1] * s_per_tick;       // side tests
+            w->phase_s[2] = (float)w->h_ctr->phase_ticks[2] * s_per_tick;       // scatter
+        }
     }
     RSFK_CHECK(!w->h_ctr->overflow, "tree batch: queue overflow in the tail phase");
     for (int t = 0; t < nb; ++t) {
