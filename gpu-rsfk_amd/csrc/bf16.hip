@@ -46,6 +46,37 @@ __global__ __launch_bounds__(256) void k_col_sum(const float* __restrict__ point
     }
 }
 
+// The same for D <= 128: the workgroup reads m = 256 / D whole rows per step (thread t: row t / D of the step, column
+// t % D, so its column never changes), eight steps in flight; the threads of a column are added up in LDS.
+__global__ __launch_bounds__(256) void k_col_sum_narrow(const float* __restrict__ points, int N, int D, float* __restrict__ sum)
+{
+    __shared__ float part[256];
+    const int m = 256 / D;
+    const int rows_per = (N + gridDim.x - 1) / gridDim.x;
+    const int r0 = blockIdx.x * rows_per, r1 = min(N, r0 + rows_per);
+    const int sub = threadIdx.x / D, col = threadIdx.x - sub * D;
+    float acc = 0.0f;
+    if (sub < m) {
+        const float* src = points + col;
+        int r = r0 + sub;
+        for (; r + 7 * m < r1; r += 8 * m) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(r + u * m) * (size_t)D];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; r < r1; r += m) acc += src[(size_t)r * (size_t)D];
+    }
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    if ((int)threadIdx.x < D) {
+        float t = 0.0f;
+        for (int u = 0; u < m; ++u) t += part[u * D + threadIdx.x];
+        atomicAdd(&sum[threadIdx.x], t);
+    }
+}
+
 // sums -> means; a mean that is not finite is replaced by 0 (any shift is a valid one)
 __global__ void k_col_mean(float* __restrict__ mu, int D, float inv_n)
 {
@@ -130,6 +161,99 @@ __global__ __launch_bounds__(256) void k_to_q8(const float* __restrict__ points,
     }
 }
 
+// The same copy for rows whose 4-byte words of the 8-bit row (pitch - 16 bytes, the padding included) fit LPR lanes
+// with at most PPL words each: LPR lanes per row (64 / LPR rows per wavefront), the coordinates are read once, as
+// 16-byte pieces, and stay in registers between the pass that finds the range and the pass that rounds.  Produces the
+// bytes and headers of k_to_q8 (minimum, maximum and rounding do not depend on the order; the sum of the absolute
+// values, which only feeds the average that chooses between the screens, is added up in another order).
+// Needs D % 4 == 0 and 16-byte aligned points.
+template <int LPR, int PPL>
+__global__ __launch_bounds__(256) void k_to_q8_regs(const float* __restrict__ points, uint8_t* __restrict__ out,
+                                                    float* __restrict__ rho_sum, int N, int D, int pitch, float c_d)
+{
+    constexpr int kRowsPerWave = 64 / LPR;
+    const int lane = threadIdx.x & 63, sub = lane / LPR, l = lane - sub * LPR;
+    const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int n_waves = (gridDim.x * blockDim.x) >> 6;
+    const int words = (pitch - 16) >> 2, pieces = D >> 2;
+    float rho_acc = 0.0f;
+    for (int rb = wave_global * kRowsPerWave; rb < N; rb += n_waves * kRowsPerWave) {
+        const int r = rb + sub;
+        const bool row_ok = r < N;
+        const float* src = points + (size_t)(row_ok ? r : 0) * (size_t)D;
+        float4 x[PPL];
+        float lo = INFINITY, hi = -INFINITY, sabs = 0.0f;
+        bool bad = false;
+#pragma unroll
+        for (int k = 0; k < PPL; ++k) {
+            const int pc = l + k * LPR;
+            x[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (row_ok && pc < pieces) {
+                x[k] = *reinterpret_cast<const float4*>(src + 4 * pc);
+                const float v[4] = {x[k].x, x[k].y, x[k].z, x[k].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    bad |= !(fabsf(v[c]) <= 3.0e38f);              // NaN or infinite
+                    lo = fminf(lo, v[c]);
+                    hi = fmaxf(hi, v[c]);
+                    sabs += fabsf(v[c]);
+                }
+            }
+        }
+        int badi = bad ? 1 : 0;
+#pragma unroll
+        for (int o = 1; o < LPR; o <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, o, 64));
+            hi = fmaxf(hi, __shfl_xor(hi, o, 64));
+            sabs += __shfl_xor(sabs, o, 64);
+            badi |= __shfl_xor(badi, o, 64);
+        }
+        const float range = hi - lo;
+        const float scale = range * (1.0f / 255.0f);
+        const float inv = range > 0.0f ? 255.0f / range : 0.0f;
+        float err = 0.0f;
+        uint8_t* dst = out + (size_t)(row_ok ? r : 0) * (size_t)pitch;
+#pragma unroll
+        for (int k = 0; k < PPL; ++k) {
+            const int pc = l + k * LPR;
+            if (row_ok && pc < words) {
+                uint32_t packed = 0u;
+                if (pc < pieces) {
+                    const float v[4] = {x[k].x, x[k].y, x[k].z, x[k].w};
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        float t = __builtin_rintf((v[c] - lo) * inv);
+                        t = fminf(fmaxf(t, 0.0f), 255.0f);
+                        packed |= (uint32_t)t << (8 * c);
+                        err = fmaxf(err, fabsf(v[c] - __builtin_fmaf(scale, t, lo)));
+                    }
+                }
+                *reinterpret_cast<uint32_t*>(dst + 16 + 4 * pc) = packed;
+            }
+        }
+#pragma unroll
+        for (int o = 1; o < LPR; o <<= 1) err = fmaxf(err, __shfl_xor(err, o, 64));
+        const float mag = fabsf(lo) + 255.0f * scale;
+        float e1 = 1.01f * err + c_d * mag + 1e-37f;
+        if (badi || !(range <= 3.0e38f)) e1 = __builtin_nanf("");      // the screen never decides for such a row
+        if (row_ok && l == 0) {
+            *reinterpret_cast<float4*>(dst) = make_float4(0.0f, lo, scale, e1);
+            const float bf = sabs / (float)D * (1.0f / 256.0f);
+            rho_acc += (e1 == e1 && bf > 0.0f) ? fminf(e1 / bf, 1000.0f) : 1000.0f;
+        }
+    }
+    // one atomic per workgroup (they all hit the same address)
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) rho_acc += __shfl_xor(rho_acc, o, 64);
+    __shared__ float part[4];
+    if (lane == 0) part[threadIdx.x >> 6] = rho_acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float t = part[0] + part[1] + part[2] + part[3];
+        if (t != 0.0f) atomicAdd(rho_sum, t);
+    }
+}
+
 }  // namespace
 
 int q8_copy_alloc(Q8Copy* c, int N, int D)
@@ -153,7 +277,18 @@ int q8_copy_fill(const Q8Copy& c, const float* points, int N, int D, hipStream_t
     const int grid = std::min((N + 3) / 4, 4096);
     // (D/8 + D/32 + D + 32) 2^-24: chains of the screen and of the exact test, sum of the normal, rounding of lo + scale q
     const float c_d = (float)(D / 8 + D / 32 + D + 32) / 16777216.0f;
-    hipLaunchKernelGGL(k_to_q8, dim3(grid), dim3(256), 0, stream, points, c.rows, c.rho_sum, N, D, q8_pitch(D), c_d);
+    const int pitch = q8_pitch(D), words = (pitch - 16) >> 2;
+    const bool vec_ok = (D & 3) == 0 && (reinterpret_cast<uintptr_t>(points) & 15) == 0;
+#define RSFK_Q8_REGS(L, P)                                                                                                 \
+    hipLaunchKernelGGL((k_to_q8_regs<L, P>), dim3(std::min((N + 4 * (64 / L) - 1) / (4 * (64 / L)), 8192)), dim3(256), 0,   \
+                       stream, points, c.rows, c.rho_sum, N, D, pitch, c_d)
+    if (vec_ok && words <= 16) RSFK_Q8_REGS(16, 1);
+    else if (vec_ok && words <= 32) RSFK_Q8_REGS(32, 1);
+    else if (vec_ok && words <= 64) RSFK_Q8_REGS(64, 1);
+    else if (vec_ok && words <= 128) RSFK_Q8_REGS(64, 2);
+    else if (vec_ok && words <= 256) RSFK_Q8_REGS(64, 4);
+    else hipLaunchKernelGGL(k_to_q8, dim3(grid), dim3(256), 0, stream, points, c.rows, c.rho_sum, N, D, pitch, c_d);
+#undef RSFK_Q8_REGS
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -192,7 +327,8 @@ int bf16_copy_fill(const Bf16Copy& c, const float* points, int N, int D, hipStre
     if (c.mu) {
         RSFK_HIP(hipMemsetAsync(c.mu, 0, sizeof(float) * (size_t)D, stream));
         const int g = std::max(1, std::min(N / 64, 2048));
-        hipLaunchKernelGGL(k_col_sum, dim3(g), dim3(256), 0, stream, points, N, D, c.mu);
+        if (D <= 128) hipLaunchKernelGGL(k_col_sum_narrow, dim3(g), dim3(256), 0, stream, points, N, D, c.mu);
+        else hipLaunchKernelGGL(k_col_sum, dim3(g), dim3(256), 0, stream, points, N, D, c.mu);
         hipLaunchKernelGGL(k_col_mean, dim3((D + 255) / 256), dim3(256), 0, stream, c.mu, D, 1.0f / (float)N);
     }
     const int grid = std::min((N + 3) / 4, 65536);
