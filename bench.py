@@ -216,25 +216,38 @@ FP32_PEAK_TFLOPS = 157.3
 
 
 def gather_probe(dX, N, D, reps=5):
-    """Rate of rsfk_probe_gather_device over all rows of dX in a random order (HIP events on the launching stream)."""
+    """Rate of rsfk_probe_gather_device over all rows of dX in a random order (HIP events on the launching stream).
+    Twice: back to back ("GB/s": the last-level cache still holds what the run before left of the matrix -- all of a
+    small one), and each time after 600 MB of other data were written ("GB/s_after_other_writes": the caches hold
+    modified lines of something else, as they do between two kernels of a build, whose K-NN rows, permutations and
+    screening copies pass through them)."""
     import torch
     from gpu_rsfk import capi
     ids = torch.randperm(N, device=dX.device, dtype=torch.int64).to(torch.int32)
     sums = torch.empty(4096, dtype=torch.float32, device=dX.device)
+    other = torch.empty(150 * 1024 * 1024, dtype=torch.float32, device=dX.device)
     stream = torch.cuda.current_stream()
-    times = []
-    for rep in range(reps + 1):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        capi._check(capi.lib().rsfk_probe_gather_device(dX.data_ptr(), N, D, ids.data_ptr(), N, sums.data_ptr(),
-                                                       stream.cuda_stream))
-        e1.record(stream)
-        e1.synchronize()
-        if rep > 0:
-            times.append(e0.elapsed_time(e1) * 1e-3)
-    t = float(np.median(times))
-    return {"row_bytes": 4 * D, "rows": N, "seconds": round(t, 7), "GB/s": round(4.0 * D * N / t / 1e9, 1),
-            "note": "rows of the point matrix read once in a random order and nothing else"}
+    rates = []
+    for spoil in (False, True):
+        times = []
+        for rep in range(reps + 1):
+            if spoil:
+                other.fill_(float(rep))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            capi._check(capi.lib().rsfk_probe_gather_device(dX.data_ptr(), N, D, ids.data_ptr(), N, sums.data_ptr(),
+                                                           stream.cuda_stream))
+            e1.record(stream)
+            e1.synchronize()
+            if rep > 0:
+                times.append(e0.elapsed_time(e1) * 1e-3)
+        rates.append(float(np.median(times)))
+    del other
+    return {"row_bytes": 4 * D, "rows": N, "seconds": round(rates[0], 7), "GB/s": round(4.0 * D * N / rates[0] / 1e9, 1),
+            "seconds_after_other_writes": round(rates[1], 7),
+            "GB/s_after_other_writes": round(4.0 * D * N / rates[1] / 1e9, 1),
+            "note": "rows of the point matrix read once in a random order and nothing else; second figure: after 600 MB "
+                    "of other data were written, so that the caches hold none of the matrix"}
 
 
 PROFILE_FILES = {"c2": "knng_build_c2_uniform_1M_d100_k32.md", "c3": "knng_build_c3_gmm64_1M_d256_k32.md",
@@ -423,6 +436,8 @@ def main():
         if roofline.get("bound") == "hbm" and roofline["gather_probe"]["GB/s"] > 0:
             # the same achieved rate against what scattered rows of this size reach on the device
             roofline["frac_of_gather_rate"] = round(roofline["achieved"] / roofline["gather_probe"]["GB/s"], 4)
+            roofline["frac_of_gather_rate_after_other_writes"] = round(
+                roofline["achieved"] / roofline["gather_probe"]["GB/s_after_other_writes"], 4)
     except Exception as e:           # the probe is an aid: the line is valid without it
         roofline["gather_probe"] = {"error": str(e)}
 
