@@ -166,7 +166,7 @@ RSFK_API int rsfk_explore_device(const float* d_points, int N, int D, int num_ne
     ExploreWorkspace* ws = nullptr;
     Bf16Copy bfc;            // centred copy for the join
     if (!rc && explore_join_enabled(N, num_neighbors)) {
-        rc = explore_ws_alloc(&ws, N, num_neighbors, explore_merge_uses_bounds(D, num_neighbors));
+        rc = explore_ws_alloc(&ws, N, num_neighbors, explore_join_keeps_bounds(N, D, num_neighbors));
         if (!rc) rc = bf16_copy_alloc(&bfc, N, D, true);
         if (!rc) rc = bf16_copy_fill(bfc, d_points, N, D, s);
     }
@@ -256,7 +256,7 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
     ExploreWorkspace* ws = nullptr;
     Bf16Copy bfc;            // centred copy for the join
     if (!rc && explore_join_enabled(N, num_neighbors)) {
-        rc = explore_ws_alloc(&ws, N, num_neighbors, explore_merge_uses_bounds(D, num_neighbors));
+        rc = explore_ws_alloc(&ws, N, num_neighbors, explore_join_keeps_bounds(N, D, num_neighbors));
         if (!rc) rc = bf16_copy_alloc(&bfc, N, D, true);
         if (!rc) rc = bf16_copy_fill(bfc, static_cast<const float*>(dp.p), N, D, nullptr);
     }

@@ -76,6 +76,20 @@ __device__ __forceinline__ bool set_insert(int* table, int mask, int c, bool see
     return false;
 }
 
+// The same for a candidate, returning its place in the table (whether new or already there), or -1 when the id is a
+// seed (or the table is full).
+__device__ __forceinline__ int set_insert_at(int* table, int mask, int c)
+{
+    uint32_t h = hash_id(c) & (uint32_t)mask;
+    for (int i = 0; i <= mask; ++i) {
+        const int old = atomicCAS(&table[h], kEmpty, c);
+        if (old == kEmpty || old == c) return (int)h;
+        if (old == -c - 1) return -1;
+        h = (h + 1) & (uint32_t)mask;
+    }
+    return -1;
+}
+
 __device__ __forceinline__ void screen_pair(uint32_t w, float x0, float x1, float& da, float& ta)
 {
     const float c0 = __uint_as_float(w << 16);
@@ -338,6 +352,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
                                                                float* __restrict__ knn_dist, int table_size,
                                                                int wave_lds_ints, int dpad, int direct_max,
                                                                const uint32_t* __restrict__ pass,
+                                                               const uint16_t* __restrict__ bounds,
                                                                const int* __restrict__ todo_in, int n_in,
                                                                int* __restrict__ todo_out, int* __restrict__ n_out)
 {
@@ -367,6 +382,10 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     L.queue2 = nullptr;
     L.table = base + tile_ints + dpad;
     L.srow = L.table + table_size;
+    // with bounds: the smallest lower bound seen for the id in the same place of the set (bfloat16 bits), behind the
+    // list of marks
+    int* tbound = bounds ? L.srow + K + table_size / 4 * 3 : nullptr;
+    const int KP = (K + 31) & ~31;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
     KnnRow<SL> row;
@@ -379,7 +398,10 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     while (ts < 2 * (n_given + K + 1)) ts <<= 1;
     ts = min(ts, table_size);
     const int mask = ts - 1;
-    for (int i = lane; i < ts; i += 64) L.table[i] = kEmpty;
+    for (int i = lane; i < ts; i += 64) {
+        L.table[i] = kEmpty;
+        if (tbound) tbound[i] = 0x7fffffff;
+    }
     wave_lds_sync();
     if (lane == 0) set_insert(L.table, mask, p, true);
 #pragma unroll
@@ -411,29 +433,85 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     wave_lds_sync();
     for (int i0 = 0; i0 < n_marked; i0 += 64) {
         const int i = i0 + lane;
-        int c = -1;
+        int c = -1, lb = 0;
         if (i < n_marked) {
             const int e = marked[i];
             c = old_idx[(size_t)L.srow[e & 255] * K + (e >> 8)];
+            // the join's lower bound of the pair: entry p K + k of the graph, column = slot in the neighbour's row
+            if (bounds) lb = bounds[((size_t)p * K + (e & 255)) * (size_t)KP + (e >> 8)];
         }
-        if (c >= 0 && c < N) set_insert(L.table, mask, c, false);
+        if (c >= 0 && c < N) {
+            if (tbound) {
+                const int at = set_insert_at(L.table, mask, c);
+                if (at >= 0) atomicMin(&tbound[at], lb);
+            } else {
+                set_insert(L.table, mask, c, false);
+            }
+        }
     }
     wave_lds_sync();
-    // compact the set in place into the candidate list
+    // compact the set in place into the candidate list (and the bounds with it)
     int U = 0;
     for (int t0 = 0; t0 < ts; t0 += 64) {
         const int v = L.table[t0 + lane];
+        const int vb = tbound ? tbound[t0 + lane] : 0;
         const bool is_cand = v >= 0;
         const uint64_t m = ballot64(is_cand);
         wave_lds_sync();
-        if (is_cand) L.table[U + mask_prefix(m)] = v;
+        if (is_cand) {
+            L.table[U + mask_prefix(m)] = v;
+            if (tbound) tbound[U + mask_prefix(m)] = vb;
+        }
         U += __popcll(m);
     }
     wave_lds_sync();
-    for (int off = 0; off < U; off += 64) {
-        wave_lds_sync();
-        if (tile_ints == 0) exact_direct<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
-        else exact_batch<SL, kMergeChunk>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
+    auto batch = [&](const int* list, int n) {
+        if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
+        else exact_batch<SL, kMergeChunk>(L, list, n, points, D, vec_ok, row);
+    };
+    if (tbound == nullptr || U <= 64) {
+        for (int off = 0; off < U; off += 64) {
+            wave_lds_sync();
+            batch(L.table + off, min(64, U - off));
+        }
+    } else {
+        // Nearer bounds first: a round takes the candidates that are left, whose bound is not above the row's last
+        // slot (it shrinks from round to round) and -- while more than a batch of them is left -- not above the
+        // mean of these bounds.  A candidate whose bound is above the last slot cannot enter the row and is never
+        // read.  The ids of a round are gathered in the list of marks, which is no longer needed.  (Taking exactly
+        // the 64 nearest bounds of every round, found by bisection, was measured slower: the bounds of a point take
+        // few distinct values at 16 bits, and the search costs more than the order gains.)
+        constexpr int kDone = 0x7fffffff;
+        int* round_ids = marked;
+        while (true) {
+            const float tau_now = row.tau;
+            int n_el = 0, sum = 0;
+            for (int t0 = 0; t0 < U; t0 += 64) {
+                const int b = t0 + lane < U ? tbound[t0 + lane] : kDone;
+                const bool el = b != kDone && !(__uint_as_float((uint32_t)b << 16) > tau_now);
+                n_el += __popcll(ballot64(el));
+                sum += el ? b : 0;
+            }
+            if (n_el == 0) break;
+            sum = wave_sum_i(sum);
+            const int cut = n_el <= 64 ? 0xffff : sum / n_el;           // (the smallest bound is never above the mean)
+            int n_round = 0;
+            for (int t0 = 0; t0 < U; t0 += 64) {
+                const int b = t0 + lane < U ? tbound[t0 + lane] : kDone;
+                const bool take = b != kDone && !(__uint_as_float((uint32_t)b << 16) > tau_now) && b <= cut;
+                const uint64_t m = ballot64(take);
+                if (take) {
+                    round_ids[n_round + mask_prefix(m)] = L.table[t0 + lane];
+                    tbound[t0 + lane] = kDone;
+                }
+                n_round += __popcll(m);
+            }
+            for (int off = 0; off < n_round; off += 64) {
+                wave_lds_sync();
+                batch(round_ids + off, min(64, n_round - off));
+            }
+            wave_lds_sync();
+        }
     }
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
@@ -704,7 +782,7 @@ int next_pow2(int v)
 
 template <int SL, int WAVES>
 int launch_merge(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
-                 int wave_ints, int dpad, const uint32_t* pass, const int* todo_in, int n_in,
+                 int wave_ints, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
                  int* todo_out, int* n_out, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
@@ -713,25 +791,26 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
     const int n_work = todo_in ? n_in : N;
     dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, todo_in, n_in, todo_out, n_out);
+                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
 
-// ints of LDS a wavefront of the merge kernel needs for a set of `table` entries
-int merge_wave_ints(int table, int dpad, int K)
+// ints of LDS a wavefront of the merge kernel needs for a set of `table` entries: tile | point | set | row | list of
+// marks | with_bounds: a bound per place of the set
+int merge_wave_ints(int table, int dpad, int K, bool with_bounds = false)
 {
-    return (merge_tile_ints(dpad, merge_direct_max()) + dpad + table + K + table / 4 * 3 + 3) / 4 * 4;
+    return (merge_tile_ints(dpad, merge_direct_max()) + dpad + table + K + table / 4 * 3 + (with_bounds ? table : 0) + 3) / 4 * 4;
 }
 
 int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
-                   float* knn_dist, int table, int dpad, const uint32_t* pass, const int* todo_in,
+                   float* knn_dist, int table, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in,
                    int n_in, int* todo_out, int* n_out, hipStream_t stream)
 {
-    const int wi = merge_wave_ints(table, dpad, K);
+    const int wi = merge_wave_ints(table, dpad, K, bounds != nullptr);
 #define RSFK_MERGE_CASE(SLV, WV)                                                                                        \
     if (sl == SLV && waves == WV)                                                                                       \
-        return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, pass,       \
+        return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, pass, bounds, \
                                      todo_in, n_in, todo_out, n_out, stream);
     RSFK_MERGE_CASE(1, 4) RSFK_MERGE_CASE(1, 2) RSFK_MERGE_CASE(1, 1)
     RSFK_MERGE_CASE(2, 4) RSFK_MERGE_CASE(2, 2) RSFK_MERGE_CASE(2, 1)
@@ -757,6 +836,23 @@ int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, cons
 }
 
 }  // namespace
+
+// Does the join keep the lower bounds of the pairs it marks (N K KP 2-byte words)?  Yes for the rows that go to the
+// workgroup-per-point merge (below), and for rows of more than 128 dimensions while the array stays below 4 GB: the
+// wavefront-per-point merge then takes the candidates of a point nearer bounds first (their rows are long, and every
+// candidate that a tighter last slot turns away is a row not read; at 100 dimensions a point has fewer than 64
+// candidates, one batch, and the bounds only cost: merge 4.05 against 3.67 ms, join 6.0 against 3.6 ms at 1M x 100).
+// RSFK_MERGE_ORDER=0 switches the second case off.
+bool explore_join_keeps_bounds(int N, int D, int K)
+{
+    if (explore_merge_uses_bounds(D, K)) return true;
+    static const bool on = [] {
+        const char* e = std::getenv("RSFK_MERGE_ORDER");
+        return !(e && e[0] == '0');
+    }();
+    const size_t KP = (size_t)((K + 31) & ~31);
+    return on && D > 128 && K <= 64 && (size_t)N * (size_t)K * KP * 2 <= ((size_t)4 << 30);
+}
 
 bool explore_merge_uses_bounds(int D, int K)
 {
@@ -826,7 +922,10 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         int* listA = explore_ws_todo(ws, 0);
         int* listB = explore_ws_todo(ws, 1);
         int* host_n = explore_ws_host_count(ws);
-        if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, pass, nullptr, 0,
+        // (the bounds of the join, when it kept them and the set with a bound per place still fits)
+        const uint16_t* wave_bounds = explore_ws_bounds(ws);
+        if (4 * merge_wave_ints(small_table, dpad, K, true) > lds_ints) wave_bounds = nullptr;
+        if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, pass, wave_bounds, nullptr, 0,
                            listA, listA + N, stream))
             return 1;
         RSFK_HIP(hipMemcpyAsync(host_n, listA + N, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -847,7 +946,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
             int rc = 0;
             if (!per_wg)
                 rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, pass,
-                                    listA, n_todo, listB, listB + N, stream);
+                                    nullptr, listA, n_todo, listB, listB + N, stream);
             else if (sl == 1)
                 rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
                                         n_todo, listB, listB + N, stream);

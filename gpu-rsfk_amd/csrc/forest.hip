@@ -237,7 +237,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         ExploreWsGuard ews;      // without a workspace every point enumerates its own candidates
         Bf16Guard bfc;           // centred copy for the join
         if (explore_join_enabled(N, K)) {
-            if (explore_ws_alloc(&ews.w, N, K, explore_merge_uses_bounds(D, K))) return 1;
+            if (explore_ws_alloc(&ews.w, N, K, explore_join_keeps_bounds(N, D, K))) return 1;
             if (bf16_copy_alloc(&bfc.c, N, D, true) || bf16_copy_fill(bfc.c, d_points, N, D, stream)) return 1;
         }
         for (int it = 0; it < nnef; ++it) {

@@ -86,6 +86,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 // true when rows of K neighbours of D-dimensional points get the merge kernel that takes a point's candidates in the
 // order of their lower bounds (the workspace should then be allocated with room for the bounds)
 bool explore_merge_uses_bounds(int D, int K);
+bool explore_join_keeps_bounds(int N, int D, int K);
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
 
