@@ -467,7 +467,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     wave_lds_sync();
     auto batch = [&](const int* list, int n) {
         if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
-        else exact_batch<SL, kMergeChunk>(L, list, n, points, D, vec_ok, row);
+        else exact_batch<SL, kMergeChunk, true>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
     };
     if (tbound == nullptr || U <= 64) {
         for (int off = 0; off < U; off += 64) {
