@@ -242,11 +242,13 @@ def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
 @pytest.mark.parametrize("N,D,K,self_in", [(3000, 32, 16, True), (2000, 100, 32, True), (1500, 5, 8, False),
                                            (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True),
                                            (1300, 6, 200, True), (40, 7, 33, True), (5000, 130, 12, True),
-                                           (2200, 24, 64, True), (1600, 300, 100, True), (2600, 48, 20, True)])
+                                           (2200, 24, 64, True), (1600, 300, 100, True), (2600, 48, 20, True),
+                                           (3000, 200, 32, True)])
 def test_explore_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, self_in, join):
     """Both ways of enumerating the candidates: the join over the reversed graph (default; with partly empty
     rows and a large K its marks overflow the small set; K above about 45 then takes the merge kernel that puts a
-    whole workgroup on a point, and the general kernel finishes what is left)
+    whole workgroup on a point, and the general kernel finishes what is left; rows of more than 128 dimensions have
+    their candidates taken nearer lower bounds first, several hundred per point at 3000 x 200 with K = 32)
     and every point for itself (RSFK_EXPLORE_JOIN=0)."""
     if join == "plain":
         monkeypatch.setenv("RSFK_EXPLORE_JOIN", "0")
