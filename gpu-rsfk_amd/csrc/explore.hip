@@ -880,7 +880,7 @@ bool explore_merge_fits(int D, int K)
 // the candidates come from the join over the reversed graph (explore_join.hip), which needs rows sorted by
 // distance.
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
-                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream)
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted)
 {
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
@@ -889,7 +889,8 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
     const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
     // (rows too long for the LDS of the merge kernel: every point enumerates its own candidates)
     const bool join = ws != nullptr && bf_join != nullptr && bf_join->rows != nullptr && explore_merge_fits(D, K);
-    if (join && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
+    // (rows_sorted: the caller knows that every row is in order, e.g. after the bucket step of a forest)
+    if (join && !rows_sorted && launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
     RSFK_HIP(hipMemcpyAsync(old_idx, knn_idx, sizeof(int) * (size_t)N * (size_t)K, hipMemcpyDeviceToDevice, stream));
     const int fixed = 64 * kPitch + dpad + kQueue2 + K;                 // ints per wavefront besides the set
     const int lds_ints = 150 * 1024 / 4;                                // usable LDS per workgroup

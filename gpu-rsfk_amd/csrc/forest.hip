@@ -241,7 +241,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             if (bf16_copy_alloc(&bfc.c, N, D, true) || bf16_copy_fill(bfc.c, d_points, N, D, stream)) return 1;
         }
         for (int it = 0; it < nnef; ++it) {
-            if (launch_explore(d_points, plain_copy ? &bf.c : nullptr, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream))
+            // (the bucket step of the forest, and every exploration pass, leave all rows in order)
+            if (launch_explore(d_points, plain_copy ? &bf.c : nullptr, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream,
+                               n_trees > 0 || it > 0))
                 return 1;
         }
         RSFK_HIP(hipStreamSynchronize(stream));

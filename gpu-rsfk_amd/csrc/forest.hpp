@@ -88,7 +88,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 bool explore_merge_uses_bounds(int D, int K);
 bool explore_join_keeps_bounds(int N, int D, int K);
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
-                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream);
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted = false);
 
 // graph_export.hip
 int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int drop_self, int* d_indptr, int* d_cols,
