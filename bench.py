@@ -216,13 +216,18 @@ FP32_PEAK_TFLOPS = 157.3
 
 
 def gather_probe(dX, N, D, reps=5):
-    """Rate of rsfk_probe_gather_device over all rows of dX in a random order (HIP events on the launching stream).
+    """Rate of rsfk_probe_gather_device (the benchmark's own helper library, gpu-rsfk_amd/bench/librsfk_probe.so)
+    over all rows of dX in a random order (HIP events on the launching stream).
     Twice: back to back ("GB/s": the last-level cache still holds what the run before left of the matrix -- all of a
     small one), and each time after 600 MB of other data were written ("GB/s_after_other_writes": the caches hold
     modified lines of something else, as they do between two kernels of a build, whose K-NN rows, permutations and
     screening copies pass through them)."""
+    import ctypes
     import torch
-    from gpu_rsfk import capi
+    probe = ctypes.CDLL(os.path.join(ROOT, "gpu-rsfk_amd", "bench", "librsfk_probe.so")).rsfk_probe_gather_device
+    probe.restype = ctypes.c_int
+    probe.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_longlong, ctypes.c_void_p,
+                      ctypes.c_void_p]
     ids = torch.randperm(N, device=dX.device, dtype=torch.int64).to(torch.int32)
     sums = torch.empty(4096, dtype=torch.float32, device=dX.device)
     other = torch.empty(150 * 1024 * 1024, dtype=torch.float32, device=dX.device)
@@ -235,8 +240,8 @@ def gather_probe(dX, N, D, reps=5):
                 other.fill_(float(rep))
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
-            capi._check(capi.lib().rsfk_probe_gather_device(dX.data_ptr(), N, D, ids.data_ptr(), N, sums.data_ptr(),
-                                                           stream.cuda_stream))
+            if probe(dX.data_ptr(), N, D, ids.data_ptr(), N, sums.data_ptr(), stream.cuda_stream) != 0:
+                raise RuntimeError("gather probe: launch failed")
             e1.record(stream)
             e1.synchronize()
             if rep > 0:

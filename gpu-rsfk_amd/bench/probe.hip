@@ -5,10 +5,12 @@
 // fast the device delivers such rows bounds those kernels from below whatever they compute; this kernel does nothing
 // else -- one wavefront per row, 16-byte pieces, eight rows in flight per wavefront -- so that bench.py can report the
 // rate next to the rate of the bucket kernel.
-#include "rsfk_common.hpp"
-#include "wave64.hpp"
+//
+// Built into its own small shared library (librsfk_probe.so, next to this file): it is an aid of the benchmark and
+// not part of the product's interface, so librsfk.so neither contains nor exports it.
+#include <hip/hip_runtime.h>
+#include <cstdint>
 
-namespace rsfk {
 namespace {
 
 constexpr int kProbeBlocks = 4096;
@@ -55,14 +57,15 @@ __global__ __launch_bounds__(256) void k_probe_gather(const float* __restrict__ 
 
 }  // namespace
 
-int probe_gather_device(const float* d_points, int N, int D, const int* d_ids, long long n_ids, float* d_sums,
-                        hipStream_t stream)
+// Reads the rows ids[0..n_ids) of the N x D matrix d_points once (ids >= N are skipped) and adds them up into
+// d_sums (one float per workgroup launched: at least 4096 floats).  stream: a hipStream_t or null.
+// Returns 0, 1 on a launch error, 2 on bad arguments.
+extern "C" __attribute__((visibility("default"))) int rsfk_probe_gather_device(const float* d_points, int N, int D,
+                                                                               const int* d_ids, long long n_ids,
+                                                                               float* d_sums, void* stream)
 {
-    RSFK_CHECK(N >= 1 && D >= 1 && n_ids >= 0, "gather probe: N and D must be positive");
-    RSFK_CHECK(d_points && d_ids && d_sums, "gather probe: null pointer");
-    hipLaunchKernelGGL(k_probe_gather, dim3(kProbeBlocks), dim3(256), 0, stream, d_points, N, D, d_ids, n_ids, d_sums);
-    RSFK_HIP(hipGetLastError());
-    return 0;
+    if (N < 1 || D < 1 || n_ids < 0 || !d_points || !d_ids || !d_sums) return 2;
+    hipLaunchKernelGGL(k_probe_gather, dim3(kProbeBlocks), dim3(256), 0, static_cast<hipStream_t>(stream), d_points, N, D,
+                       d_ids, n_ids, d_sums);
+    return hipGetLastError() == hipSuccess ? 0 : 1;
 }
-
-}  // namespace rsfk

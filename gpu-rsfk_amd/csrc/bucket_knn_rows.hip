@@ -107,8 +107,10 @@ __global__ __launch_bounds__(kRowsThreads) void k_bucket_knn_rows(const float* _
 #pragma unroll
         for (int t = 0; t < NT; ++t) ok[t] = t < nt && cid[t] >= 0 && 64 * t + lane != m;
         // the first 64 candidates tell whether most candidates are below the row's last slot
+        // (the histogram below only ever sees candidates that passed enters(): a NaN distance would otherwise land in
+        // its first interval and push finite candidates out)
         int n_ok = DENSE ? __popcll(ballot64(ok[0] && row.enters(cid[0], acc[0]))) : 0;
-        if (DENSE && n_ok > 40) {
+        if (DENSE && n_ok > min(40, K + 16)) {
             n_ok = 0;
 #pragma unroll
             for (int t = 0; t < NT; ++t) {

@@ -274,12 +274,6 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
     return 0;
 }
 
-RSFK_API int rsfk_probe_gather_device(const float* d_points, int N, int D, const int* d_ids, long long n_ids, float* d_sums,
-                                      void* stream)
-{
-    return probe_gather_device(d_points, N, D, d_ids, n_ids, d_sums, static_cast<hipStream_t>(stream));
-}
-
 RSFK_API const char* rsfk_last_error(void) { return last_error(); }
 
 RSFK_API void rsfk_release_workspace(void)

@@ -68,8 +68,6 @@ void release_copy_buffers();
 
 // explore_join.hip
 struct ExploreWorkspace;
-int probe_gather_device(const float* d_points, int N, int D, const int* d_ids, long long n_ids, float* d_sums,
-                        hipStream_t stream);
 bool explore_join_enabled(int N, int K);
 bool explore_merge_fits(int D, int K);
 size_t explore_ws_bytes(int N, int K);

@@ -209,7 +209,9 @@ int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int d
 
 // ---------------------------------------------------------------------------------------------------------------------
 // The count-only call (row lengths, d_indptr and the number of entries) for callers that cannot allocate device memory:
-// code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Its working memory -- the edge
+// tight serving loops, harnesses that forbid hipMalloc, code that records a HIP graph.  With nnz == nullptr the call
+// only enqueues kernels (the count is left in d_indptr[N] on the device); with nnz != nullptr it also copies the
+// count to the host and synchronises the stream, which a stream under capture refuses.  Its working memory -- the edge
 // flags, the three per-point counters and the temporary storage of the prefix sum, which symmetrize_device takes from
 // the workspace pool -- lives in a file-scope device array of fixed size.  Every GPU the library runs on holds its
 // own copy of that array until the process ends; its address on a device is looked up once per device and kept.
@@ -261,7 +263,7 @@ __global__ __launch_bounds__(256) void k_zero_counters(int* __restrict__ v, int 
 
 int symmetrize_count_noalloc(const int* d_idx, int N, int K, int drop_self, int* d_indptr, long long* nnz, hipStream_t stream)
 {
-    RSFK_CHECK(d_idx && d_indptr && nnz, "graph export: null argument");
+    RSFK_CHECK(d_idx && d_indptr, "graph export: null argument");
     RSFK_CHECK(N >= 1 && K >= 1 && K <= 256, "graph export: N must be positive and K in 1..256");
     RSFK_CHECK(N <= kNaMaxPoints && (long long)N * K <= kNaMaxSlots,
                "graph export without allocation: at most 2^20 points and 2^25 neighbour slots (N * K)");
@@ -282,6 +284,7 @@ int symmetrize_count_noalloc(const int* d_idx, int N, int K, int drop_self, int*
     hipLaunchKernelGGL(k_sym_len, dim3((unsigned)(N / 256 + 1)), dim3(256), 0, stream, n_own, ext, N, len);
     RSFK_HIP(hipGetLastError());
     RSFK_HIP(rocprim::exclusive_scan(scan_tmp, tmp_bytes, len, d_indptr, 0, (size_t)N + 1, rocprim::plus<int>(), stream));
+    if (nnz == nullptr) return 0;                       // the count stays in d_indptr[N]; nothing but kernels was queued
     int total = 0;
     RSFK_HIP(hipMemcpyAsync(&total, d_indptr + N, sizeof(int), hipMemcpyDeviceToHost, stream));
     RSFK_HIP(hipStreamSynchronize(stream));

@@ -31,7 +31,6 @@ SYMBOLS = {
     "rsfk_explore_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _f32, _ci]),
     "rsfk_last_error": (ctypes.c_char_p, []),
     "rsfk_device_count": (_ci, []),
-    "rsfk_probe_gather_device": (_ci, [_vp, _ci, _ci, _vp, ctypes.c_longlong, _vp, _vp]),
     "rsfk_release_workspace": (None, []),
 }
 
@@ -151,13 +150,14 @@ def symmetrize_device(d_idx, d_dist, N, K, drop_self, d_indptr, d_cols, d_vals, 
     return int(nnz.value)
 
 
-def symmetrize_count_noalloc(d_idx, N, K, drop_self, d_indptr, stream=0):
+def symmetrize_count_noalloc(d_idx, N, K, drop_self, d_indptr, stream=0, fetch_count=True):
     """Row offsets and number of entries of the symmetrised graph without any allocation in the library (fixed
-    working memory: N <= 2^20, N * K <= 2^25) -> number of entries."""
+    working memory: N <= 2^20, N * K <= 2^25) -> number of entries.  fetch_count=False: the library only enqueues
+    its kernels (no copy to the host, no synchronisation); the count is d_indptr[N] on the device and None is returned."""
     nnz = ctypes.c_longlong(0)
     _check(lib().rsfk_symmetrize_count_noalloc(_vp(d_idx), int(N), int(K), int(bool(drop_self)), _vp(d_indptr),
-                                               ctypes.byref(nnz), _vp(stream)))
-    return int(nnz.value)
+                                               ctypes.byref(nnz) if fetch_count else None, _vp(stream)))
+    return int(nnz.value) if fetch_count else None
 
 
 def bucket_knn_device(d_points, N, D, K, d_ids, d_starts, d_sizes, n_buckets, stride, d_idx, d_dist, stream=0):

@@ -120,8 +120,10 @@ int rsfk_symmetrize_device(const int* d_knn_indices, const float* d_knn_sqr_dist
 
 /* The count-only form of rsfk_symmetrize_device (d_indices = d_data = NULL there): fills d_indptr (N + 1 ints) and *nnz
  * with the row offsets and the number of entries of the symmetrised graph.  It has no counterpart in the reference.
- * It is for callers that cannot allocate device memory -- code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc: it calls no hipMalloc, hipFree or other allocating routine.  Its working memory
+ * It is for callers that cannot allocate device memory -- tight serving loops, harnesses that forbid hipMalloc, code
+ * that records a HIP graph: it calls no hipMalloc, hipFree or other allocating routine.  With nnz != NULL it ends with
+ * a copy of the count to the host and a synchronisation of the stream (not allowed on a stream under capture); with
+ * nnz == NULL it only enqueues kernels and the count is d_indptr[N] on the device.  Its working memory
  * (edge flags, per-point counters, the temporary storage of the prefix sum) is a fixed array of 45 MiB that every GPU
  * the library runs on holds until the process ends.  Limits: N <= 2^20 and N * num_neighbors <= 2^25; larger inputs
  * are refused with an error.  All calls on one GPU share the array, so calls that overlap on one GPU (other
@@ -175,14 +177,6 @@ void rsfk_release_workspace(void);
 
 /* number of HIP devices visible to the library (0 when there is none) */
 int rsfk_device_count(void);
-
-/* Measurement aid, no counterpart in the reference: reads the rows ids[0..n_ids) of the device matrix points
- * (N x D floats) the way the bucket kernels gather them -- one wavefront per row, 16-byte pieces -- and adds them
- * up into sums (one float per workgroup launched, at least 4096 floats).  bench.py times it to report the rate at
- * which this device delivers scattered rows of 4 D bytes, next to the rate of the bucket K-NN kernel.  stream: a
- * hipStream_t or null.  Returns 0, or nonzero with the reason in rsfk_last_error(). */
-int rsfk_probe_gather_device(const float* d_points, int N, int D, const int* d_ids, long long n_ids, float* d_sums,
-                             void* stream);
 
 #ifdef __cplusplus
 }

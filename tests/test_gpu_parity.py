@@ -812,6 +812,27 @@ def test_points_with_nan_coordinates(gpu, orc, rng):
     assert_knn_equal(gi, gd, oi, od)
 
 
+@pytest.mark.parametrize("K,D", [(8, 24), (5, 32), (20, 16)])
+def test_points_with_nan_coordinates_in_large_buckets(gpu, orc, rng, K, D):
+    """The same rule in the kernel that keeps a bucket's points in LDS (buckets of 80..256 low-dimensional points),
+    with a third of the points NaN and K small: in the first two trees of a build nearly every candidate of a member
+    is below its row's last slot, so the step that drops candidates by a histogram of their distances runs, and it
+    must see the candidates with a NaN distance as absent."""
+    import gpu_rsfk
+    N, T = 9000, 3
+    X = rng.standard_normal((N, D)).astype(np.float32)
+    bad = np.arange(0, N, 3)
+    X[bad, rng.integers(0, D, size=len(bad))] = np.nan
+    _say("nan rows, large buckets", K, D)
+    gi, gd = gpu_rsfk.RSFK(random_state=5).find_nearest_neighbors(X, K, n_trees=T, min_tree_children=80,
+                                                                  max_tree_children=256, nn_exploring_factor=0)
+    oi, od = orc.init_lists(N, K, self_in=True)
+    orc.forest(X, K, T, 80, 256, 5000, 5, 0, knn_idx=oi, knn_dist=od)
+    assert not np.isnan(gd).any() and not np.isnan(od).any()
+    assert (gi[bad, 0] == bad).all() and (gi[bad, 1:] == -1).all()
+    assert_knn_equal(gi, gd, oi, od)
+
+
 def test_forest_in_several_batches(gpu, orc, rng, monkeypatch):
     """Trees are built a batch at a time (all at once when memory allows); two per batch must give the same graph,
     for the K-NN graph (buckets of both kinds, so both streams of the bucket step are in use) and the query search."""

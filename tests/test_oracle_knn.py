@@ -88,6 +88,39 @@ def test_explore_matches_python_restatement(orc, rng, N, D, K):
     assert_knn_equal(idx, dist, pi, pd)
 
 
+@pytest.mark.parametrize("N,D,K,trees,self_in", [(300, 5, 6, 2, True), (500, 9, 12, 1, True), (400, 3, 8, 2, False),
+                                                 (350, 2, 10, 1, True)])
+def test_explore_is_the_k_smallest_of_row_and_neighbours_of_neighbours(orc, rng, N, D, K, trees, self_in):
+    """Set definition, no loop restated: after a pass the row of p holds the K smallest (distance, index) pairs of
+    its old row joined with the rows (of the snapshot) of its old neighbours, p itself left out of what is offered.
+    Distances come from an independent float64 evaluation rounded through the same fp32 chain (orc.sqdist is pinned
+    by test_oracle_math.py); integer lattice points (the D = 2 case) make ties at the K-th distance common."""
+    if D == 2:
+        X = rng.integers(0, 7, size=(N, D)).astype(np.float32)
+    else:
+        X = rng.random((N, D), dtype=np.float32)
+    idx, dist = orc.init_lists(N, K, self_in=self_in)
+    for seed in range(trees):
+        perm, ls, lz, _ = orc.build_tree(X, 4, 11, 5000, seed)      # small buckets: some rows stay partly empty
+        orc.bucket_knn(X, K, perm, lz, idx, dist, starts=ls)
+    old_i, old_d = idx.copy(), dist.copy()
+    orc.explore(X, K, idx, dist)
+    si, sd = sort_rows(idx, dist)
+    for p in range(N):
+        mine = {int(c): float(d) for c, d in zip(old_i[p], old_d[p]) if c >= 0}
+        offered = set()
+        for q in old_i[p]:
+            if q >= 0:
+                offered.update(int(c) for c in old_i[q] if c >= 0)
+        offered.discard(p)
+        for c in offered - set(mine):
+            mine[c] = float(orc.sqdist(X[p], X[c]))
+        want = sorted((d, c) for c, d in mine.items())[:K]
+        got = [(float(d), int(c)) for d, c in zip(sd[p], si[p]) if c >= 0]
+        assert got == want, "row %d" % p
+        assert (si[p, len(want):] == -1).all()
+
+
 def test_explore_with_empty_slots_and_without_self(orc, rng):
     """-1 neighbours are skipped (the reference reads out of range there) and a
     point is never offered to itself."""
@@ -249,3 +282,39 @@ def test_infinite_distance_never_enters(orc):
         mates = {0, 1, 2} if p < 3 else {3, 4, 5}
         assert set(idx[p][idx[p] >= 0]) == mates
         assert not np.isin(idx[p], list({0, 1, 2, 3, 4, 5} - mates)).any()
+
+
+def _reference_rule_bucket(orc, X, K, bucket, idx, dist):
+    """The reference's own rule, unordered rows and all (compute_knn_from_buckets.cu:1198-1286): every pair i < j of
+    the bucket in the order of its diagonals; a candidate enters iff it is strictly below the row's maximum and is
+    not in the row, and it overwrites the first slot that holds the maximum."""
+    s = len(bucket)
+    for diag in range(1, s):
+        for i in range(s - diag):
+            a, b = bucket[i], bucket[i + diag]
+            d = orc.sqdist(X[a], X[b])
+            for p, c in ((a, b), (b, a)):
+                worst = int(np.argmax(dist[p]))
+                if not d < dist[p, worst] or c in idx[p]:
+                    continue
+                idx[p, worst] = c
+                dist[p, worst] = d
+
+
+def test_rows_equal_those_of_the_reference_rule_where_nothing_ties(orc, rng):
+    """The (distance, index) order of the rows differs from the reference's strict first-arrival rule only among
+    points tied at a row's K-th distance: on points in general position (no two pair distances of a row equal) the
+    rows, as sets, are the ones the reference's unordered replace-the-maximum rule produces."""
+    N, D, K = 260, 6, 7
+    X = rng.random((N, D), dtype=np.float32)
+    idx, dist = orc.init_lists(N, K)
+    ri, rd = idx.copy(), dist.copy()
+    for seed in range(3):
+        perm, ls, lz, _ = orc.build_tree(X, 8, 20, 5000, seed)
+        orc.bucket_knn(X, K, perm, lz, idx, dist, starts=ls)
+        for s, z in zip(ls, lz):
+            _reference_rule_bucket(orc, X, K, [int(p) for p in perm[s:s + z]], ri, rd)
+    # general position: no row holds two equal distances (so no tie can have been decided either way)
+    sd = np.sort(rd, 1)
+    assert (sd[:, 1:] != sd[:, :-1]).all()
+    assert_knn_equal(idx, dist, ri, rd)

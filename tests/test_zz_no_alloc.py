@@ -1,6 +1,7 @@
 """The entry point that allocates nothing (rsfk_symmetrize_count_noalloc) against the count-only call of
 rsfk_symmetrize_device: identical row offsets and entry counts, on two calls in a row, the second with a smaller
-input (the fixed working memory keeps the first call's contents), and refusal of inputs beyond its limits."""
+input (the fixed working memory keeps the first call's contents), the form that leaves the count on the device, the
+amount of free device memory before and after, and refusal of inputs beyond its limits."""
 import numpy as np
 import pytest
 
@@ -29,10 +30,21 @@ def test_no_alloc_entry_point_matches_the_allocating_one(gpu):
         want = torch.empty(N + 1, dtype=torch.int32, device="cuda")
         got = torch.full((N + 1,), -7, dtype=torch.int32, device="cuda")
         nnz_want = gpu.symmetrize_device(d_idx.data_ptr(), 0, N, K, drop_self, want.data_ptr(), 0, 0, 0)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
         nnz_got = gpu.symmetrize_count_noalloc(d_idx.data_ptr(), N, K, drop_self, got.data_ptr())
         torch.cuda.synchronize()
+        # the device's free memory did not move (the allocating call would take 7 MB and more for the first input;
+        # the slack is for the runtime's own small pools)
+        assert abs(torch.cuda.mem_get_info()[0] - free_before) <= (1 << 20)
         assert nnz_got == nnz_want and nnz_got > 0
         assert torch.equal(got, want)
+        # the form that only enqueues kernels: no count comes back, it is the last row offset on the device
+        got.fill_(-7)
+        assert gpu.symmetrize_count_noalloc(d_idx.data_ptr(), N, K, drop_self, got.data_ptr(), fetch_count=False) is None
+        torch.cuda.synchronize()
+        assert abs(torch.cuda.mem_get_info()[0] - free_before) <= (1 << 20)
+        assert torch.equal(got, want) and int(got[N]) == nnz_want
     with pytest.raises(gpu.RsfkError):
         gpu.symmetrize_count_noalloc(d_idx.data_ptr(), (1 << 20) + 1, 1, True, got.data_ptr())
     with pytest.raises(gpu.RsfkError):
