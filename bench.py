@@ -8,7 +8,15 @@ pass, buckets 33..66; ``--config c1..c5`` selects any of the five.  Prints one
 JSON line.  ``host_call_seconds`` is the region the reference times
 (``RSFK._last_search_time``: host arrays in, host arrays out).
 
-The roofline object is for the bucket K-NN step: algorithmic bytes per launch
+``value`` times the device-resident build (``timed_region``).  Three roofline objects, one per subsystem:
+``roofline`` (bucket K-NN, the metric's kernel), ``roofline_tree`` (tree build: sum over the levels of the points of
+the nodes that are split, times the bytes of a screening row and of the permutation entry read and written by the side
+test and by the scatter, plus the fp32 rows of the points the screen leaves to the exact test, plus the permutation
+written once) and ``roofline_explore`` (one pass: the fp32 rows of the candidates that get an exact distance, the
+K^2 ids of the neighbours' rows and the K-NN row read and written); the counts come from the library's report of
+the build (``rsfk_last_build_report``), as do the names of the bucket kernels that ran.
+
+The first roofline object is for the bucket K-NN step: algorithmic bytes per launch
 (one launch = one tree) = N*(4D + 4 + 16K) -- every point row gathered once, every
 id read once, every K-NN row (index + distance) read once and written once --
 or, where the arithmetic intensity is above the machine balance, 3 D P flops
@@ -260,16 +268,32 @@ PROFILE_FILES = {"c2": "knng_build_c2_uniform_1M_d100_k32.md", "c3": "knng_build
 FETCH_SCALE = 1.92          # FETCH_SIZE reads 0.52 of the bytes a copy kernel of known size loads; WRITE_SIZE matches
 
 
+def bucket_sources_hash():
+    """Hash of the sources of the bucket K-NN kernels: a tracked profile states the hash it was made with, and its
+    counters are only taken for this run's line when the kernels are still the same."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "gpu-rsfk_amd", "csrc")
+    for fn in sorted(os.listdir(src)):
+        if fn.startswith("bucket_knn") or fn in ("knn_list.hpp", "mfma_split.hpp", "wave64.hpp"):
+            h.update(open(os.path.join(src, fn), "rb").read())
+    return h.hexdigest()[:16]
+
+
 def profiled_traffic(config, steps_profiled=2):
     """HBM bytes per tree of the bucket K-NN kernels from the tracked rocprofv3 summary of this workload
-    (profiles/: FETCH_SIZE and WRITE_SIZE in KiB per launch, launches of two builds), or None.  The counters cannot be
-    collected inside this run; the summary is of the same command (bench.py --config <c>) and says how it was made."""
+    (profiles/: FETCH_SIZE and WRITE_SIZE in KiB per launch, launches of two builds), or None -- also None when the
+    summary was made with other sources of the bucket kernels than this run's (its line "bucket kernel sources:").
+    The counters cannot be collected inside this run; the summary is of the same command (bench.py --config <c>)."""
     fn = PROFILE_FILES.get(config)
     path = os.path.join(ROOT, "profiles", fn) if fn else None
     if not path or not os.path.exists(path):
         return None
+    text = open(path).read()
+    if ("bucket kernel sources: " + bucket_sources_hash()) not in text:
+        return None
     launches, kib = {}, {}
-    for line in open(path):
+    for line in text.splitlines():
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
         if len(cells) == 7 and cells[0].startswith("k_bucket_knn"):
             try:
@@ -286,32 +310,25 @@ def profiled_traffic(config, steps_profiled=2):
     return total / steps_profiled if total > 0 else None
 
 
-def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts):
+def bucket_roofline(N, D, K, T, mn, mx, knn_s, leaf_counts, kernels):
     """Roofline object of the bucket K-NN step of one tree (one step of the forest loop = one tree's launches).
 
     Bytes: N (4D + 4 + 16K) per tree.  Flops: 3 D P with P = pairs of the tree's buckets, estimated from the number of
     buckets L the run reported as N (N / L - 1) / 2 (equal buckets: a lower bound of the true sum).  The bound is the
-    one the workload's arithmetic intensity selects: fp32 when flops / bytes exceeds peak flops / peak bandwidth."""
+    one the workload's arithmetic intensity selects: fp32 when flops / bytes exceeds peak flops / peak bandwidth.
+    kernels: what the library says it launched (runs of trees and kernel names, rsfk_last_build_report)."""
     alg_bytes = float(N) * (4 * D + 4 + 16 * K)
     mean_leaves = float(np.mean(leaf_counts)) if len(leaf_counts) else max(1.0, N / (0.75 * mx))
     pairs = 0.5 * N * (N / mean_leaves - 1.0)
     alg_flops = 3.0 * D * pairs
     balance = FP32_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
-    small = K <= 64 and mx <= 72
-    gram = os.environ.get("RSFK_GRAM_FROM")
-    scr = os.environ.get("RSFK_BUCKET_SCREEN")
-    first = (4 if D >= 128 else 8) if not scr else (int(scr) if scr.isdigit() else None)
-    kernel = (("k_bucket_knn_small<64> (buckets <= 64" + ("" if first is None else "; trees 0..%d" % (first - 1) if first > 0 else "; no tree")
-               + ")" + ("" if first is None else " / k_bucket_knn_screen (later trees: pair matrix bounded on the matrix cores)")
-               + " + k_bucket_knn_small<72> (65..72)") if small
-              else ("k_bucket_knn_rows (a bucket's points resident in LDS, every K-NN row touched once)"
-                    if K <= 64 and mx <= 64 * min(4, (40960 - 1024) // (64 * (4 * (((D + 3) & ~3) + (4 if (((D + 3) >> 2) & 1) == 0 else 0)) + 4)))
-                    else "k_bucket_knn (64 x 64 tiles of the pair matrix)") + ("" if mx <= 72 or K > 64 else " + k_bucket_knn_small for the buckets up to 72 points"))
-    if gram is not None:
-        kernel += "; k_bucket_knn_gram from tree %s on (RSFK_GRAM_FROM)" % gram
+    kernel = "; ".join("trees %d..%d: %s" % (a, b, " + ".join(names)) for a, b, names in kernels) if kernels else "none"
     if alg_flops / alg_bytes > balance:
         ach = alg_flops / knn_s / 1e12 if knn_s > 0 else 0.0
-        return {"kernel": kernel, "bound": "mfma", "achieved": round(ach, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+        # "mfma" is the name the bench contract has for the compute roofline; the peak used is the fp32 one (vector
+        # and matrix fp32 peaks are the same figure on this device) and "unit_used" names what the kernel ran on
+        return {"kernel": kernel, "bound": "mfma", "unit_used": "fp32 vector ALUs (the chains of the direct-difference path)",
+                "achieved": round(ach, 2), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(ach / FP32_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops_per_launch": alg_flops,
                 "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": round(knn_s * 1e3, 4), "launches_per_step": T,
                 "note": "flops = 3 D P of the direct-difference path (fp32 peak 157.3 TFLOP/s); HBM traffic: see profiles/"}
@@ -399,6 +416,7 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     sec_per_step = elapsed / max(args.steps, 1)
+    report = capi.last_build_report()               # of the last timed step
 
     # recall against exact K-NN on a seeded sample of query rows
     nq = min(args.recall_queries, N)
@@ -424,15 +442,44 @@ def main():
     tree_s = float(np.mean([np.mean(f.data["Total Tree Building Time"]) for f in fls])) if fls and T > 0 else 0.0
     expl_s = float(np.mean([f.exploration_time for f in fls])) if fls else 0.0
     leaves = fls[0].data["Total Leaves"] if fls and T > 0 else []
-    roofline = bucket_roofline(N, D, K, T, mn, mx, knn_s, leaves)
+    roofline = bucket_roofline(N, D, K, T, mn, mx, knn_s, leaves, report.get("bucket_kernels", []))
+    roofline_tree = roofline_explore = None
+    if T > 0 and report.get("tree_points_tested", 0) > 0:
+        R = report["tree_screen_row_bytes"]
+        tb = (report["tree_points_tested"] * (R + 16.0) + report["tree_points_undecided"] * 4.0 * D) / T + 4.0 * N
+        ach = tb / tree_s / 1e9 if tree_s > 0 else 0.0
+        roofline_tree = {"kernel": "tree build of one tree (k_pm_sweep / k_side, k_scatter, k_tail; trees are built in batches, level by level)",
+                         "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_launch": round(tb),
+                         "avg_launch_ms": round(tree_s * 1e3, 4), "launches_per_step": T,
+                         "point_levels_per_point": round(report["tree_points_tested"] / float(T) / N, 3),
+                         "undecided_share": round(report["tree_points_undecided"] / float(report["tree_points_tested"]), 5),
+                         "screen_row_bytes": R,
+                         "note": "bytes = sum over levels of the points of split nodes x (screening row + 16 for the permutation entry "
+                                 "read and written by side test and scatter) + undecided points x 4 D + 4 N; time = host time of a "
+                                 "batch of trees / trees"}
+    if args.explore > 0 and report.get("explore_passes", 0) > 0:
+        per_pass = report["explore_exact_distances"] / float(report["explore_passes"])
+        eb = per_pass * 4.0 * D + float(N) * (4.0 * K * K + 16.0 * K)
+        es = expl_s / report["explore_passes"]
+        ach = eb / es / 1e9 if es > 0 else 0.0
+        roofline_explore = {"kernel": "one exploration pass (reversed graph, join on the matrix cores, merge)", "bound": "hbm",
+                            "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                            "traffic": None, "algorithmic_bytes_per_launch": round(eb), "avg_launch_ms": round(es * 1e3, 4),
+                            "launches_per_step": report["explore_passes"],
+                            "exact_distances_per_point": round(per_pass / N, 2),
+                            "note": "bytes = N (U 4 D + 4 K^2 + 16 K), U = exact distances per point counted by the merge kernels"}
     cfg_name = next((name for name, c in CONFIGS.items()
                      if (args.workload, N, D, K, T, mn, mx, args.explore) == c), None)
     per_build = profiled_traffic(cfg_name) if T > 0 and cfg_name else None
     if per_build:
         roofline["traffic"] = round(per_build / T)
         roofline["note"] = ("traffic: HBM bytes per tree of the bucket K-NN kernels from the tracked rocprofv3 summary of this "
-                            "command (profiles/%s: FETCH_SIZE x %.2f + WRITE_SIZE, all bucket kernels of a build / trees)"
-                            % (PROFILE_FILES[cfg_name], FETCH_SCALE))
+                            "command, made with the same kernel sources (profiles/%s: FETCH_SIZE x %.2f + WRITE_SIZE, all "
+                            "bucket kernels of a build / trees)" % (PROFILE_FILES[cfg_name], FETCH_SCALE))
+    elif cfg_name:
+        roofline["note"] = ("traffic: null -- the tracked rocprofv3 summary (profiles/%s) was made with other sources of the "
+                            "bucket kernels than this run's" % PROFILE_FILES[cfg_name])
     # what the device delivers when scattered rows of 4 D bytes are only read: every row of the matrix once, in a random
     # order, by rsfk_probe_gather_device (one wavefront per row, nothing computed); the bucket kernels gather the same
     # rows in the order of a tree's permutation and cannot be faster than this on their N 4 D bytes
@@ -484,6 +531,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "%s%s N=%d D=%d K=%d n_trees=%d buckets=%d..%d exploration=%d seed=0" % (
             (args.config + " = ") if args.config else "", args.workload, N, D, K, T, mn, mx, args.explore)},
+        "timed_region": "device-resident build: points and K-NN rows in HBM before and after (rsfk_knn_forest_device); "
+                        "host_call_seconds is the region the reference times (host arrays in and out)",
         "build_seconds": round(sec_per_step, 5),
         "host_call_seconds": None if host_s is None else round(host_s, 5),
         "host_call_points_per_sec": None if host_s is None else round(N / host_s, 1),
@@ -492,6 +541,8 @@ def main():
         "phase_seconds": {"tree_build_per_tree": round(tree_s, 6), "bucket_knn_per_tree": round(knn_s, 6),
                           "exploration": round(expl_s, 6)},
         "roofline": roofline,
+        "roofline_tree": roofline_tree,
+        "roofline_explore": roofline_explore,
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -254,7 +254,7 @@ namespace {
 
 int launch_general(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
                    int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted = false,
-                   int max_bucket = -1)
+                   int max_bucket = -1, int* launched = nullptr)
 {
     if (n_buckets <= 0) return 0;
     const int rs = rows_sorted ? 1 : 0;
@@ -263,6 +263,7 @@ int launch_general(const float* points, int D, int K, const int* ids, const int*
     const char* env = std::getenv("RSFK_BUCKET_STRIP");        // 0 / 1 overrides the choice (the results are the same)
     const bool strip = max_tiles > 1 && (env && *env ? env[0] == '1' : n_buckets <= kStripBuckets);
     dim3 grid((unsigned)n_buckets * (unsigned)(strip ? max_tiles : 1)), block(256);
+    if (launched) *launched |= strip ? kBucketKernelStrip : kBucketKernelTiled;
 #define RSFK_GENERAL_CASE(SLV)                                                                                              \
     do {                                                                                                                    \
         if (strip)                                                                                                          \
@@ -387,11 +388,14 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // far from done (first trees of a build).
 int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part, bool young_rows)
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part, bool young_rows, int* launched)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
+    int none = 0;
+    int& used = launched ? *launched : none;              // which kernels this tree's buckets went to (kBucketKernel...)
     if (gram && rows_sorted) {
+        used |= kBucketKernelGram;
         // pair matrix screened on the matrix cores; buckets of 65..72 points (K <= 64) keep their own kernel
         if (n_small > 0 && part != 2 &&
             launch_bucket_knn_gram(points, D, K, ids, starts, sizes, n_small, 0, 2, kBucketSplit, knn_idx, knn_dist, stream))
@@ -400,6 +404,7 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
         const int off = leaf_cap - n_big;
         int from = kBucketSplit + 1;
         if (K <= 64) {
+            used |= kBucketKernelMedium;
             if (launch_bucket_knn_medium(points, D, K, ids, starts + off, sizes + off, n_big, 0, rows_sorted, knn_idx, knn_dist, stream))
                 return 1;
             if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
@@ -411,11 +416,13 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
     }
     if (n_small > 0 && part != 2) {
         if (K <= 64 && screen && rows_sorted) {
+            used |= kBucketKernelScreen;
             if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
         } else if (K <= 64) {
+            used |= kBucketKernelSmall;
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted,
-                                  kBucketSplit)) {
+                                  kBucketSplit, &used)) {
             return 1;
         }
     }
@@ -424,12 +431,14 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
     const int off = leaf_cap - n_big;
     int skip_upto = 0;
     if (K <= 64) {
+        used |= kBucketKernelMedium;
         if (launch_bucket_knn_medium(points, D, K, ids, starts + off, sizes + off, n_big, 0, rows_sorted, knn_idx, knn_dist, stream))
             return 1;
         if (max_bucket >= 0 && max_bucket <= medium_bucket_cap()) return 0;
         skip_upto = medium_bucket_cap();
         const int rows_cap = resident_rows_cap(D, K);
         if (rows_cap > skip_upto) {
+            used |= kBucketKernelRows;
             if (launch_bucket_knn_rows(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto + 1,
                                        max_bucket >= 0 ? std::min(max_bucket, rows_cap) : rows_cap, rows_sorted, young_rows, knn_idx,
                                        knn_dist, stream))
@@ -439,7 +448,7 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
         }
     }
     return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream,
-                          rows_sorted, max_bucket);
+                          rows_sorted, max_bucket, &used);
 }
 
 }  // namespace rsfk

@@ -198,7 +198,9 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                 const float S = nrm[m] + nn;
                 const float dt = __builtin_fmaf(-2.0f, g[i], S);
                 const float lower = (dt - __builtin_fmaf(c_err, S, 1e-35f)) * one_minus_gamma;
-                const bool drop = lower > fmaxf(M.tau[m], tn);                // false if anything is NaN
+                // a NaN bound never drops a pair (the comparison is false); a NaN last slot cannot occur: rows only
+                // hold what passed `distance < last slot`, +inf where they are empty
+                const bool drop = lower > fmaxf(M.tau[m], tn);
                 const bool valid = n < s && (qi == qj ? m < n : m < s);
                 if (valid && !drop) bits |= 1u << i;
             }

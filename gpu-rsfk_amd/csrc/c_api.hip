@@ -276,6 +276,8 @@ RSFK_API int rsfk_explore_host(const float* points, int N, int D, int num_neighb
 
 RSFK_API const char* rsfk_last_error(void) { return last_error(); }
 
+RSFK_API int rsfk_last_build_report(char* buf, int capacity) { return build_report_json(buf, capacity); }
+
 RSFK_API void rsfk_release_workspace(void)
 {
     ws_release_all();

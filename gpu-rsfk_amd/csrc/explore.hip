@@ -154,6 +154,13 @@ __device__ __forceinline__ void screen_consume(const ScreenLoads& S, const Explo
     }
 }
 
+// Count of the exact distances of a launch, for the report of a build: one addition per wavefront, to one of 256
+// slots a cache line apart (stat may be null).
+__device__ __forceinline__ void count_exact(unsigned long long* stat, int n)
+{
+    if (stat && n > 0 && lane_id() == 0) atomicAdd(&stat[32 * (blockIdx.x & 255)], (unsigned long long)n);
+}
+
 // Stages are numbered s = batch * nblk + block; list holds U candidates.
 struct ScreenCtx {
     const int* list;
@@ -163,7 +170,7 @@ struct ScreenCtx {
 template <int SL>
 __device__ __forceinline__ void screen_stage_finish(const ScreenCtx& C, const ExploreLds& L, const Bf16Copy& bf, int batch,
                                                     float da, float ta, KnnRow<SL>& row, int& queued2,
-                                                    const float* __restrict__ points, bool vec_ok)
+                                                    const float* __restrict__ points, bool vec_ok, int& n_exact)
 {
     const int lane = lane_id();
     const int n = min(64, C.U - batch * 64);
@@ -179,6 +186,7 @@ __device__ __forceinline__ void screen_stage_finish(const ScreenCtx& C, const Ex
     if (queued2 >= 64) {
         wave_lds_sync();
         exact_batch<SL>(L, L.queue2, 64, points, C.D, vec_ok, row);
+        n_exact += 64;
         const int rest = queued2 - 64;
         const int mv = lane < rest ? L.queue2[64 + lane] : 0;
         wave_lds_sync();
@@ -190,7 +198,7 @@ __device__ __forceinline__ void screen_stage_finish(const ScreenCtx& C, const Ex
 
 template <int SL>
 __device__ __forceinline__ void screen_all(const ScreenCtx& C, const ExploreLds& L, const Bf16Copy& bf, KnnRow<SL>& row,
-                                           int& queued2, const float* __restrict__ points, bool vec_ok)
+                                           int& queued2, const float* __restrict__ points, bool vec_ok, int& n_exact)
 {
     const int nb = (C.U + 63) >> 6;
     const int stages = nb * C.nblk;
@@ -204,7 +212,7 @@ __device__ __forceinline__ void screen_all(const ScreenCtx& C, const ExploreLds&
         const int batch = s / C.nblk, blk = s - batch * C.nblk;
         if (blk == 0) { da = 0.0f; ta = 0.0f; }
         screen_consume(S, L, C.Dv, blk * kBlockB, da, ta);
-        if (blk == C.nblk - 1) screen_stage_finish<SL>(C, L, bf, batch, da, ta, row, queued2, points, vec_ok);
+        if (blk == C.nblk - 1) screen_stage_finish<SL>(C, L, bf, batch, da, ta, row, queued2, points, vec_ok, n_exact);
     };
     if (stages > 0) issue(A, 0);
     for (int s = 0; s < stages; s += 2) {
@@ -222,7 +230,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
                                                          const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                          float* __restrict__ knn_dist, int table_size, int wave_lds_ints,
                                                          int dpad, int rows_per_group, const int* __restrict__ todo,
-                                                         int n_todo)
+                                                         int n_todo, unsigned long long* __restrict__ stat)
 {
     extern __shared__ __align__(16) int lds_i[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -253,6 +261,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
     C.D = D;
     C.nblk = (C.Dv + kBlockB - 1) / kBlockB;
     int queued2 = 0;                                       // wave-uniform
+    int n_exact = 0;                                       // exact distances of this point (wave-uniform)
 
     for (int i0 = 0; i0 < K; i0 += rows_per_group) {
         const int i1 = min(K, i0 + rows_per_group);
@@ -300,12 +309,13 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
         C.U = U;
         // ---- screen / exact ------------------------------------------------------------
         if (use_screen) {
-            screen_all<SL>(C, L, bf, row, queued2, points, vec_ok);
+            screen_all<SL>(C, L, bf, row, queued2, points, vec_ok, n_exact);
         } else {
             for (int off = 0; off < U; off += 64) {
                 wave_lds_sync();
                 exact_batch<SL>(L, L.table + off, min(64, U - off), points, D, vec_ok, row);
             }
+            n_exact += U;
         }
     }
     // drain the second queue (at most 127 entries)
@@ -313,6 +323,8 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore(const float* __restrict_
         wave_lds_sync();
         exact_batch<SL>(L, L.queue2 + off, min(64, queued2 - off), points, D, vec_ok, row);
     }
+    n_exact += queued2;
+    count_exact(stat, n_exact);
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
 
@@ -354,7 +366,8 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
                                                                const uint32_t* __restrict__ pass,
                                                                const uint16_t* __restrict__ bounds,
                                                                const int* __restrict__ todo_in, int n_in,
-                                                               int* __restrict__ todo_out, int* __restrict__ n_out)
+                                                               int* __restrict__ todo_out, int* __restrict__ n_out,
+                                                               unsigned long long* __restrict__ stat)
 {
     extern __shared__ __align__(16) int lds_m[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -465,7 +478,9 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
         U += __popcll(m);
     }
     wave_lds_sync();
+    int n_exact = 0;                                      // exact distances of this point (wave-uniform)
     auto batch = [&](const int* list, int n) {
+        n_exact += n;
         if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
         else exact_batch<SL, kMergeChunk, true>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
     };
@@ -513,6 +528,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
             wave_lds_sync();
         }
     }
+    count_exact(stat, n_exact);
     if (row.changed) row.store(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K);
 }
 
@@ -565,7 +581,8 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
                                                           const uint32_t* __restrict__ pass,
                                                           const uint16_t* __restrict__ bounds,
                                                           const int* __restrict__ todo_in, int n_in,
-                                                          int* __restrict__ todo_out, int* __restrict__ n_out)
+                                                          int* __restrict__ todo_out, int* __restrict__ n_out,
+                                                          unsigned long long* __restrict__ stat)
 {
     extern __shared__ __align__(16) int lds_w[];
     __shared__ int wave_tot[4];
@@ -666,9 +683,11 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     L.table = nullptr;
     L.srow = nullptr;
     int have = 0;                                                 // candidates waiting in ids (wave-uniform)
+    int n_exact = 0;                                              // exact distances this wavefront asked for
     auto run_batch = [&]() {
         wave_lds_sync();
         const int n_now = min(64, have);
+        n_exact += n_now;
         const float cap_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
         exact_batch<SL, kWgChunk, true>(L, ids, n_now, points, D, vec_ok, row, cap_now);
         if (lane == 0) atomicMin(&tau_s, __float_as_uint(row.tau));   // non-negative floats order like their bits
@@ -717,6 +736,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         prev = thr;
     }
     if (have > 0) run_batch();
+    count_exact(stat, n_exact);
 
     // ---- 3. one row out of four: wavefronts 0 and 1 take the rows of 2 and 3, then 0 takes the row of 1
     auto put_row = [&](int at) {
@@ -761,14 +781,14 @@ int merge_wg_ints(int cap, int dpad, int K, int sl)
 template <int SL>
 int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int cap,
                     int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
-                    int* todo_out, int* n_out, hipStream_t stream)
+                    int* todo_out, int* n_out, unsigned long long* stat, hipStream_t stream)
 {
     const size_t lds = (size_t)merge_wg_ints(cap, dpad, K, SL) * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge_wg<SL>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
     hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3((unsigned)n_work), dim3(256), lds, stream, points, N, D, K, old_idx,
-                       knn_idx, knn_dist, cap, dpad, pass, bounds, todo_in, n_in, todo_out, n_out);
+                       knn_idx, knn_dist, cap, dpad, pass, bounds, todo_in, n_in, todo_out, n_out, stat);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -783,7 +803,7 @@ int next_pow2(int v)
 template <int SL, int WAVES>
 int launch_merge(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
                  int wave_ints, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
-                 int* todo_out, int* n_out, hipStream_t stream)
+                 int* todo_out, int* n_out, unsigned long long* stat, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES>),
@@ -791,7 +811,7 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
     const int n_work = todo_in ? n_in : N;
     dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out);
+                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out, stat);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -805,13 +825,13 @@ int merge_wave_ints(int table, int dpad, int K, bool with_bounds = false)
 
 int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
                    float* knn_dist, int table, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in,
-                   int n_in, int* todo_out, int* n_out, hipStream_t stream)
+                   int n_in, int* todo_out, int* n_out, unsigned long long* stat, hipStream_t stream)
 {
     const int wi = merge_wave_ints(table, dpad, K, bounds != nullptr);
 #define RSFK_MERGE_CASE(SLV, WV)                                                                                        \
     if (sl == SLV && waves == WV)                                                                                       \
         return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, pass, bounds, \
-                                     todo_in, n_in, todo_out, n_out, stream);
+                                     todo_in, n_in, todo_out, n_out, stat, stream);
     RSFK_MERGE_CASE(1, 4) RSFK_MERGE_CASE(1, 2) RSFK_MERGE_CASE(1, 1)
     RSFK_MERGE_CASE(2, 4) RSFK_MERGE_CASE(2, 2) RSFK_MERGE_CASE(2, 1)
     RSFK_MERGE_CASE(4, 4) RSFK_MERGE_CASE(4, 2) RSFK_MERGE_CASE(4, 1)
@@ -822,7 +842,7 @@ int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, 
 template <int SL, int WAVES>
 int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, const int* old_idx, int* knn_idx,
                float* knn_dist, int table, int wave_ints, int dpad, int rows_per_group, const int* todo, int n_todo,
-               hipStream_t stream)
+               unsigned long long* stat, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore<SL, WAVES>),
@@ -830,7 +850,7 @@ int launch_one(const float* points, const Bf16Copy& b, int N, int D, int K, cons
     const int n_work = todo ? n_todo : N;
     dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore<SL, WAVES>), grid, block, lds, stream, points, b, N, D, K, old_idx, knn_idx, knn_dist,
-                       table, wave_ints, dpad, rows_per_group, todo, n_todo);
+                       table, wave_ints, dpad, rows_per_group, todo, n_todo, stat);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -880,7 +900,8 @@ bool explore_merge_fits(int D, int K)
 // the candidates come from the join over the reversed graph (explore_join.hip), which needs rows sorted by
 // distance.
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
-                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted)
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted,
+                   unsigned long long* stat)
 {
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
@@ -927,7 +948,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         const uint16_t* wave_bounds = explore_ws_bounds(ws);
         if (4 * merge_wave_ints(small_table, dpad, K, true) > lds_ints) wave_bounds = nullptr;
         if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, pass, wave_bounds, nullptr, 0,
-                           listA, listA + N, stream))
+                           listA, listA + N, stat, stream))
             return 1;
         RSFK_HIP(hipMemcpyAsync(host_n, listA + N, sizeof(int), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
@@ -947,16 +968,16 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
             int rc = 0;
             if (!per_wg)
                 rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, pass,
-                                    nullptr, listA, n_todo, listB, listB + N, stream);
+                                    nullptr, listA, n_todo, listB, listB + N, stat, stream);
             else if (sl == 1)
                 rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
-                                        n_todo, listB, listB + N, stream);
+                                        n_todo, listB, listB + N, stat, stream);
             else if (sl == 2)
                 rc = launch_merge_wg<2>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
-                                        n_todo, listB, listB + N, stream);
+                                        n_todo, listB, listB + N, stat, stream);
             else
                 rc = launch_merge_wg<4>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
-                                        n_todo, listB, listB + N, stream);
+                                        n_todo, listB, listB + N, stat, stream);
             if (rc)
                 return 1;
             RSFK_HIP(hipMemcpyAsync(host_n, listB + N, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -969,7 +990,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
 #define RSFK_EXPLORE_CASE(SLV, WV)                                                                                      \
     if (sl == SLV && waves == WV)                                                                                       \
         return launch_one<SLV, WV>(points, b, N, D, K, old_idx, knn_idx, knn_dist, table, wave_ints, dpad,              \
-                                   rows_per_group, todo, n_todo, stream);
+                                   rows_per_group, todo, n_todo, stat, stream);
     RSFK_EXPLORE_CASE(1, 4) RSFK_EXPLORE_CASE(1, 2) RSFK_EXPLORE_CASE(1, 1)
     RSFK_EXPLORE_CASE(2, 4) RSFK_EXPLORE_CASE(2, 2) RSFK_EXPLORE_CASE(2, 1)
     RSFK_EXPLORE_CASE(4, 4) RSFK_EXPLORE_CASE(4, 2) RSFK_EXPLORE_CASE(4, 1)

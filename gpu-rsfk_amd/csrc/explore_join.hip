@@ -610,9 +610,12 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
         return 1;
     }
     if (with_bounds) {
-        // 2 bytes per pair of the join; without them the merge still works, in the order of the marks
+        // 2 bytes per pair of the join; without them the merge still works, in the order of the marks.  The array grows
+        // with N K^2 (17 GB at N = 1M, K = 90): it is only asked for up to 16 GiB, and as a block the call can do
+        // without (no idle block is given up for it, a refusal leaves no error text behind)
+        const size_t bytes = total * w->MW * 32 * sizeof(uint16_t);
         void* b = nullptr;
-        if (ws_alloc(&b, total * w->MW * 32 * sizeof(uint16_t)) == 0) w->bounds = static_cast<uint16_t*>(b);
+        if (bytes <= ((size_t)16 << 30) && ws_try_alloc(&b, bytes) == 0) w->bounds = static_cast<uint16_t*>(b);
     }
     *out = w;
     return 0;

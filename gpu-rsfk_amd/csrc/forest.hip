@@ -36,6 +36,17 @@ const char* last_error()
 
 namespace {
 
+// the last build of this process (knn_forest_device), for build_report_json
+struct BuildReport {
+    int N = 0, D = 0, K = 0, n_trees = 0, passes = 0, row_bytes = 0, screen_from = 0;
+    std::vector<int> kernels;                          // per tree: kBucketKernel... bits
+    unsigned long long tested = 0, undecided = 0;      // tree build: point-levels, and those left to the exact test
+    unsigned long long exact = 0;                      // exploration: exact distances over all passes
+    double tree_s = 0.0, bucket_s = 0.0, explore_s = 0.0;
+};
+std::mutex g_report_mutex;
+BuildReport g_report;
+
 double now_s()
 {
     return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -129,6 +140,52 @@ int make_tree_screen(Q8Guard& q8, const float* d_points, int N, int D, int verbo
 
 }  // namespace
 
+int build_report_json(char* buf, int cap)
+{
+    BuildReport r;
+    {
+        std::lock_guard<std::mutex> lock(g_report_mutex);
+        r = g_report;
+    }
+    static const struct { int bit; const char* name; } names[] = {
+        {kBucketKernelSmall, "k_bucket_knn_small<64>"}, {kBucketKernelScreen, "k_bucket_knn_screen"},
+        {kBucketKernelMedium, "k_bucket_knn_small<72>"}, {kBucketKernelRows, "k_bucket_knn_rows"},
+        {kBucketKernelTiled, "k_bucket_knn<per bucket>"}, {kBucketKernelStrip, "k_bucket_knn<per 64 members>"},
+        {kBucketKernelGram, "k_bucket_knn_gram"}};
+    std::string s = "{";
+    auto num = [&](const char* key, double v, bool last = false) {
+        char t[96];
+        std::snprintf(t, sizeof t, "\"%s\": %.9g%s", key, v, last ? "" : ", ");
+        s += t;
+    };
+    num("N", r.N); num("D", r.D); num("K", r.K); num("n_trees", r.n_trees);
+    // runs of trees that went to the same kernels: [first tree, last tree, [names]]
+    s += "\"bucket_kernels\": [";
+    for (size_t a = 0; a < r.kernels.size();) {
+        size_t b = a;
+        while (b + 1 < r.kernels.size() && r.kernels[b + 1] == r.kernels[a]) ++b;
+        if (a) s += ", ";
+        s += "[" + std::to_string(a) + ", " + std::to_string(b) + ", [";
+        bool first = true;
+        for (const auto& nm : names)
+            if (r.kernels[a] & nm.bit) { s += std::string(first ? "\"" : ", \"") + nm.name + "\""; first = false; }
+        s += "]]";
+        a = b + 1;
+    }
+    s += "], ";
+    num("tree_points_tested", (double)r.tested); num("tree_points_undecided", (double)r.undecided);
+    num("tree_screen_row_bytes", r.row_bytes); num("tree_seconds", r.tree_s); num("bucket_seconds", r.bucket_s);
+    num("explore_passes", r.passes); num("explore_exact_distances", (double)r.exact);
+    num("explore_seconds", r.explore_s, true);
+    s += "}";
+    if (buf && cap > 0) {
+        const size_t n = std::min(s.size(), (size_t)cap - 1);
+        std::memcpy(buf, s.data(), n);
+        buf[n] = 0;
+    }
+    return (int)s.size();
+}
+
 int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MAX_DEPTH, int verbose, int seed,
                       int nnef, const float* d_points, int* d_idx, float* d_dist, float* log_forest,
                       hipStream_t stream)
@@ -140,6 +197,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (n_trees == 0 && nnef <= 0) return 0;          // nothing to do: no copies are made, nothing is queued
     const double t_forest0 = now_s();
     const int screen_from = bucket_screen_from(D, K);
+    BuildReport rep;
+    rep.N = N; rep.D = D; rep.K = K; rep.n_trees = n_trees; rep.passes = std::max(nnef, 0); rep.screen_from = screen_from;
+    rep.kernels.assign((size_t)n_trees, 0);
 
     Q8Guard q8;
     const uint8_t* q8_rows = nullptr;
@@ -152,6 +212,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     Bf16Guard bf;
     if (plain_copy && (bf16_copy_alloc(&bf.c, N, D) || bf16_copy_fill(bf.c, d_points, N, D, stream))) return 1;
 
+    rep.row_bytes = tree_screen_row_bytes(D, q8_rows != nullptr);
     if (n_trees > 0) {
         // the bucket kernels read a row's maximum from its last slot: rows the caller passed in unsorted are put
         // in order once
@@ -176,6 +237,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             rc = build_tree_batch(ws.w, d_points, bf.c.rows, q8_rows, N, D, MIN, MAX, MAX_DEPTH, seed + t0, nb, stats.data(), stream);
             if (rc) break;
             const double tb = now_s() - tb0;
+            rep.tree_s += tb;
+            rep.tested += tree_ws_counts(ws.w)[0];
+            rep.undecided += tree_ws_counts(ws.w)[1];
             // The larger buckets of a tree (a few per cent of the points at the default sizes: a grid too small to fill
             // the device) run on a second stream beside the small ones: different buckets of one tree touch different
             // rows.  Both parts of tree j wait for both parts of tree j - 1.
@@ -189,11 +253,12 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 const bool gram = t0 + j >= gram_from;
                 rc = launch_bucket_knn_tree(d_points, t0 + j >= screen_from, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
-                                            d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees);
+                                            d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees, &rep.kernels[(size_t)(t0 + j)]);
                 if (!rc && split) {
                     rc = launch_bucket_knn_tree(d_points, false, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
-                                                stats[5 * j + 2], d_idx, d_dist, sync.side, 2, t0 + j < kYoungTrees);
+                                                stats[5 * j + 2], d_idx, d_dist, sync.side, 2, t0 + j < kYoungTrees,
+                                                &rep.kernels[(size_t)(t0 + j)]);
                     (void)hipEventRecord(sync.big, sync.side);
                 }
                 big_pending = split;
@@ -205,6 +270,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             for (int j = 0; j < nb; ++j) {
                 float ms = 0.0f;
                 (void)hipEventElapsedTime(&ms, ev[j].e, ev[j + 1].e);
+                rep.bucket_s += ms * 1e-3;
                 const int t = t0 + j;
                 if (log_forest) {
                     log_forest[(size_t)0 * n_trees + t] = (float)stats[5 * j + 1];   // Tree Depth
@@ -236,6 +302,9 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         if (ws_alloc(&old.p, sizeof(int) * (size_t)N * (size_t)K)) return 1;
         ExploreWsGuard ews;      // without a workspace every point enumerates its own candidates
         Bf16Guard bfc;           // centred copy for the join
+        DevBuf stat;             // count of the exact distances (for the report)
+        if (ws_alloc(&stat.p, sizeof(unsigned long long) * kExploreStatWords)) return 1;
+        RSFK_HIP(hipMemsetAsync(stat.p, 0, sizeof(unsigned long long) * kExploreStatWords, stream));
         if (explore_join_enabled(N, K)) {
             if (explore_ws_alloc(&ews.w, N, K, explore_join_keeps_bounds(N, D, K))) return 1;
             if (bf16_copy_alloc(&bfc.c, N, D, true) || bf16_copy_fill(bfc.c, d_points, N, D, stream)) return 1;
@@ -243,16 +312,24 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         for (int it = 0; it < nnef; ++it) {
             // (the bucket step of the forest, and every exploration pass, leave all rows in order)
             if (launch_explore(d_points, plain_copy ? &bf.c : nullptr, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream,
-                               n_trees > 0 || it > 0))
+                               n_trees > 0 || it > 0, static_cast<unsigned long long*>(stat.p)))
                 return 1;
         }
+        std::vector<unsigned long long> h_stat((size_t)kExploreStatWords);
+        RSFK_HIP(hipMemcpyAsync(h_stat.data(), stat.p, sizeof(unsigned long long) * kExploreStatWords, hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
+        for (int i = 0; i < kExploreStatWords; i += 32) rep.exact += h_stat[(size_t)i];
     }
     const double t_exp = now_s() - t_exp0;
     if (verbose >= 1) std::printf("Nearest Neighbors Exploring computation Kernel takes %lf seconds\n", t_exp);
     if (log_forest) {
         log_forest[(size_t)16 * n_trees] = (float)t_forest;
         log_forest[(size_t)16 * n_trees + 1] = (float)t_exp;
+    }
+    rep.explore_s = t_exp;
+    {
+        std::lock_guard<std::mutex> lock(g_report_mutex);
+        g_report = std::move(rep);
     }
     return 0;
 }

@@ -20,6 +20,8 @@ const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
 int tree_small_threshold();
 const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w);
+const unsigned long long* tree_ws_counts(const TreeBatchWorkspace* w);
+int tree_screen_row_bytes(int D, bool q8);
 int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t* pb16, const uint8_t* q8, int N, int D,
                      int MIN, int MAX,
                      int MAX_DEPTH, int seed0, int nb, int* host_stats, hipStream_t stream);
@@ -36,9 +38,26 @@ int launch_bucket_knn_gram(const float* points, int D, int K, const int* ids, co
 // trees from this index on take the kernel that screens the pair matrix on the matrix cores (RSFK_GRAM_FROM)
 int bucket_gram_from();
 
+// Kernels a tree's buckets can go to (bits of *launched of launch_bucket_knn_tree, and of the report of a build)
+enum : int {
+    kBucketKernelSmall = 1,      // k_bucket_knn_small<64>: two wavefronts per bucket of up to 64 points, every pair exact
+    kBucketKernelScreen = 2,     // k_bucket_knn_screen: the same with the pair matrix bounded on the matrix cores first
+    kBucketKernelMedium = 4,     // k_bucket_knn_small<72>: three wavefronts, buckets of 65..72 points
+    kBucketKernelRows = 8,       // k_bucket_knn_rows: a bucket's points resident in LDS
+    kBucketKernelTiled = 16,     // k_bucket_knn<SL, false>: 64 x 64 tiles, a workgroup per bucket
+    kBucketKernelStrip = 32,     // k_bucket_knn<SL, true>: 64 x 64 tiles, a workgroup per 64 members of a bucket
+    kBucketKernelGram = 64,      // k_bucket_knn_gram: any bucket size, pair matrix bounded on the matrix cores
+};
 int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
                            const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0, bool young_rows = true);
+                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0, bool young_rows = true,
+                           int* launched = nullptr);
+
+// What the last K-NN-graph build of this process did, as a line of JSON (rsfk_last_build_report): which bucket
+// kernels every tree went to, the counts the algorithmic bytes of the tree build and of the exploration are made of,
+// and the time of each of the three steps.  Returns the length of the text (without the final zero), which is
+// truncated to cap - 1 characters.
+int build_report_json(char* buf, int cap);
 
 // bucket_knn_screen.hip
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);
@@ -86,7 +105,9 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
 bool explore_merge_uses_bounds(int D, int K);
 bool explore_join_keeps_bounds(int N, int D, int K);
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
-                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted = false);
+                   float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted = false,
+                   unsigned long long* stat = nullptr);      // stat: kExploreStatWords words, or null (count_exact)
+constexpr int kExploreStatWords = 32 * 256;
 
 // graph_export.hip
 int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int drop_self, int* d_indptr, int* d_cols,

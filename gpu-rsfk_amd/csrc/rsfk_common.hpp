@@ -17,6 +17,7 @@ const char* last_error();
 
 // workspace.hip: device memory for working buffers, kept for the next call after use
 int ws_alloc(void** out, size_t bytes);
+int ws_try_alloc(void** out, size_t bytes);      // optional block: fails quietly, releases nothing
 void ws_free(void* p);
 void ws_release_all();
 

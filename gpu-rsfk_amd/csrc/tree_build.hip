@@ -55,6 +55,15 @@ struct LevelCounters {
     long long phase_ticks[3];
 };
 
+// Counts for the report of a build (how many points the side tests of all levels looked at, and how many of them
+// the screen left to the exact test): kStatSlots slots a cache line apart, so that the workgroups' additions do not
+// all go to one address; slot s holds [points, undecided points] at stat[kStatPitch * s + 0 / 1].
+constexpr int kStatSlots = 64, kStatPitch = 32;
+__device__ __forceinline__ void stat_add(unsigned long long* stat, int slot, int which, int v)
+{
+    if (stat && v) atomicAdd(&stat[kStatPitch * (slot & (kStatSlots - 1)) + which], (unsigned long long)v);
+}
+
 // ended: the step that ends where the calling kernel begins (-1: none, the clock is only started)
 __device__ __forceinline__ void phase_tick(LevelCounters* ctr, int ended)
 {
@@ -407,7 +416,8 @@ __global__ void k_init_roots(TreeNode* nodes, TreeNode* tail, LevelCounters* ctr
 
 // chunk_base[i] = number of chunks of nodes [0,i); one workgroup.
 __global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict__ nodes, int node_cap, int chunk,
-                                                      int* __restrict__ chunk_base, LevelCounters* ctr)
+                                                      int* __restrict__ chunk_base, LevelCounters* ctr,
+                                                      unsigned long long* __restrict__ stat)
 {
     __shared__ int wsum[16];
     __shared__ int carry_s;
@@ -418,9 +428,12 @@ __global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict
         phase_tick(ctr, 2);
     }
     __syncthreads();
+    int members = 0;                                      // points of the nodes this thread looked at
     for (int base = 0; base < n_nodes; base += 1024) {
         const int i = base + tid;
-        const int v = i < n_nodes ? (nodes[i].count + chunk - 1) / chunk : 0;
+        const int cnt_i = i < n_nodes ? nodes[i].count : 0;
+        members += cnt_i;
+        const int v = (cnt_i + chunk - 1) / chunk;
         // inclusive scan inside the wavefront
         int x = v;
 #pragma unroll
@@ -439,6 +452,8 @@ __global__ __launch_bounds__(1024) void k_scan_chunks(const TreeNode* __restrict
         __syncthreads();
     }
     if (tid == 0) { chunk_base[n_nodes] = carry_s; ctr->n_chunks = carry_s; }
+    members = wave_sum_i(members);
+    if (lane == 0) stat_add(stat, wave, 0, members);
 }
 
 // (also empties the queue of the level being produced, which the scatter kernel of this level fills)
@@ -496,7 +511,7 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
                                                  int* __restrict__ perm0, int* __restrict__ perm1,
                                                  const TreeNode* __restrict__ nodes, const int* __restrict__ chunk_base,
                                                  const int* __restrict__ chunk2node, int* __restrict__ chunk_left,
-                                                 const float* __restrict__ planes)
+                                                 const float* __restrict__ planes, unsigned long long* __restrict__ stat)
 {
     extern __shared__ __align__(16) float side_lds[];      // record of the node's hyperplane (k_level_planes)
     float* hp_s = side_lds;                                 // offset, bound of the 1-norm, sum of the components
@@ -559,7 +574,10 @@ __global__ __launch_bounds__(kBlock) void k_side(const float* __restrict__ point
                   });
     if (lefts) atomicAdd(&left_s, lefts);
     __syncthreads();
-    if (threadIdx.x == 0) chunk_left[c] = left_s;
+    if (threadIdx.x == 0) {
+        chunk_left[c] = left_s;
+        stat_add(stat, c, 1, n_def_s);
+    }
 }
 
 // Stable scatter of one chunk into the other permutation buffer; the workgroup
@@ -764,7 +782,8 @@ __global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
                                                  const TreeNode* __restrict__ tasks, int n_tasks, int node_cap, int G,
                                                  int leaf_cap, int* __restrict__ leaf_start, int* __restrict__ leaf_size,
                                                  TreeStats* stats, LevelCounters* ctr,
-                                                 TreeRec* __restrict__ recs_all, int* __restrict__ n_rec_all, int rec_cap)
+                                                 TreeRec* __restrict__ recs_all, int* __restrict__ n_rec_all, int rec_cap,
+                                                 unsigned long long* __restrict__ stat)
 {
     // dynamic LDS: seg[small] | tmp[small] | nvec[G][nvec_len(D)] | lrec[node_cap] | level lists 2 x node_cap | fmap[small]
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -781,6 +800,7 @@ __global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
     __shared__ float b_s[kMaxGroup], hp_s[kMaxGroup][3];
     __shared__ int left_s[kMaxGroup], pre_s[kMaxGroup + 1], start_s[kMaxGroup], pair_s[kMaxGroup][2];
     __shared__ int n_cur_s, n_nxt_s, nrec_s, kind_s[2], base_s[2], lev_s, mx_s, mn_s, n_def_s;
+    __shared__ int seen_s, unsure_s;        // points tested over all levels of the subtree, and left to the exact test
 
     const int task = blockIdx.x;
     if (task >= n_tasks) return;
@@ -809,6 +829,7 @@ __global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
         r.depth = tk.depth; r.leaf = 0; r.key = tk.key; r.rec = tk.rec; r.pad_ = 0;
         cur[0] = r;
         n_cur_s = 1; n_nxt_s = 0; nrec_s = 0; kind_s[0] = 0; kind_s[1] = 0; lev_s = 0; mx_s = 0; mn_s = 0x7fffffff;
+        seen_s = 0; unsure_s = 0;
     }
     __syncthreads();
 
@@ -883,6 +904,7 @@ __global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
                 }
             }
             __syncthreads();
+            if (tid == 0) { seen_s += total; unsure_s += n_def_s; }
             resolve_exact(tmp, n_def_s, nvec, Dv, b_s, points, P.D, [&](int pos) { return seg[pos] & kIdMask; },
                           [&](int pos, bool right) { if (right) seg[pos] |= (int)0x80000000; });
             __syncthreads();
@@ -945,6 +967,8 @@ __global__ __launch_bounds__(TB) void k_tail(const float* __restrict__ points,
         atomicMax(&st->levels, lev_s);
         atomicMax(&st->max_leaf, mx_s);
         atomicMin(&st->min_leaf, mn_s);
+        stat_add(stat, task, 0, seen_s);
+        stat_add(stat, task, 1, unsure_s);
     }
     __syncthreads();
     const int nrec = min(nrec_s, node_cap);
@@ -983,6 +1007,9 @@ struct TreeBatchWorkspace {
     int D = 0;
     LevelCounters* h_ctr = nullptr;      // pinned
     TreeStats* h_stats = nullptr;        // pinned
+    unsigned long long* stat = nullptr;  // kStatSlots x kStatPitch: counts for the report (stat_add)
+    unsigned long long* h_stat = nullptr;        // pinned
+    unsigned long long counts[2] = {0, 0};       // of the last batch: points the side tests looked at, undecided ones
     // index of the trees for routing query points (allocated by tree_ws_enable_index)
     TreeRec* recs = nullptr;             // B x rec_cap
     int* n_rec = nullptr;                // B
@@ -1007,9 +1034,10 @@ static void free_ws(TreeBatchWorkspace& w)
 {
     void* dev[] = {w.perm[0], w.perm[1], w.nodes[0], w.nodes[1], w.tail, w.chunk_base, w.chunk2node,
                    w.chunk_left, w.leaf_start, w.leaf_size, w.stats, w.ctr, w.recs, w.n_rec, w.planes,
-                   w.pm_path, w.pm_side, w.pm_undec, w.pm_map[0], w.pm_map[1], w.pm_sc, w.pm_aq, w.pm_child};
+                   w.pm_path, w.pm_side, w.pm_undec, w.pm_map[0], w.pm_map[1], w.pm_sc, w.pm_aq, w.pm_child, w.stat};
     for (void* p : dev) ws_free(p);
     if (w.h_ctr) (void)hipHostFree(w.h_ctr);
+    if (w.h_stat) (void)hipHostFree(w.h_stat);
     if (w.h_stats) (void)hipHostFree(w.h_stats);
     for (hipEvent_t e : w.ev)
         if (e) (void)hipEventDestroy(e);
@@ -1077,6 +1105,7 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     if (dmalloc(&w->leaf_size, (size_t)B * w->leaf_cap)) return 1;
     if (dmalloc(&w->stats, (size_t)B)) return 1;
     if (dmalloc(&w->ctr, (size_t)1)) return 1;
+    if (dmalloc(&w->stat, (size_t)kStatSlots * kStatPitch)) return 1;
     if (D <= 256 && N > small && B <= 64) {
         w->pm_ks = D <= 32 ? 1 : D <= 64 ? 2 : D <= 128 ? 4 : 8;
         w->pm_W = 2 * ((N + 63) / 64);                     // an even number of 32-point tiles
@@ -1092,12 +1121,18 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     }
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_ctr), sizeof(LevelCounters)));
     RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stats), sizeof(TreeStats) * (size_t)B));
+    RSFK_HIP(hipHostMalloc(reinterpret_cast<void**>(&w->h_stat), sizeof(unsigned long long) * kStatSlots * kStatPitch));
     for (hipEvent_t& e : w->ev) RSFK_HIP(hipEventCreate(&e));
     return 0;
 }
 
 // seconds the last batch spent in: side tests, hyperplanes of the wide levels, scatter, tail kernel
 const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w) { return w->phase_s; }
+// of the last batch: [0] points the side tests of all levels and trees looked at (the sum over the levels of the
+// members of the nodes that were split), [1] those the screen left to the exact fp32 test
+const unsigned long long* tree_ws_counts(const TreeBatchWorkspace* w) { return w->counts; }
+// bytes of a row of the copy the side tests are screened on
+int tree_screen_row_bytes(int D, bool q8) { return q8 ? q8_pitch(D) : 2 * bf16_pitch(D); }
 
 // Builds nb (<= B) trees with seeds seed0 .. seed0+nb-1.  pb16 = rows of the bfloat16 copy of the points (may be
 // null: every side test then reads the fp32 row).  On return perm[0] of
@@ -1129,6 +1164,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     std::memcpy(w->h_stats, init.data(), sizeof(TreeStats) * (size_t)nb);
     RSFK_HIP(hipMemcpyAsync(w->stats, w->h_stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyHostToDevice, stream));
     RSFK_HIP(hipMemsetAsync(w->ctr, 0, sizeof(LevelCounters), stream));
+    RSFK_HIP(hipMemsetAsync(w->stat, 0, sizeof(unsigned long long) * kStatSlots * kStatPitch, stream));
     // Levels whose side tests are taken point by point (needs the 8-bit copy).  RSFK_PM_LEVELS overrides (0 = none).
     // The sweep multiplies every tile of points with every block of 16 hyperplanes of a tree, so its cost doubles
     // per level from the fifth on; measured, the seventh level is the last one it takes faster than k_side.
@@ -1163,7 +1199,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     while (true) {
         // one trip to the host per level: the chunk table of the level is made first (from the node count on the
         // device), then both counts come back together
-        hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], w->node_cap, P.chunk, w->chunk_base, w->ctr);
+        hipLaunchKernelGGL(k_scan_chunks, dim3(1), dim3(1024), 0, stream, w->nodes[cur], w->node_cap, P.chunk, w->chunk_base, w->ctr,
+                           w->stat);
         RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
         RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
@@ -1196,7 +1233,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
 #undef RSFK_SWEEP_LAUNCH
             const size_t words = (size_t)nb * W;
             hipLaunchKernelGGL(pm::k_pm_resolve, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, points, D, W,
-                               w->pm_Bs, words, w->pm_path, w->pm_sc, w->planes, rec, w->pm_side, w->pm_undec);
+                               w->pm_Bs, words, w->pm_path, w->pm_sc, w->planes, rec, w->pm_side, w->pm_undec, w->stat);
             hipLaunchKernelGGL(k_pm_mark, dim3(n_chunks), dim3(kBlock), 0, stream, P, w->perm[0], w->perm[1], w->nodes[cur],
                                w->chunk_base, w->chunk2node, w->chunk_left, w->pm_side, W);
         } else {
@@ -1204,7 +1241,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         const int q8_pieces = q8_padded(D) >> 4;
 #define RSFK_SIDE_LAUNCH(Q, L)                                                                                              \
         hipLaunchKernelGGL((k_side<Q, L>), dim3(n_chunks), dim3(kBlock), side_lds, stream, points, pb16, q8, P, w->perm[0],    \
-                           w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes)
+                           w->perm[1], w->nodes[cur], w->chunk_base, w->chunk2node, w->chunk_left, w->planes, w->stat)
         if (!q8) RSFK_SIDE_LAUNCH(false, 8);
         else if (q8_pieces <= 2) RSFK_SIDE_LAUNCH(true, 2);
         else if (q8_pieces <= 4) RSFK_SIDE_LAUNCH(true, 4);
@@ -1248,7 +1285,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                          \
             hipLaunchKernelGGL((k_tail<Q, T>), dim3(n_tail), dim3(T), lds, stream, points, pb16, q8, P, w->perm[0],         \
                                w->perm[1], w->perm[0], w->tail, n_tail, node_cap, G, w->leaf_cap, w->leaf_start,            \
-                               w->leaf_size, w->stats, w->ctr, w->recs, w->n_rec, w->rec_cap);                             \
+                               w->leaf_size, w->stats, w->ctr, w->recs, w->n_rec, w->rec_cap, w->stat);                    \
         } while (0)
         if (tail_q8 && wide_wg) RSFK_TAIL_LAUNCH(true, 1024);
         else if (tail_q8) RSFK_TAIL_LAUNCH(true, 256);
@@ -1260,7 +1297,13 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     }
     RSFK_HIP(hipMemcpyAsync(w->h_stats, w->stats, sizeof(TreeStats) * (size_t)nb, hipMemcpyDeviceToHost, stream));
     RSFK_HIP(hipMemcpyAsync(w->h_ctr, w->ctr, sizeof(LevelCounters), hipMemcpyDeviceToHost, stream));
+    RSFK_HIP(hipMemcpyAsync(w->h_stat, w->stat, sizeof(unsigned long long) * kStatSlots * kStatPitch, hipMemcpyDeviceToHost, stream));
     RSFK_HIP(hipStreamSynchronize(stream));
+    w->counts[0] = w->counts[1] = 0;
+    for (int sl = 0; sl < kStatSlots; ++sl) {
+        w->counts[0] += w->h_stat[kStatPitch * sl];
+        w->counts[1] += w->h_stat[kStatPitch * sl + 1];
+    }
     if (n_tail > 0) {
         float ms = 0.0f;
         if (hipEventElapsedTime(&ms, w->ev[0], w->ev[1]) == hipSuccess) w->phase_s[3] = ms * 1e-3f;

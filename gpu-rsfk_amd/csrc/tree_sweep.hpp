@@ -357,7 +357,8 @@ __global__ __launch_bounds__(256) void k_pm_resolve(const float* __restrict__ po
                                                     size_t total_words, const uint8_t* __restrict__ path,
                                                     const PlaneQ* __restrict__ sc, const float* __restrict__ planes,
                                                     int rec, uint32_t* __restrict__ sidebits,
-                                                    const uint32_t* __restrict__ undec)
+                                                    const uint32_t* __restrict__ undec,
+                                                    unsigned long long* __restrict__ stat)
 {
     __shared__ uint16_t list_s[4][2048];
     __shared__ int e_ni[4][64], e_pt[4][64];
@@ -371,6 +372,8 @@ __global__ __launch_bounds__(256) void k_pm_resolve(const float* __restrict__ po
     const int off = wave_excl_scan_i(cnt);
     const int total = read_lane_i(off + cnt, 63);
     if (total == 0) return;
+    // (count of the points left to the exact test, for the report of a build: slots a cache line apart)
+    if (stat && lane == 0) atomicAdd(&stat[32 * (blockIdx.x & 63) + 1], (unsigned long long)total);
     uint16_t* list = list_s[wave];
     {
         uint32_t w = bits;

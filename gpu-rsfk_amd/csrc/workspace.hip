@@ -48,7 +48,10 @@ Pool& pool()
 
 }  // namespace
 
-int ws_alloc(void** out, size_t bytes)
+namespace {
+// must: a block the caller cannot do without (idle blocks are given back to make room, the error text is set);
+// otherwise one plain attempt that leaves the pool and the error text alone
+int ws_alloc_impl(void** out, size_t bytes, bool must)
 {
     *out = nullptr;
     if (bytes == 0) bytes = 1;
@@ -69,6 +72,10 @@ int ws_alloc(void** out, size_t bytes)
     }
     void* p = nullptr;
     hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess && !must) {
+        (void)hipGetLastError();
+        return 1;
+    }
     if (e != hipSuccess) {
         // give the idle blocks back and try once more
         (void)hipGetLastError();
@@ -85,6 +92,13 @@ int ws_alloc(void** out, size_t bytes)
     *out = p;
     return 0;
 }
+}  // namespace
+
+int ws_alloc(void** out, size_t bytes) { return ws_alloc_impl(out, bytes, true); }
+
+// A block the caller can do without (it only makes something faster): nonzero, with nothing else changed, when the
+// device does not have the room.
+int ws_try_alloc(void** out, size_t bytes) { return ws_alloc_impl(out, bytes, false); }
 
 // The caller has made sure that no work that uses the block is still running.
 void ws_free(void* p)

@@ -30,6 +30,7 @@ SYMBOLS = {
     "rsfk_bucket_knn_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _ci, _vp, _i32, _ci, _ci, _i32, _f32]),
     "rsfk_explore_host": (_ci, [_f32, _ci, _ci, _ci, _i32, _f32, _ci]),
     "rsfk_last_error": (ctypes.c_char_p, []),
+    "rsfk_last_build_report": (_ci, [ctypes.c_char_p, _ci]),
     "rsfk_device_count": (_ci, []),
     "rsfk_release_workspace": (None, []),
 }
@@ -148,6 +149,14 @@ def symmetrize_device(d_idx, d_dist, N, K, drop_self, d_indptr, d_cols, d_vals, 
                                         _vp(d_indptr), _vp(d_cols) if d_cols else None, _vp(d_vals) if d_vals else None,
                                         int(capacity), ctypes.byref(nnz), _vp(stream)))
     return int(nnz.value)
+
+
+def last_build_report():
+    """What the last K-NN-graph build of this process did (kernels per tree, counts, seconds) as a dict."""
+    import json
+    buf = ctypes.create_string_buffer(1 << 16)
+    lib().rsfk_last_build_report(buf, len(buf))
+    return json.loads(buf.value.decode())
 
 
 def symmetrize_count_noalloc(d_idx, N, K, drop_self, d_indptr, stream=0, fetch_count=True):

@@ -170,6 +170,16 @@ int rsfk_explore_host(const float* points, int N, int D, int num_neighbors,
 /* text of the last error of a call that returned non-zero */
 const char* rsfk_last_error(void);
 
+/* What the last K-NN-graph build of this process did (pymodule_rsfk_knn, rsfk_knn_forest_device, ...), as one line
+ * of JSON written to buf (at most capacity - 1 characters and a final zero); returns the length of the whole text.
+ * Keys: "bucket_kernels" (runs of trees [first, last, [kernel names]] -- which kernels the buckets of those trees
+ * went to), "tree_points_tested" (sum over all trees and levels of the members of the nodes that were split),
+ * "tree_points_undecided" (those the low-precision screen left to the exact fp32 test), "tree_screen_row_bytes",
+ * "explore_exact_distances" (exact distances of all exploration passes), and the seconds of the three steps.  The
+ * reference prints its phase times (src/rsfk.cu:1164-1176) and has no counterpart for the counts; bench.py computes
+ * the algorithmic bytes of the tree build and of the exploration from them. */
+int rsfk_last_build_report(char* buf, int capacity);
+
 /* The library keeps the device buffers of a call (permutations, screening copies, exploration workspace) for the
  * next call instead of returning them to the driver; this returns all idle ones.  No counterpart in the
  * reference, which allocates and frees inside every tree level (src/rsfk.cu:640-1180). */
