@@ -355,8 +355,8 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
     int skip_upto = 0;
     if (K <= 64) {
         // buckets of up to 72 points go to the specialised kernels; the general one skips them
-        if (bucket_screen_from(D, K) == 0) {
-            // RSFK_BUCKET_SCREEN=0: the screened kernel for every call; it needs sorted rows
+        if (bucket_screen_share_q16() == kScreenAlways) {
+            // RSFK_BUCKET_SCREEN=always: the screened kernel for every call; it needs sorted rows
             if (launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
             if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_buckets, stride, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_buckets, stride, false, knn_idx, knn_dist, stream))
@@ -382,13 +382,15 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
 // (starts, sizes), n_big larger ones at the back of the table of leaf_cap entries.  rows_sorted: every K-NN row is
-// known to be sorted by distance.  screen: the small buckets go to the kernel that bounds the pair matrix on the matrix
-// cores first (needs sorted rows, K <= 64).  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
+// known to be sorted by distance.  stats (8 zeroed words; with K <= 64 and sorted rows): the small buckets go to the
+// kernel that chooses between the direct and the screened form from the pairs of the tree before (prev_stats, null for
+// the first tree) and leaves its own numbers in stats.  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
 // kinds touch different rows, so the two parts of one tree may run side by side).  young_rows: the rows may be new or
 // far from done (first trees of a build).
-int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
-                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part, bool young_rows, int* launched)
+int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_stats, unsigned long long* stats,
+                           bool rows_sorted, bool gram, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int leaf_cap, int n_small, int n_big, int max_bucket, int* knn_idx, float* knn_dist,
+                           hipStream_t stream, int part, bool young_rows, int* launched)
 {
     RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
@@ -415,9 +417,10 @@ int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, b
                                       stream);
     }
     if (n_small > 0 && part != 2) {
-        if (K <= 64 && screen && rows_sorted) {
-            used |= kBucketKernelScreen;
-            if (launch_bucket_knn_screen(points, D, K, ids, starts, sizes, n_small, 0, knn_idx, knn_dist, stream)) return 1;
+        if (K <= 64 && stats && rows_sorted) {
+            used |= kBucketKernelAuto;
+            if (launch_bucket_knn_auto(points, D, K, ids, starts, sizes, n_small, knn_idx, knn_dist, prev_stats, stats, stream))
+                return 1;
         } else if (K <= 64) {
             used |= kBucketKernelSmall;
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;

@@ -37,6 +37,7 @@
 #include "knn_list.hpp"
 #include "forest.hpp"
 #include "mfma_split.hpp"
+#include "bucket_small_body.hpp"
 #include <algorithm>
 #include <cstdlib>
 
@@ -51,7 +52,10 @@ constexpr int kDistPitch = kCap + 1;
 constexpr int kChunk = 64;                 // dimensions staged at once (a multiple of 16)
 constexpr int kMaxPairs = kCap * (kCap - 1) / 2;
 constexpr int kMaxRounds = (kMaxPairs + kThreads - 1) / kThreads;     // listed pairs per thread
-constexpr int kListSlots = (kMaxPairs + 7) & ~7;
+// Pairs the list holds.  A bucket with more pairs to evaluate (nearly half of those of a full bucket: the first trees
+// of a build) evaluates all its pairs, which then need no list.  With this size the workgroup's LDS is 20 KB and eight
+// workgroups share a compute unit.
+constexpr int kListCap = 880;
 
 // LDS after the row / distance region: ids, last slots, flags, norms as seen by either wavefront, pair counter, list
 struct ScreenMeta {
@@ -60,7 +64,7 @@ struct ScreenMeta {
     int flag[kCap];
     float nrm[2][kCap];
     int n_pairs[4];
-    uint16_t list[kListSlots];
+    uint16_t list[kListCap];
 };
 
 // The rows of the bucket on their way from HBM to LDS: 16 lanes (a quarter wavefront) per row, a lane moves 16 bytes
@@ -105,21 +109,28 @@ struct RowLoads {
     }
 };
 
-// SINGLE: D <= kChunk, the rows are staged once and stay in LDS until the exact chains have run.
+// SINGLE: D <= kChunk, the rows are staged once and stay in LDS until the exact chains have run.  Otherwise the Gram
+// pass takes the chunks from the last to the first, so that the first one is still in LDS when the exact chains --
+// which must run from dimension 0 upwards -- begin; only the chunks after it pass through LDS a second time, and the
+// first of those is requested before the bounds are evaluated.
+// stats (may be null): the workgroups whose number is a multiple of 2^stat_shift add pairs of the bucket << 32 | pairs
+// that got an exact distance to one of its 8 words (a sample of the buckets, see small_bucket_body).
+// The work of one workgroup on bucket blockIdx.x; lds: kScreenLdsBytes bytes of LDS.
+constexpr int kPitch = kChunk + 4;                        // an odd number of 16-byte units: rows start in different banks
+constexpr int kRegion = kCap * kPitch > kCap * kDistPitch ? kCap * kPitch : kCap * kDistPitch;
+constexpr size_t kScreenLdsBytes = sizeof(float) * kRegion + sizeof(ScreenMeta);
+static_assert(kScreenLdsBytes <= 160 * 1024 / 8, "eight workgroups per compute unit");
+
 template <bool SINGLE>
-__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* __restrict__ points, int D, int K,
-                                                                   const int* __restrict__ ids,
-                                                                   const int* __restrict__ starts,
-                                                                   const int* __restrict__ sizes, int stride,
-                                                                   int* __restrict__ knn_idx, float* __restrict__ knn_dist,
-                                                                   float c_err, float one_minus_gamma)
+__device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, const float* __restrict__ points, int D, int K,
+                                                   const int* __restrict__ ids, const int* __restrict__ starts,
+                                                   const int* __restrict__ sizes, int stride, int* __restrict__ knn_idx,
+                                                   float* __restrict__ knn_dist, float c_err, float one_minus_gamma,
+                                                   unsigned long long* __restrict__ stats, int stat_shift)
 {
-    constexpr int kPitch = kChunk + 4;                    // an odd number of 16-byte units: rows start in different banks
-    constexpr int kRegion = kCap * kPitch > kCap * kDistPitch ? kCap * kPitch : kCap * kDistPitch;
-    __shared__ __align__(16) float region[kRegion];       // the rows, later the distance matrix
-    __shared__ ScreenMeta M;
-    float* rows = region;
-    float* dist = region;
+    float* rows = lds;                                    // kRegion floats: the rows, later the distance matrix
+    float* dist = lds;
+    ScreenMeta& M = *reinterpret_cast<ScreenMeta*>(lds + kRegion);
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
@@ -128,6 +139,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const int n_chunks = SINGLE ? 1 : (D + kChunk - 1) / kChunk;
+    const int fm = wave + 2 * lane;                       // bit u of a member set: member wave + 2 u
+    const int* lids = M.lids;
 
     if (tid < kCap) {
         const int id = tid < s ? bid[tid] : -1;
@@ -137,7 +150,6 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     }
     if (tid == kCap) M.n_pairs[0] = 0;
     __syncthreads();
-
     // ---- 1. Gram quadrants and norms
     const bool two_blocks = s > 32;
     const bool act0 = wave == 0 || two_blocks;            // this wavefront's diagonal quadrant (block `wave`)
@@ -150,12 +162,14 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         float n0 = 0.0f, n1 = 0.0f;
         const float* pa = rows + (32 * wave + (lane & 31)) * kPitch + 8 * (lane >> 5);
         const float* pb = rows + (32 + (lane & 31)) * kPitch + 8 * (lane >> 5);
-        ld.request(M.lids, s, points, D, 0, vec_ok);
-        for (int c = 0; c < n_chunks; ++c) {
-            if (!SINGLE && c > 0) __syncthreads();       // the previous chunk has been consumed
+        ld.request(lids, s, points, D, (n_chunks - 1) * kChunk, vec_ok);
+        for (int step = 0; step < n_chunks; ++step) {
+            const int c = n_chunks - 1 - step;           // the last chunk first
+            if (!SINGLE && step > 0) __syncthreads();    // the previous chunk has been consumed
             ld.commit(rows, kPitch);
             __syncthreads();
-            if (!SINGLE && c + 1 < n_chunks) ld.request(M.lids, s, points, D, (c + 1) * kChunk, vec_ok);
+            // the next chunk of this pass; after the last one (chunk 0) the first chunk of the second pass
+            if (!SINGLE) ld.request(lids, s, points, D, (c > 0 ? c - 1 : 1) * kChunk, vec_ok);
             const int ksteps = min(kChunk, (D - c * kChunk + 15) & ~15) >> 4;
             if (act0) {
                 for (int k = 0; k < ksteps; ++k) {
@@ -210,24 +224,39 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                 const int i = __ffs(bits) - 1;
                 bits &= bits - 1;
                 const int m = mbase + 8 * (i >> 2) + (i & 3);
-                M.list[at++] = (uint16_t)(m | (n << 6));
+                if (at < kListCap) M.list[at] = (uint16_t)(m | (n << 6));
+                ++at;
             }
         };
         if (act0) screen(g0, wave, wave);
         if (act1) screen(g1, 0, 1);
     }
     __syncthreads();
-    const int n_list = M.n_pairs[0];
-    if (n_list == 0) return;                          // no pair of this bucket can change a row
+    const int n_passed = M.n_pairs[0];
+    if (stats && tid == 0 && (bkt & ((1 << stat_shift) - 1)) == 0)
+        atomicAdd(&stats[(bkt >> stat_shift) & 7], ((unsigned long long)(s * (s - 1) / 2) << 32) | (unsigned long long)n_passed);
+    if (n_passed == 0) return;                        // no pair of this bucket can change a row
 
     // ---- 3. exact distances of the listed pairs: thread t takes entries t, t + 128, ...
+    // More pairs than the list holds: all pairs, in the order (a, a + o mod s) for o = 1 .. (s - 1) / 2 and all a, then
+    // o = s / 2 with a < s / 2 when s is even: pair number p has o = p / s + 1, a = p mod s.
+    const bool all_pairs = n_passed > kListCap;
+    const int n_list = all_pairs ? s * (s - 1) / 2 : n_passed;
     const int rounds = (n_list + kThreads - 1) / kThreads;
+    const float inv_s = 1.0f / (float)s;
     float acc[kMaxRounds];
 #pragma unroll
     for (int r = 0; r < kMaxRounds; ++r) acc[r] = 0.0f;
     auto entry = [&](int r) {                         // idle threads compute pair (0, 0)
         const int p = tid + r * kThreads;
-        return p < n_list ? (uint32_t)M.list[p] : 0u;
+        if (p >= n_list) return 0u;
+        if (!all_pairs) return (uint32_t)M.list[p];
+        // p / s (exact: p < 2048 and (p + 0.5) / s is never within 1 / 128 of an integer)
+        const int q = (int)(((float)p + 0.5f) * inv_s);
+        const int a = p - q * s;
+        int b = a + q + 1;
+        if (b >= s) b -= s;
+        return (uint32_t)(a | (b << 6));
     };
     auto chains = [&](int np) {
 #pragma unroll
@@ -237,6 +266,8 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
                 const float* ra = rows + (e & 63u) * (uint32_t)kPitch;
                 const float* rb = rows + (e >> 6) * (uint32_t)kPitch;
                 float a = acc[r];
+                // (not unrolled all the way: with a whole chunk's reads hoisted the registers do not suffice)
+#pragma unroll 4
                 for (int q = 0; q < np; ++q) {
                     const float4 x = *reinterpret_cast<const float4*>(ra + 4 * q);
                     const float4 y = *reinterpret_cast<const float4*>(rb + 4 * q);
@@ -253,12 +284,12 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     if (SINGLE) {
         chains((D + 3) >> 2);                         // the rows are still in LDS
     } else {
-        ld.request(M.lids, s, points, D, 0, vec_ok);
-        for (int c = 0; c < n_chunks; ++c) {
+        chains(kChunk >> 2);                          // so is the first chunk; the second is on its way
+        for (int c = 1; c < n_chunks; ++c) {
             __syncthreads();
             ld.commit(rows, kPitch);
             __syncthreads();
-            if (c + 1 < n_chunks) ld.request(M.lids, s, points, D, (c + 1) * kChunk, vec_ok);
+            if (c + 1 < n_chunks) ld.request(lids, s, points, D, (c + 1) * kChunk, vec_ok);
             chains(min(kChunk, (D - c * kChunk + 3) & ~3) >> 2);
         }
     }
@@ -279,10 +310,9 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
     }
     __syncthreads();
 
-    // ---- 4. top-K update: a wavefront walks its members that have a candidate, four at a time, with the rows of the
-    //         next four in flight
-    const int my_id = M.lids[lane];
-    const int fm = wave + 2 * lane;                   // bit u: member wave + 2 u has a candidate
+    // ---- 4. top-K update: a wavefront walks its members that have a candidate, eight at a time, with the rows of the
+    //         next eight in flight
+    const int my_id = lids[lane];
     uint32_t active = (uint32_t)ballot64(lane < 32 && M.flag[fm < kCap ? fm : 0] != 0);
     auto next_member = [&]() {
         if (active == 0) return -1;
@@ -294,12 +324,12 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
         ri = -2;
         rd = INFINITY;
         if (i >= 0 && lane < K) {
-            const size_t at = (size_t)M.lids[i] * (size_t)K + lane;
+            const size_t at = (size_t)lids[i] * (size_t)K + lane;
             ri = knn_idx[at];
             rd = knn_dist[at];
         }
     };
-    constexpr int kAhead = 4;
+    constexpr int kAhead = 8;
     int cur_i[kAhead], cur_ri[kAhead], nxt_i[kAhead], nxt_ri[kAhead];
     float cur_rd[kAhead], nxt_rd[kAhead];
 #pragma unroll
@@ -323,13 +353,60 @@ __global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* 
             row.init_sorted(K);
             row.merge(lane < s && lane != i, my_id, dist[i * kDistPitch + lane]);
             if (row.changed) {
-                const size_t at = (size_t)M.lids[i] * (size_t)K;
+                const size_t at = (size_t)lids[i] * (size_t)K;
                 row.store(knn_idx + at, knn_dist + at);
             }
         }
 #pragma unroll
         for (int u = 0; u < kAhead; ++u) { cur_i[u] = nxt_i[u]; cur_ri[u] = nxt_ri[u]; cur_rd[u] = nxt_rd[u]; }
     }
+}
+
+template <bool SINGLE>
+__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_screen(const float* __restrict__ points, int D, int K,
+                                                                   const int* __restrict__ ids,
+                                                                   const int* __restrict__ starts,
+                                                                   const int* __restrict__ sizes, int stride,
+                                                                   int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                                   float c_err, float one_minus_gamma)
+{
+    extern __shared__ __align__(16) float lds_s[];
+    screen_bucket_body<SINGLE>(lds_s, points, D, K, ids, starts, sizes, stride, knn_idx, knn_dist, c_err, one_minus_gamma,
+                               nullptr, 0);
+}
+
+// The kernel of a forest's trees: every workgroup looks at the numbers of pairs the tree before this one left behind
+// (prev: 8 words, pairs << 32 | pairs that had to be evaluated exactly, as both forms of the kernel count them in a
+// sample of the buckets) and
+// takes the screened form when fewer than share_q16 / 65536 of the pairs had to be, the direct form otherwise (and
+// for the first tree, prev == null).  One scalar load and a few scalar instructions per workgroup; both forms leave
+// their own numbers in stats for the next tree.  All K-NN rows sorted on entry.
+template <bool SINGLE>
+__global__ __launch_bounds__(kThreads, 4) void k_bucket_knn_auto(const float* __restrict__ points, int D, int K,
+                                                                 const int* __restrict__ ids, const int* __restrict__ starts,
+                                                                 const int* __restrict__ sizes, int* __restrict__ knn_idx,
+                                                                 float* __restrict__ knn_dist, float c_err,
+                                                                 float one_minus_gamma, int chunk, int pitch,
+                                                                 int region_floats,
+                                                                 const unsigned long long* __restrict__ prev,
+                                                                 unsigned int share_q16,
+                                                                 unsigned long long* __restrict__ stats, int stat_shift)
+{
+    extern __shared__ __align__(16) float lds_a[];
+    bool screened = share_q16 == kScreenAlways;
+    if (prev && !screened) {
+        unsigned long long sum = 0;                      // (the halves cannot carry into each other: a tree has < 2^32 pairs)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += prev[i];
+        const unsigned long long listed = sum & 0xffffffffull, total = sum >> 32;
+        screened = total > 0 && (listed << 16) < total * share_q16;
+    }
+    if (screened)
+        screen_bucket_body<SINGLE>(lds_a, points, D, K, ids, starts, sizes, 0, knn_idx, knn_dist, c_err, one_minus_gamma, stats,
+                                   stat_shift);
+    else
+        small_bucket::small_bucket_body<kCap, kThreads, 33>(lds_a, points, D, K, ids, starts, sizes, 0, 2, knn_idx, knn_dist,
+                                                            chunk, pitch, region_floats, 1, stats, stat_shift);
 }
 
 // one wavefront per row: rows that are not sorted by distance are rebuilt by insertion
@@ -368,26 +445,63 @@ int launch_bucket_knn_screen(const float* points, int D, int K, const int* ids, 
     RSFK_CHECK(one_minus_gamma > 0.5f, "screened small-bucket kernel: D too large");
     const dim3 grid((unsigned)n_buckets), block(kThreads);
     if (D <= kChunk)
-        hipLaunchKernelGGL(k_bucket_knn_screen<true>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx,
-                           knn_dist, c_err, one_minus_gamma);
+        hipLaunchKernelGGL(k_bucket_knn_screen<true>, grid, block, kScreenLdsBytes, stream, points, D, K, ids, starts, sizes,
+                           stride, knn_idx, knn_dist, c_err, one_minus_gamma);
     else
-        hipLaunchKernelGGL(k_bucket_knn_screen<false>, grid, block, 0, stream, points, D, K, ids, starts, sizes, stride, knn_idx,
-                           knn_dist, c_err, one_minus_gamma);
+        hipLaunchKernelGGL(k_bucket_knn_screen<false>, grid, block, kScreenLdsBytes, stream, points, D, K, ids, starts, sizes,
+                           stride, knn_idx, knn_dist, c_err, one_minus_gamma);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
 
-// First tree of a build whose small buckets take the screened kernel (later trees too).  RSFK_BUCKET_SCREEN=<tree>
-// overrides (0 = every tree and the stage-level call, "off" = never).
-int bucket_screen_from(int D, int K)
+// The small buckets (2..64 points, starts / sizes form) of one tree of a forest; every K-NN row sorted on entry.
+// prev: the 8 words a launch of this kind (or of either form) left for the tree before, or null for the first tree;
+// stats: 8 zeroed words for this tree.  The form of the kernel is chosen on the device from prev (k_bucket_knn_auto).
+int launch_bucket_knn_auto(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int n_buckets, int* knn_idx, float* knn_dist, const unsigned long long* prev,
+                           unsigned long long* stats, hipStream_t stream)
 {
-    if (K > 64) return 0x7fffffff;
-    const char* e = std::getenv("RSFK_BUCKET_SCREEN");
-    if (e && *e) return (e[0] >= '0' && e[0] <= '9') ? std::atoi(e) : 0x7fffffff;
-    // The first trees of a build change most rows with most pairs, and every pair that passes the screen costs more
-    // here than in the direct kernel; measured on uniform (D = 100) and clustered (D = 256) points the screened kernel
-    // is the faster one from the 8th and the 4th tree on.
-    return D >= 128 ? 4 : 8;
+    if (n_buckets <= 0) return 0;
+    RSFK_CHECK(K >= 1 && K <= 64 && D >= 1, "small-bucket kernel: K must be in 1..64 and D positive");
+    const float c_err = split_gram_error_coefficient((D + 15) & ~15);
+    const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);
+    RSFK_CHECK(one_minus_gamma > 0.5f, "small-bucket kernel: D too large");
+    int chunk, pitch;
+    small_bucket::small_bucket_shape(D, &chunk, &pitch);
+    const int region_floats = small_bucket::small_bucket_region_floats<kCap, kThreads, 33>(pitch);
+    const size_t lds = std::max(kScreenLdsBytes, small_bucket::small_bucket_lds_bytes<kCap, kThreads, 33>(pitch));
+    const unsigned int share_q16 = bucket_screen_share_q16();
+    // about 256 to 512 of the buckets are counted
+    int stat_shift = 0;
+    while ((n_buckets >> (stat_shift + 1)) >= 256) ++stat_shift;
+    const dim3 grid((unsigned)n_buckets), block(kThreads);
+    if (D <= kChunk)
+        hipLaunchKernelGGL(k_bucket_knn_auto<true>, grid, block, lds, stream, points, D, K, ids, starts, sizes, knn_idx, knn_dist,
+                           c_err, one_minus_gamma, chunk, pitch, region_floats, prev, share_q16, stats, stat_shift);
+    else
+        hipLaunchKernelGGL(k_bucket_knn_auto<false>, grid, block, lds, stream, points, D, K, ids, starts, sizes, knn_idx, knn_dist,
+                           c_err, one_minus_gamma, chunk, pitch, region_floats, prev, share_q16, stats, stat_shift);
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+// The small buckets of a tree take the screened form of the kernel when, in the tree before, less than this share
+// (in 1 / 65536) of the pairs had to be evaluated exactly.  Every pair that passes the bound costs more in the
+// screened form (its chain reads two rows from LDS on its own, where the direct form shares them among the four pairs
+// of a block, and the rows pass through LDS twice), every pair that does not costs less: measured on uniform 100-
+// dimensional and clustered 256-dimensional points the two forms take the same time when about four fifths of the
+// pairs pass (the second tree of a build), and the screened form is ahead from the third tree on (43 to 48 %).  RSFK_BUCKET_SCREEN=<percent> overrides; "never" = 0; "always" = the screened form for every tree and for the
+// stage-level call as well (kScreenAlways).
+unsigned int bucket_screen_share_q16()
+{
+    double pct = 60.0;
+    const char* e = std::getenv("RSFK_BUCKET_SCREEN");          // (read at every call: tests change it)
+    if (e && *e) {
+        if (e[0] == 'a') return kScreenAlways;
+        pct = e[0] >= '0' && e[0] <= '9' ? std::atof(e) : 0.0;
+    }
+    pct = std::min(100.0, std::max(0.0, pct));
+    return (unsigned int)(pct * 65536.0 / 100.0 + (pct >= 100.0 ? 1.0 : 0.0));
 }
 
 }  // namespace rsfk

@@ -38,8 +38,10 @@ namespace {
 
 // the last build of this process (knn_forest_device), for build_report_json
 struct BuildReport {
-    int N = 0, D = 0, K = 0, n_trees = 0, passes = 0, row_bytes = 0, screen_from = 0;
+    int N = 0, D = 0, K = 0, n_trees = 0, passes = 0, row_bytes = 0;
     std::vector<int> kernels;                          // per tree: kBucketKernel... bits
+    std::vector<unsigned long long> pairs;             // per tree: pairs of its small buckets << 32 | those evaluated exactly
+    unsigned int screen_share_q16 = 0;
     unsigned long long tested = 0, undecided = 0;      // tree build: point-levels, and those left to the exact test
     unsigned long long exact = 0;                      // exploration: exact distances over all passes
     double tree_s = 0.0, bucket_s = 0.0, explore_s = 0.0;
@@ -151,7 +153,7 @@ int build_report_json(char* buf, int cap)
         {kBucketKernelSmall, "k_bucket_knn_small<64>"}, {kBucketKernelScreen, "k_bucket_knn_screen"},
         {kBucketKernelMedium, "k_bucket_knn_small<72>"}, {kBucketKernelRows, "k_bucket_knn_rows"},
         {kBucketKernelTiled, "k_bucket_knn<per bucket>"}, {kBucketKernelStrip, "k_bucket_knn<per 64 members>"},
-        {kBucketKernelGram, "k_bucket_knn_gram"}};
+        {kBucketKernelGram, "k_bucket_knn_gram"}, {kBucketKernelAuto, "k_bucket_knn_auto"}};
     std::string s = "{";
     auto num = [&](const char* key, double v, bool last = false) {
         char t[96];
@@ -173,6 +175,26 @@ int build_report_json(char* buf, int cap)
         a = b + 1;
     }
     s += "], ";
+    // k_bucket_knn_auto: share of the pairs of a tree's small buckets that had to be evaluated exactly, and the form of
+    // the kernel that share selected for the next tree (the first tree takes the direct form)
+    s += "\"bucket_pair_share\": [";
+    for (size_t t = 0; t < r.pairs.size(); ++t) {
+        const double total = (double)(r.pairs[t] >> 32), listed = (double)(r.pairs[t] & 0xffffffffull);
+        char tmp[32];
+        std::snprintf(tmp, sizeof tmp, "%s%.4f", t ? ", " : "", total > 0 ? listed / total : 0.0);
+        s += tmp;
+    }
+    s += "], \"bucket_screened\": [";
+    for (size_t t = 0; t < r.pairs.size(); ++t) {
+        bool scr = r.screen_share_q16 == kScreenAlways;
+        if (t > 0 && !scr) {
+            const unsigned long long total = r.pairs[t - 1] >> 32, listed = r.pairs[t - 1] & 0xffffffffull;
+            scr = total > 0 && (listed << 16) < total * r.screen_share_q16;
+        }
+        s += std::string(t ? ", " : "") + ((r.kernels[t] & kBucketKernelAuto) && scr ? "1" : "0");
+    }
+    s += "], ";
+    num("bucket_screen_share", r.screen_share_q16 == kScreenAlways ? 2.0 : r.screen_share_q16 / 65536.0);
     num("tree_points_tested", (double)r.tested); num("tree_points_undecided", (double)r.undecided);
     num("tree_screen_row_bytes", r.row_bytes); num("tree_seconds", r.tree_s); num("bucket_seconds", r.bucket_s);
     num("explore_passes", r.passes); num("explore_exact_distances", (double)r.exact);
@@ -196,9 +218,8 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
     if (n_trees == 0 && nnef <= 0) return 0;          // nothing to do: no copies are made, nothing is queued
     const double t_forest0 = now_s();
-    const int screen_from = bucket_screen_from(D, K);
     BuildReport rep;
-    rep.N = N; rep.D = D; rep.K = K; rep.n_trees = n_trees; rep.passes = std::max(nnef, 0); rep.screen_from = screen_from;
+    rep.N = N; rep.D = D; rep.K = K; rep.n_trees = n_trees; rep.passes = std::max(nnef, 0);
     rep.kernels.assign((size_t)n_trees, 0);
 
     Q8Guard q8;
@@ -226,6 +247,14 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         std::vector<TimedEvent> ev((size_t)B + 1);
         for (auto& e : ev)
             if (e.create()) return 1;
+        // numbers of pairs of every tree's small buckets (8 words per tree, added up on the host for the report): the
+        // kernel of tree t reads those of tree t - 1 to choose its form
+        DevBuf pair_stats;
+        const size_t stat_words = (size_t)8 * (size_t)n_trees;
+        if (ws_alloc(&pair_stats.p, sizeof(unsigned long long) * stat_words)) return 1;
+        RSFK_HIP(hipMemsetAsync(pair_stats.p, 0, sizeof(unsigned long long) * stat_words, stream));
+        unsigned long long* d_pairs = static_cast<unsigned long long*>(pair_stats.p);
+        rep.screen_share_q16 = bucket_screen_share_q16();
         const int gram_from = bucket_gram_from();
         constexpr int kYoungTrees = 2;          // trees of a build whose bucket step still finds rows that are far from done
         SideStream sync;
@@ -251,11 +280,13 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 (void)hipEventRecord(ev[j].e, stream);                         // both parts of the previous tree are done
                 if (split) (void)hipStreamWaitEvent(sync.side, ev[j].e, 0);      // everything before this tree
                 const bool gram = t0 + j >= gram_from;
-                rc = launch_bucket_knn_tree(d_points, t0 + j >= screen_from, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                const int t = t0 + j;
+                rc = launch_bucket_knn_tree(d_points, t > 0 ? d_pairs + (size_t)8 * (t - 1) : nullptr, d_pairs + (size_t)8 * t, true,
+                                            gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
                                             d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees, &rep.kernels[(size_t)(t0 + j)]);
                 if (!rc && split) {
-                    rc = launch_bucket_knn_tree(d_points, false, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
+                    rc = launch_bucket_knn_tree(d_points, nullptr, nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
                                                 stats[5 * j + 2], d_idx, d_dist, sync.side, 2, t0 + j < kYoungTrees,
                                                 &rep.kernels[(size_t)(t0 + j)]);
@@ -292,6 +323,10 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             }
         }
         if (rc) return rc;
+        std::vector<unsigned long long> h_pairs(stat_words);
+        RSFK_HIP(hipMemcpy(h_pairs.data(), d_pairs, sizeof(unsigned long long) * stat_words, hipMemcpyDeviceToHost));
+        rep.pairs.assign((size_t)n_trees, 0);
+        for (size_t i = 0; i < stat_words; ++i) rep.pairs[i / 8] += h_pairs[i];
     }
     const double t_forest = now_s() - t_forest0;
     if (verbose >= 1) std::printf("Creating RSFK forest takes %lf seconds\n", t_forest);

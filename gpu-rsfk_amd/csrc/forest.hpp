@@ -42,16 +42,17 @@ int bucket_gram_from();
 enum : int {
     kBucketKernelSmall = 1,      // k_bucket_knn_small<64>: two wavefronts per bucket of up to 64 points, every pair exact
     kBucketKernelScreen = 2,     // k_bucket_knn_screen: the same with the pair matrix bounded on the matrix cores first
+    kBucketKernelAuto = 128,     // k_bucket_knn_auto: one of the two, chosen on the device from the previous tree's pairs
     kBucketKernelMedium = 4,     // k_bucket_knn_small<72>: three wavefronts, buckets of 65..72 points
     kBucketKernelRows = 8,       // k_bucket_knn_rows: a bucket's points resident in LDS
     kBucketKernelTiled = 16,     // k_bucket_knn<SL, false>: 64 x 64 tiles, a workgroup per bucket
     kBucketKernelStrip = 32,     // k_bucket_knn<SL, true>: 64 x 64 tiles, a workgroup per 64 members of a bucket
     kBucketKernelGram = 64,      // k_bucket_knn_gram: any bucket size, pair matrix bounded on the matrix cores
 };
-int launch_bucket_knn_tree(const float* points, bool screen, bool rows_sorted, bool gram, int D, int K, const int* ids,
-                           const int* starts, const int* sizes, int leaf_cap, int n_small, int n_big, int max_bucket,
-                           int* knn_idx, float* knn_dist, hipStream_t stream, int part = 0, bool young_rows = true,
-                           int* launched = nullptr);
+int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_stats, unsigned long long* stats,
+                           bool rows_sorted, bool gram, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int leaf_cap, int n_small, int n_big, int max_bucket, int* knn_idx, float* knn_dist,
+                           hipStream_t stream, int part = 0, bool young_rows = true, int* launched = nullptr);
 
 // What the last K-NN-graph build of this process did, as a line of JSON (rsfk_last_build_report): which bucket
 // kernels every tree went to, the counts the algorithmic bytes of the tree build and of the exploration are made of,
@@ -63,8 +64,15 @@ int build_report_json(char* buf, int cap);
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream);
 int launch_bucket_knn_screen(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
                              int n_buckets, int stride, int* knn_idx, float* knn_dist, hipStream_t stream);
-// trees from this index on send their buckets of up to 64 points to that kernel (RSFK_BUCKET_SCREEN)
-int bucket_screen_from(int D, int K);
+// Buckets of up to 64 points of one tree of a forest, the form of the kernel (every pair exact, or bounded on the matrix
+// cores first) chosen on the device from the numbers of pairs the tree before left in prev (8 words; null: first tree);
+// stats: 8 zeroed words for this tree's numbers.
+int launch_bucket_knn_auto(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes,
+                           int n_buckets, int* knn_idx, float* knn_dist, const unsigned long long* prev,
+                           unsigned long long* stats, hipStream_t stream);
+// share of the pairs (in 1 / 65536) below which the screened form is taken (RSFK_BUCKET_SCREEN); kScreenAlways: always
+constexpr unsigned int kScreenAlways = 0xffffffffu;
+unsigned int bucket_screen_share_q16();
 
 // bucket_knn_rows.hip
 int bucket_rows_cap(int D, int K);

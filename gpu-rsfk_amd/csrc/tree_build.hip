@@ -42,7 +42,7 @@ namespace rsfk {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kGroups = kBlock / 8;      // groups of 8 lanes per workgroup: one point each per iteration
+
 
 struct LevelCounters {
     int n_next;        // nodes appended for the next wide level

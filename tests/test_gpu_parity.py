@@ -95,7 +95,7 @@ def test_tree_edge_cases(gpu, orc, rng):
 def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
     """kernel: "direct" = fp32 chains for every pair; "gram" = the kernel that bounds the pair matrix on the matrix
     cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0); "screen" = the same
-    idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=0; other buckets, and K > 64,
+    idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=always; other buckets, and K > 64,
     take the direct kernels); "direct_per_bucket" = the tiled direct kernel with a workgroup per bucket, as launches
     over many buckets run it (RSFK_BUCKET_STRIP=0; with the few buckets of a test it otherwise takes a workgroup per 64
     members), and without the kernel that keeps a bucket's points in LDS (RSFK_BUCKET_ROWS=0)."""
@@ -109,7 +109,7 @@ def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX
     if kernel == "screen":
         if K > 64 or MIN > 64:
             pytest.skip("no bucket of this shape reaches the screened small-bucket kernel")
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "0")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "always")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K)
     gi, gd = orc.init_lists(N, K)
@@ -307,7 +307,7 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
 def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, T, kw, variant):
     import gpu_rsfk
     if variant == "bucket_screen":
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")       # every tree but the first through the screened small-bucket kernel
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "100")     # every tree but the first through the screened small-bucket kernel
     X = rng.standard_normal((N, D)).astype(np.float32)
     r = gpu_rsfk.RSFK(random_state=17)
     _say("forest", N, D, K, T, kw)
@@ -339,9 +339,9 @@ def test_baseline_config_workloads_match_oracle(gpu, orc, monkeypatch, config, N
     if kernel == "screen":
         if config != "c3":
             pytest.skip("no bucket of this configuration reaches the screened small-bucket kernel")
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "1")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "100")
     else:
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "off")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "never")
     X = baseline_points(config, N)
     r = gpu_rsfk.RSFK(random_state=0)
     _say("forest", config, N, X.shape[1], K, T, kw)
@@ -540,11 +540,11 @@ def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant
     """The bfloat16 screens only skip work whose outcome is certain: trees, bucket K-NN and exploration on inputs
     that defeat a 8-bit mantissa must still be identical to the fp32 oracle.  "bucket_screen" also switches the
     buckets of up to 64 points to the two-wavefront kernel that bounds the pair matrix on the matrix cores
-    (RSFK_BUCKET_SCREEN=0: every tree and the stage-level call), "bucket_gram" all buckets to the tiled kernel that
+    (RSFK_BUCKET_SCREEN=always: every tree and the stage-level call), "bucket_gram" all buckets to the tiled kernel that
     does the same (RSFK_GRAM_FROM=0)."""
     import gpu_rsfk
     if variant == "bucket_screen":
-        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "0")
+        monkeypatch.setenv("RSFK_BUCKET_SCREEN", "always")
     if variant == "bucket_gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     N, D, K = 6000, 24, 10
