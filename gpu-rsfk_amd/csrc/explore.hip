@@ -367,13 +367,14 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
                                                                const uint16_t* __restrict__ bounds,
                                                                const int* __restrict__ todo_in, int n_in,
                                                                int* __restrict__ todo_out, int* __restrict__ n_out,
-                                                               unsigned long long* __restrict__ stat)
+                                                               unsigned long long* __restrict__ stat,
+                                                               const int* __restrict__ order)
 {
     extern __shared__ __align__(16) int lds_m[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int slot = blockIdx.x * WAVES + wave;
+    const int slot = die_local_place(blockIdx.x, gridDim.x) * WAVES + wave;
     if (slot >= (todo_in ? n_in : N)) return;             // whole wavefront leaves together
-    const int p = todo_in ? todo_in[slot] : slot;
+    const int p = todo_in ? todo_in[slot] : (order ? order[slot] : slot);
     const int MW = (K + 31) >> 5;
     int bits = 0;
     for (int k = lane; k < K; k += 64) {
@@ -589,7 +590,8 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     __shared__ int n_set_s;
     __shared__ uint32_t tau_s;                                    // bits of the smallest last slot reached so far
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int slot = blockIdx.x;
+    // (the list of points a launch before this one left over is in the order in which that launch came to them)
+    const int slot = die_local_place(blockIdx.x, gridDim.x);
     if (slot >= (todo_in ? n_in : N)) return;
     const int p = todo_in ? todo_in[slot] : slot;
     const int MW = (K + 31) >> 5, KP = MW * 32;
@@ -787,7 +789,7 @@ int launch_merge_wg(const float* points, int N, int D, int K, const int* old_idx
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge_wg<SL>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
-    hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3((unsigned)n_work), dim3(256), lds, stream, points, N, D, K, old_idx,
+    hipLaunchKernelGGL((k_explore_merge_wg<SL>), dim3(grid_for_dies((size_t)n_work)), dim3(256), lds, stream, points, N, D, K, old_idx,
                        knn_idx, knn_dist, cap, dpad, pass, bounds, todo_in, n_in, todo_out, n_out, stat);
     RSFK_HIP(hipGetLastError());
     return 0;
@@ -803,15 +805,16 @@ int next_pow2(int v)
 template <int SL, int WAVES>
 int launch_merge(const float* points, int N, int D, int K, const int* old_idx, int* knn_idx, float* knn_dist, int table,
                  int wave_ints, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in, int n_in,
-                 int* todo_out, int* n_out, unsigned long long* stat, hipStream_t stream)
+                 int* todo_out, int* n_out, unsigned long long* stat, const int* order, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES>),
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
-    dim3 grid((unsigned)((n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
+    dim3 grid(grid_for_dies(((size_t)n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
     hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out, stat);
+                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out, stat,
+                       order);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -825,13 +828,13 @@ int merge_wave_ints(int table, int dpad, int K, bool with_bounds = false)
 
 int dispatch_merge(int sl, int waves, const float* points, int N, int D, int K, const int* old_idx, int* knn_idx,
                    float* knn_dist, int table, int dpad, const uint32_t* pass, const uint16_t* bounds, const int* todo_in,
-                   int n_in, int* todo_out, int* n_out, unsigned long long* stat, hipStream_t stream)
+                   int n_in, int* todo_out, int* n_out, unsigned long long* stat, const int* order, hipStream_t stream)
 {
     const int wi = merge_wave_ints(table, dpad, K, bounds != nullptr);
 #define RSFK_MERGE_CASE(SLV, WV)                                                                                        \
     if (sl == SLV && waves == WV)                                                                                       \
         return launch_merge<SLV, WV>(points, N, D, K, old_idx, knn_idx, knn_dist, table, wi, dpad, pass, bounds, \
-                                     todo_in, n_in, todo_out, n_out, stat, stream);
+                                     todo_in, n_in, todo_out, n_out, stat, order, stream);
     RSFK_MERGE_CASE(1, 4) RSFK_MERGE_CASE(1, 2) RSFK_MERGE_CASE(1, 1)
     RSFK_MERGE_CASE(2, 4) RSFK_MERGE_CASE(2, 2) RSFK_MERGE_CASE(2, 1)
     RSFK_MERGE_CASE(4, 4) RSFK_MERGE_CASE(4, 2) RSFK_MERGE_CASE(4, 1)
@@ -901,7 +904,7 @@ bool explore_merge_fits(int D, int K)
 // distance.
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted,
-                   unsigned long long* stat)
+                   unsigned long long* stat, const int* order)
 {
     if (N <= 0) return 0;
     RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
@@ -939,7 +942,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         // Marks from the join, then the merge kernel with a small set (little LDS, many wavefronts per CU).
         // The points it cannot take come back in a list and get a second launch with the largest set that
         // fits; what is left after that goes to the general kernel below.
-        if (launch_explore_join(ws, *bf_join, N, D, K, old_idx, knn_dist, stream)) return 1;
+        if (launch_explore_join(ws, *bf_join, N, D, K, old_idx, knn_dist, stream, order)) return 1;
         const uint32_t* pass = explore_ws_pass(ws);
         int* listA = explore_ws_todo(ws, 0);
         int* listB = explore_ws_todo(ws, 1);
@@ -948,7 +951,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
         const uint16_t* wave_bounds = explore_ws_bounds(ws);
         if (4 * merge_wave_ints(small_table, dpad, K, true) > lds_ints) wave_bounds = nullptr;
         if (dispatch_merge(sl, 4, points, N, D, K, old_idx, knn_idx, knn_dist, small_table, dpad, pass, wave_bounds, nullptr, 0,
-                           listA, listA + N, stat, stream))
+                           listA, listA + N, stat, order, stream))
             return 1;
         RSFK_HIP(hipMemcpyAsync(host_n, listA + N, sizeof(int), hipMemcpyDeviceToHost, stream));
         RSFK_HIP(hipStreamSynchronize(stream));
@@ -968,7 +971,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
             int rc = 0;
             if (!per_wg)
                 rc = dispatch_merge(sl, big_waves, points, N, D, K, old_idx, knn_idx, knn_dist, big_table, dpad, pass,
-                                    nullptr, listA, n_todo, listB, listB + N, stat, stream);
+                                    nullptr, listA, n_todo, listB, listB + N, stat, nullptr, stream);
             else if (sl == 1)
                 rc = launch_merge_wg<1>(points, N, D, K, old_idx, knn_idx, knn_dist, wg_cap, dpad, pass, bounds, listA,
                                         n_todo, listB, listB + N, stat, stream);

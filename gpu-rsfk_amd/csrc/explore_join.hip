@@ -239,12 +239,13 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join(Bf16Copy bf, int N,
                                                               const int* __restrict__ offs, const int* __restrict__ rev,
                                                               uint32_t* __restrict__ pass, uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
                                                               float kappa, float one_minus_gamma, int wave_lds_ints,
-                                                              uint32_t div_m, int div_s)
+                                                              uint32_t div_m, int div_s, const int* __restrict__ order)
 {
     extern __shared__ __align__(16) int lds_join[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int q = blockIdx.x * WAVES + wave;
-    if (q >= N) return;                                   // whole wavefront leaves together
+    const int item = die_local_place(blockIdx.x, gridDim.x) * WAVES + wave;
+    if (item >= N) return;                                // whole wavefront leaves together
+    const int q = order ? order[item] : item;
     const int r0 = offs[q], R = offs[q + 1] - r0;
     if (R <= 0) return;
     int* cq = lds_join + (size_t)wave * (size_t)wave_lds_ints;
@@ -340,13 +341,15 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_join_short(Bf16Copy bf, 
                                                                     const float2* __restrict__ norm_tau,
                                                                     const int* __restrict__ offs, const int* __restrict__ rev,
                                                                     uint32_t* __restrict__ pass, int bpitch, int ksteps,
-                                                                    float kappa, float one_minus_gamma, uint32_t div_m, int div_s)
+                                                                    float kappa, float one_minus_gamma, uint32_t div_m, int div_s,
+                                                                    const int* __restrict__ order)
 {
     __shared__ int pid_s[WAVES][32];
     __shared__ float pn_s[WAVES][32], ptau_s[WAVES][32];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int q = blockIdx.x * WAVES + wave;
-    if (q >= N) return;                                   // whole wavefront leaves together
+    const int item = die_local_place(blockIdx.x, gridDim.x) * WAVES + wave;
+    if (item >= N) return;                                // whole wavefront leaves together
+    const int q = order ? order[item] : item;
     const int r0 = offs[q], R = offs[q + 1] - r0;
     const int col = lane & 31, hi = lane >> 5;
     int cid = col < K ? old_idx[(size_t)q * K + col] : -1;
@@ -434,7 +437,8 @@ __global__ __launch_bounds__(256) void k_explore_join_wg(Bf16Copy bf, int N, int
                                                          const float2* __restrict__ norm_tau, const int* __restrict__ offs,
                                                          const int* __restrict__ rev, uint32_t* __restrict__ pass,
                                                          uint16_t* __restrict__ bounds, int KP, int bpitch, int ksteps,
-                                                         float kappa, float one_minus_gamma, uint32_t div_m, int div_s)
+                                                         float kappa, float one_minus_gamma, uint32_t div_m, int div_s,
+                                                         const int* __restrict__ order)
 {
     constexpr int kPieces = (kJwP + (NPW == 3 ? 128 : 256)) * 8 / 256;      // 16-byte pieces a thread stages per step
     extern __shared__ __align__(16) unsigned char lds_jw[];
@@ -447,9 +451,11 @@ __global__ __launch_bounds__(256) void k_explore_join_wg(Bf16Copy bf, int N, int
     float* ptau = pn + kJwP;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n = lane & 31, h = lane >> 5;
-    const int q = blockIdx.x;
+    const int item = die_local_place(blockIdx.x, gridDim.x);
+    if (item >= N) return;                                                 // the whole workgroup leaves together
+    const int q = order ? order[item] : item;
     const int r0 = offs[q], R = offs[q + 1] - r0;
-    if (R <= 0) return;                                                    // the whole workgroup leaves together
+    if (R <= 0) return;
     const int MW = KP >> 5;
     const int nrows = kJwP + KP;
     for (int k = tid; k < KP; k += 256) {
@@ -638,7 +644,7 @@ int* explore_ws_host_count(ExploreWorkspace* w) { return w->host_count; }
 
 // Fill pass (and bounds) from the snapshot old_idx and the current last slots of knn_dist (rows sorted by distance).
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
-                        const float* knn_dist, hipStream_t stream)
+                        const float* knn_dist, hipStream_t stream, const int* order)
 {
     RSFK_CHECK(w && w->N == N && w->K == K, "exploration join: workspace does not match");
     RSFK_CHECK(K >= 1 && K <= 256, "exploration join: K must be in 1..256");
@@ -668,10 +674,10 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     const float one_minus_gamma = 1.0f - (float)(D + 8) * (1.0f / 4194304.0f);      // 1 - (D + 8) 2^-22
     RSFK_CHECK(one_minus_gamma > 0.5f, "exploration join: D too large");
     if (!w->bounds && KP == 32 && ksteps <= 8) {
-        const dim3 grid((unsigned)((N + kWaves - 1) / kWaves)), block(64 * kWaves);
+        const dim3 grid(grid_for_dies(((size_t)N + kWaves - 1) / kWaves)), block(64 * kWaves);
 #define RSFK_JOIN_SHORT(KSV)                                                                                                \
         hipLaunchKernelGGL((k_explore_join_short<kWaves, KSV>), grid, block, 0, stream, bf, N, K, old_idx, w->norm_tau, w->offs, \
-                           w->rev, w->pass, bf16_pitch(D), ksteps, kappa, one_minus_gamma, w->div_m, w->div_s)
+                           w->rev, w->pass, bf16_pitch(D), ksteps, kappa, one_minus_gamma, w->div_m, w->div_s, order)
         if (ksteps <= 2) RSFK_JOIN_SHORT(2);
         else if (ksteps <= 4) RSFK_JOIN_SHORT(4);
         else RSFK_JOIN_SHORT(8);
@@ -684,9 +690,9 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
         do {                                                                                                               \
             RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_join_wg<BV, NV>),                         \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_wg));                       \
-            hipLaunchKernelGGL((k_explore_join_wg<BV, NV>), dim3((unsigned)N), dim3(256), lds_wg, stream, bf, N, K, old_idx,  \
-                               w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps, kappa,           \
-                               one_minus_gamma, w->div_m, w->div_s);                                                       \
+            hipLaunchKernelGGL((k_explore_join_wg<BV, NV>), dim3(grid_for_dies((size_t)N)), dim3(256), lds_wg, stream, bf, N, K,  \
+                               old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps, kappa,  \
+                               one_minus_gamma, w->div_m, w->div_s, order);                                                \
         } while (0)
         if (w->bounds && KP <= 128) RSFK_JOIN_WG(true, 3);
         else if (w->bounds) RSFK_JOIN_WG(true, 6);
@@ -694,13 +700,13 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
         else RSFK_JOIN_WG(false, 6);
 #undef RSFK_JOIN_WG
     } else if (w->bounds)
-        hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
+        hipLaunchKernelGGL((k_explore_join<kWaves, true>), dim3(grid_for_dies(((size_t)N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
-                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
+                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s, order);
     else
-        hipLaunchKernelGGL((k_explore_join<kWaves, false>), dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
+        hipLaunchKernelGGL((k_explore_join<kWaves, false>), dim3(grid_for_dies(((size_t)N + kWaves - 1) / kWaves)), dim3(64 * kWaves), lds,
                            stream, bf, N, K, old_idx, w->norm_tau, w->offs, w->rev, w->pass, w->bounds, KP, bf16_pitch(D), ksteps,
-                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s);
+                           kappa, one_minus_gamma, wave_ints, w->div_m, w->div_s, order);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

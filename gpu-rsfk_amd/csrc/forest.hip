@@ -225,6 +225,11 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     Q8Guard q8;
     const uint8_t* q8_rows = nullptr;
     if (n_trees > 0 && make_tree_screen(q8, d_points, N, D, verbose, stream, &q8_rows)) return 1;
+    // The permutation of the last tree (points grouped by bucket) is kept for the exploration: points of a bucket are
+    // close to each other and share neighbours, so working on them one after the other on the same die finds the rows
+    // of those neighbours in its L2.
+    DevBuf order;
+    if (n_trees > 0 && nnef > 0 && ws_alloc(&order.p, sizeof(int) * (size_t)N)) return 1;
     // The uncentred bfloat16 copy screens the side tests when the 8-bit copy does not, and the general exploration
     // kernel; with the 8-bit screen and the join nobody needs it (the few points the merge kernels may hand back to
     // the general kernel are then worked on without a screen).
@@ -323,6 +328,11 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
             }
         }
         if (rc) return rc;
+        if (order.p) {
+            // (finished before the tree workspace goes back to the pool)
+            RSFK_HIP(hipMemcpyAsync(order.p, tree_ws_perm(ws.w, (n_trees - 1) % B), sizeof(int) * (size_t)N, hipMemcpyDeviceToDevice, stream));
+            RSFK_HIP(hipStreamSynchronize(stream));
+        }
         std::vector<unsigned long long> h_pairs(stat_words);
         RSFK_HIP(hipMemcpy(h_pairs.data(), d_pairs, sizeof(unsigned long long) * stat_words, hipMemcpyDeviceToHost));
         rep.pairs.assign((size_t)n_trees, 0);
@@ -347,7 +357,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         for (int it = 0; it < nnef; ++it) {
             // (the bucket step of the forest, and every exploration pass, leave all rows in order)
             if (launch_explore(d_points, plain_copy ? &bf.c : nullptr, &bfc.c, N, D, K, d_idx, d_dist, static_cast<int*>(old.p), ews.w, stream,
-                               n_trees > 0 || it > 0, static_cast<unsigned long long*>(stat.p)))
+                               n_trees > 0 || it > 0, static_cast<unsigned long long*>(stat.p), static_cast<const int*>(order.p)))
                 return 1;
         }
         std::vector<unsigned long long> h_stat((size_t)kExploreStatWords);

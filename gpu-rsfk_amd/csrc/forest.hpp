@@ -18,7 +18,7 @@ int tree_ws_leaf_cap(const TreeBatchWorkspace* w);
 const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
-int tree_small_threshold();
+int tree_small_threshold(int D);
 const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w);
 const unsigned long long* tree_ws_counts(const TreeBatchWorkspace* w);
 int tree_screen_row_bytes(int D, bool q8);
@@ -104,8 +104,10 @@ const uint32_t* explore_ws_pass(const ExploreWorkspace* w);
 const uint16_t* explore_ws_bounds(const ExploreWorkspace* w);
 int* explore_ws_todo(ExploreWorkspace* w, int which);
 int* explore_ws_host_count(ExploreWorkspace* w);
+// order: null, or a permutation of the points that keeps nearby points together (the buckets of a tree): the points
+// are then worked on in that order, a contiguous eighth of it per die (die_local_place)
 int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, int K, const int* old_idx,
-                        const float* knn_dist, hipStream_t stream);
+                        const float* knn_dist, hipStream_t stream, const int* order = nullptr);
 
 // explore.hip
 // true when rows of K neighbours of D-dimensional points get the merge kernel that takes a point's candidates in the
@@ -114,7 +116,8 @@ bool explore_merge_uses_bounds(int D, int K);
 bool explore_join_keeps_bounds(int N, int D, int K);
 int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_join, int N, int D, int K, int* knn_idx,
                    float* knn_dist, int* old_idx, ExploreWorkspace* ws, hipStream_t stream, bool rows_sorted = false,
-                   unsigned long long* stat = nullptr);      // stat: kExploreStatWords words, or null (count_exact)
+                   unsigned long long* stat = nullptr,       // stat: kExploreStatWords words, or null (count_exact)
+                   const int* order = nullptr);              // order: see launch_explore_join
 constexpr int kExploreStatWords = 32 * 256;
 
 // graph_export.hip

@@ -44,6 +44,16 @@ void ws_release_all();
     } while (0)
 
 // ---------------------------------------------------------------------------
+// Which item a workgroup takes when neighbouring items should meet in the same L2 cache.  The device has eight dies
+// (XCDs), each with its own L2, and workgroup b of a launch runs on die b mod 8: with a grid that is a multiple of 8,
+// workgroup b takes place (b mod 8) * (grid / 8) + b / 8, so that each die works through one contiguous eighth of the
+// items in order.  (Places beyond the number of items are for the caller to skip.)
+// ---------------------------------------------------------------------------
+constexpr int kDies = 8;
+__device__ __forceinline__ int die_local_place(int block, int grid) { return (block & (kDies - 1)) * (grid / kDies) + block / kDies; }
+inline unsigned grid_for_dies(size_t n_blocks) { return (unsigned)((n_blocks + kDies - 1) / kDies * kDies); }
+
+// ---------------------------------------------------------------------------
 // counter-based random numbers.  A node of a tree is identified by a 64-bit key
 // derived from the tree seed and the left/right path to the node, so a tree is
 // a pure function of (points, MIN, MAX, MAX_DEPTH, seed) whatever the launch

@@ -36,6 +36,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <chrono>
 
 namespace rsfk {
 
@@ -1056,7 +1057,16 @@ const int* tree_ws_perm(const TreeBatchWorkspace* w, int t) { return w->perm[0] 
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t) { return w->leaf_start + (size_t)t * w->leaf_cap; }
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t) { return w->leaf_size + (size_t)t * w->leaf_cap; }
 
-int tree_small_threshold() { return 1024; }
+// Nodes of at most this many points are finished by one workgroup (k_tail): 1024, or 2048 for short rows, where a
+// wide level costs more per byte of row it reads (the permutation entries it moves weigh more) -- measured on 10M x 32
+// points 4.46 against 4.81 ms per tree, on 1M x 100 points 0.548 against 0.520.  RSFK_TREE_SMALL overrides (tests).
+int tree_small_threshold(int D)
+{
+    const char* e = std::getenv("RSFK_TREE_SMALL");
+    const int v = e && *e ? std::atoi(e) : (D <= 48 ? 2048 : 1024);
+    return std::min(2048, std::max(64, v));
+}
+constexpr int kWideChunk = 1024;         // points per workgroup in the wide passes (k_side keeps a chunk's undecided points in LDS)
 
 // bytes of device memory a batch of B trees needs
 size_t tree_ws_bytes(int N, int D, int MIN, int B)
@@ -1087,11 +1097,11 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     TreeBatchWorkspace* w = new TreeBatchWorkspace();
     *out = w;
     w->B = B; w->N = N; w->D = D;
-    const int small = tree_small_threshold();
+    const int small = tree_small_threshold(D);
     w->leaf_cap = N / std::max(MIN, 1) + 2;
     w->node_cap = B * (N / small + 2);
     w->tail_cap = B * w->leaf_cap;
-    w->chunk_cap = B * (N / small + 2) * 2 + 16;      // sum ceil(count/chunk) <= N/chunk + nodes
+    w->chunk_cap = B * (N / kWideChunk + N / small + 4) + 16;      // sum ceil(count/chunk) <= N/chunk + nodes
     if (dmalloc(&w->perm[0], (size_t)B * N)) return 1;
     if (dmalloc(&w->perm[1], (size_t)B * N)) return 1;
     if (dmalloc(&w->nodes[0], (size_t)w->node_cap)) return 1;
@@ -1147,9 +1157,8 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_CHECK(N >= 1 && D >= 1, "tree batch: N and D must be positive");
     TreeParams P;
     P.N = N; P.D = D; P.MIN = MIN; P.MAX = MAX; P.MAX_DEPTH = MAX_DEPTH;
-    P.small = tree_small_threshold();
-    P.chunk = P.small;
-    RSFK_CHECK(P.chunk <= 1024, "tree batch: chunk size");
+    P.small = tree_small_threshold(D);
+    P.chunk = kWideChunk;
     // bfloat16 rounding 2^-8 (1 + 2^-7), plus the summation errors of the screen (D/8 terms per lane and a 3-step
     // tree) and of the exact test (D/32 terms per lane and a 5-step tree), 1 % on top
     P.band = 1.01f * ((1.0f + 1.0f / 128.0f) / 256.0f + (float)(D / 8 + D / 32 + 16) / 16777216.0f);
@@ -1205,6 +1214,13 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
         RSFK_HIP(hipStreamSynchronize(stream));
         RSFK_CHECK(!w->h_ctr->overflow, "tree batch: node queue overflow");
         const int n_nodes = w->h_ctr->n_next;
+        if (std::getenv("RSFK_TREE_TRACE")) {
+            static double t_prev = 0.0;
+            const double t_now = std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+            std::fprintf(stderr, "level %d: %d nodes, %d chunks, tail %d, previous level %.3f ms\n", level, n_nodes,
+                         w->h_ctr->n_chunks, w->h_ctr->n_tail, level ? (t_now - t_prev) * 1e3 : 0.0);
+            t_prev = t_now;
+        }
         if (n_nodes == 0) break;
         RSFK_CHECK(n_nodes <= w->node_cap, "tree batch: node queue overflow");
         const int n_chunks = w->h_ctr->n_chunks;
