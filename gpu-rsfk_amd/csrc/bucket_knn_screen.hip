@@ -28,8 +28,10 @@
 //      chains of its pairs of the list (arithmetic of euclidean_distance_sqr,
 //      compute_knn_from_buckets.cu:40-54: a pair has the same distance value as in
 //      every other kernel);
-//   4. the exact distances go into the bucket's distance matrix in LDS (+inf
-//      elsewhere) and the rows that got a candidate are merged as in the other kernel.
+//   4. an exact distance that is not above the last slot of a row goes into the
+//      bucket's distance matrix in LDS and sets the member's bit in that row's
+//      candidate set (nothing else of the matrix is written or read); the rows
+//      with a candidate are merged as in the other kernel.
 //
 // Requires every K-NN row to be sorted on entry (the last slot is its maximum);
 // launch_sort_rows establishes that once per build.
@@ -55,13 +57,14 @@ constexpr int kMaxRounds = (kMaxPairs + kThreads - 1) / kThreads;     // listed 
 // Pairs the list holds.  A bucket with more pairs to evaluate (nearly half of those of a full bucket: the first trees
 // of a build) evaluates all its pairs, which then need no list.  With this size the workgroup's LDS is 20 KB and eight
 // workgroups share a compute unit.
-constexpr int kListCap = 880;
+constexpr int kListCap = 752;
 
-// LDS after the row / distance region: ids, last slots, flags, norms as seen by either wavefront, pair counter, list
-struct ScreenMeta {
+// LDS after the row / distance region: ids, last slots, candidate sets, norms as seen by either wavefront, pair
+// counter, list
+struct alignas(16) ScreenMeta {
     int lids[kCap];
     float tau[kCap];
-    int flag[kCap];
+    unsigned long long cand[kCap];          // bit j of cand[i]: member j is at a distance not above the last slot of row i
     float nrm[2][kCap];
     int n_pairs[4];
     uint16_t list[kListCap];
@@ -146,7 +149,7 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
         const int id = tid < s ? bid[tid] : -1;
         M.lids[tid] = id;
         M.tau[tid] = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
-        M.flag[tid] = 0;
+        M.cand[tid] = 0ull;
     }
     if (tid == kCap) M.n_pairs[0] = 0;
     __syncthreads();
@@ -207,16 +210,24 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
             const int mbase = 32 * qi + 4 * (lane >> 5);
             uint32_t bits = 0;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int m = mbase + 8 * (i >> 2) + (i & 3);
-                const float S = nrm[m] + nn;
-                const float dt = __builtin_fmaf(-2.0f, g[i], S);
-                const float lower = (dt - __builtin_fmaf(c_err, S, 1e-35f)) * one_minus_gamma;
-                // a NaN bound never drops a pair (the comparison is false); a NaN last slot cannot occur: rows only
-                // hold what passed `distance < last slot`, +inf where they are empty
-                const bool drop = lower > fmaxf(M.tau[m], tn);
-                const bool valid = n < s && (qi == qj ? m < n : m < s);
-                if (valid && !drop) bits |= 1u << i;
+            for (int i4 = 0; i4 < 4; ++i4) {
+                // four consecutive members at a time (16-byte reads of their norms and last slots)
+                const int m0 = mbase + 8 * i4;
+                const float4 nm4 = *reinterpret_cast<const float4*>(&nrm[m0]);
+                const float4 tm4 = *reinterpret_cast<const float4*>(&M.tau[m0]);
+                const float nm[4] = {nm4.x, nm4.y, nm4.z, nm4.w}, tm[4] = {tm4.x, tm4.y, tm4.z, tm4.w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int i = 4 * i4 + c, m = m0 + c;
+                    const float S = nm[c] + nn;
+                    const float dt = __builtin_fmaf(-2.0f, g[i], S);
+                    const float lower = (dt - __builtin_fmaf(c_err, S, 1e-35f)) * one_minus_gamma;
+                    // a NaN bound never drops a pair (the comparison is false); a NaN last slot cannot occur: rows
+                    // only hold what passed `distance < last slot`, +inf where they are empty
+                    const bool drop = lower > fmaxf(tm[c], tn);
+                    const bool valid = n < s && (qi == qj ? m < n : m < s);
+                    if (valid && !drop) bits |= 1u << i;
+                }
             }
             const int cnt = __popc(bits);
             int at = cnt ? atomicAdd(&M.n_pairs[0], cnt) : 0;
@@ -294,18 +305,21 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
         }
     }
     __syncthreads();                                  // rows no longer needed: the region becomes the distance matrix
-    for (int i = tid; i < kCap * kDistPitch; i += kThreads) dist[i] = INFINITY;
-    __syncthreads();
+    // (only the entries a row may take are written, and cand says which they are: nothing else of the matrix is read)
 #pragma unroll
     for (int r = 0; r < kMaxRounds; ++r) {
         if (tid + r * kThreads < n_list) {
             const uint32_t e = entry(r);
             const int i = (int)(e & 63u), j = (int)(e >> 6);
             const float d = acc[r];
-            dist[i * kDistPitch + j] = d;
-            dist[j * kDistPitch + i] = d;
-            if (d <= M.tau[i]) M.flag[i] = 1;         // plain stores of the same value: no ordering needed
-            if (d <= M.tau[j]) M.flag[j] = 1;
+            if (d <= M.tau[i]) {
+                dist[i * kDistPitch + j] = d;
+                atomicOr(&M.cand[i], 1ull << j);
+            }
+            if (d <= M.tau[j]) {
+                dist[j * kDistPitch + i] = d;
+                atomicOr(&M.cand[j], 1ull << i);
+            }
         }
     }
     __syncthreads();
@@ -313,7 +327,7 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
     // ---- 4. top-K update: a wavefront walks its members that have a candidate, eight at a time, with the rows of the
     //         next eight in flight
     const int my_id = lids[lane];
-    uint32_t active = (uint32_t)ballot64(lane < 32 && M.flag[fm < kCap ? fm : 0] != 0);
+    uint32_t active = (uint32_t)ballot64(lane < 32 && M.cand[fm < kCap ? fm : 0] != 0ull);
     auto next_member = [&]() {
         if (active == 0) return -1;
         const int u = __ffs(active) - 1;
@@ -351,7 +365,8 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
             row.idx[0] = cur_ri[u];
             row.dist[0] = cur_rd[u];
             row.init_sorted(K);
-            row.merge(lane < s && lane != i, my_id, dist[i * kDistPitch + lane]);
+            const bool offered = (M.cand[i] >> lane) & 1ull;
+            row.merge(offered, my_id, offered ? dist[i * kDistPitch + lane] : INFINITY);
             if (row.changed) {
                 const size_t at = (size_t)lids[i] * (size_t)K;
                 row.store(knn_idx + at, knn_dist + at);
