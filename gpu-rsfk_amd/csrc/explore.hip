@@ -483,7 +483,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     auto batch = [&](const int* list, int n) {
         n_exact += n;
         if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
-        else exact_batch<SL, kMergeChunk, true>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
+        else exact_batch<SL, kMergeChunk, 2>(L, list, n, points, D, vec_ok, row);       // two steps of gathers in flight
     };
     if (tbound == nullptr || U <= 64) {
         for (int off = 0; off < U; off += 64) {
@@ -543,24 +543,30 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
 // of gathering a whole fp32 row.  Here:
 //   1. all threads list the marked (neighbour, slot) pairs of the point together with the lower bound L the join
 //      kept for each (explore_join.hip; 0 when it kept none), one 32-bit word per pair;
-//   2. every wavefront walks its quarter of the list kWgRounds times with a rising limit -- the distances at the
-//      1/8, 2/8, ... of its own copy of the row, which improves from round to round, capped by the smallest last slot
-//      any wavefront has reached (shared through LDS) -- and takes the pairs whose bound lies between the previous
-//      limit and this one: near candidates first, without sorting anything.  A pair whose bound is above the shared
-//      last slot at its turn is never looked at.  The others have their id read, pass through a hash set (seeded
-//      with the row; drops repeats -- only a saving: a repeated candidate would be rejected by the row), wait until 64
-//      of them are together, get the exact distance and are merged into the wavefront's copy of the row;
-//   3. the first wavefront merges the four rows and stores the result.
+//   2. every wavefront walks its quarter of the list in rounds with a rising limit: the smallest limit that takes 64
+//      marks it has not taken yet (found by bisection on the 16 bits of the bounds), never above the shared last
+//      slot -- near candidates first, without sorting anything.  A pair whose bound is above the shared last slot at
+//      its turn is never looked at.  The others have their id read, pass through a hash set (seeded with the row;
+//      drops repeats -- only a saving: a repeated candidate would be rejected by the row), get the exact distance,
+//      64 at a time and what is left at the end of the round, and are merged into the wavefront's copy of the row.
+//      Between the rounds the wavefronts work out what the last slot of their four rows taken together would be
+//      (shared_last_slot below, no merge needed), which is the limit nobody goes beyond: measured on 70,000 x 784 rows
+//      with K = 90, 184 exact distances per point instead of 544 with a limit from each wavefront's own row, for the
+//      85 entries of a row that change;
+//   3. the four rows become one in two steps (2 -> 0 and 3 -> 1, then 1 -> 0), entries above that limit left out,
+//      and the first wavefront stores the result.
 // A bound is below the exact distance of its pair, the shared last slot is never below the final one: a dropped
 // candidate could not have been in the final row, so the result is the one of any other order.
 // (Sorting the list by the bounds first, a bitonic network over up to 4096 words in LDS, cost more than it saved.)
-// LDS (ints): table[kWgTable] | srow[K] | jrow[K] | xrow[dpad] | marked[cap] | 4 tiles | 3 rows for the exchange | 4 x 128 ids.
+// LDS (ints): table[kWgTable] | srow[K] | jrow[K] | xrow[dpad] | marked[cap] | 4 tiles | 3 rows for the exchange | 4 x 128 ids
+// | distances of the row as loaded [K] | distances of the four rows as last shown [4][K].
 constexpr int kWgChunk = 32;
 constexpr int kWgTile = 64 * (kWgChunk + 4);
 constexpr int kWgTable = 2048;              // hash set; when three quarters are taken, new ids are no longer recorded
 constexpr int kWgMinCap = 1024;             // the kernel is not used when fewer marks than this would fit
 
-constexpr int kWgRounds = 8;
+constexpr int kWgMaxRounds = 12;
+constexpr int kWgDepth = 2;                 // steps of gathers in flight (a third one changed nothing)            // the last one takes everything that is left below the last slot
 constexpr int kWgMaxCap = 6656;             // marks per point: 26 steps of the walk of a wavefront
 constexpr int kWgMaxSteps = kWgMaxCap / 256;
 
@@ -603,6 +609,9 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     int* tiles = reinterpret_cast<int*>(marked + cap);
     int* xch = tiles + 4 * kWgTile;                               // rows on their way to another wavefront: [3][idx | dist][64 SL]
     int* ids = xch + 6 * 64 * SL + 128 * wave;                    // this wavefront's candidates: a batch and what is left over
+    const int kq = (K + 3) & ~3;
+    float* old_d = reinterpret_cast<float*>(xch + 6 * 64 * SL + 4 * 128);  // distances of the row as it was loaded
+    float* seen_d = old_d + kq;                                   // [4][kq]: the rows of the wavefronts as they last showed them
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
     KnnRow<SL> row;
@@ -617,6 +626,13 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     if (k < K) {
         srow[k] = old_idx[(size_t)p * K + k];
         jrow[k] = j;
+    }
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+        if (lane + 64 * s < K) {
+            seen_d[wave * kq + lane + 64 * s] = row.dist[s];      // every wavefront starts from the same sorted row
+            if (wave == 0) old_d[lane + 64 * s] = row.dist[s];
+        }
     }
     int mine = 0;
     if (j >= 0)
@@ -691,30 +707,118 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         const int n_now = min(64, have);
         n_exact += n_now;
         const float cap_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
-        exact_batch<SL, kWgChunk, true>(L, ids, n_now, points, D, vec_ok, row, cap_now);
+        exact_batch<SL, kWgChunk, kWgDepth>(L, ids, n_now, points, D, vec_ok, row, cap_now);
         if (lane == 0) atomicMin(&tau_s, __float_as_uint(row.tau));   // non-negative floats order like their bits
         have -= n_now;
         const int left = lane < have ? ids[64 + lane] : 0;        // the candidates beyond the batch move to the front
         wave_lds_sync();
         if (lane < have) ids[lane] = left;
     };
-    float prev = -1.0f;                                           // bounds are never negative
-    for (int r = 0; r < kWgRounds; ++r) {
-        const float thr = r + 1 < kWgRounds ? row_slot_dist(row, max(0, K * (r + 1) / kWgRounds - 1)) : INFINITY;
-        if (!(thr > prev)) continue;
+    // The last slot of the four rows taken together, without merging them.  The wavefronts evaluate disjoint sets of
+    // new candidates (the hash set, as long as it records), none of them in the row as loaded, so for any t the
+    // candidates and old entries at a distance <= t number at least sum_w c_w(t) - 3 o(t), with c_w(t) the entries
+    // <= t of the row of wavefront w and o(t) those of the row as loaded (a row holds every old entry below its own
+    // last slot, and what it dropped is above it).  The smallest t among this wavefront's own entries for which
+    // that number reaches K is at least the last slot of the final row.  Rows of the other wavefronts are read as
+    // they were last shown, possibly half-way through being shown again: entries only fall, the search only moves
+    // past an entry it has seen to be <= t, so a stale or mixed row gives a smaller count and a larger t.
+    auto shared_last_slot = [&]() {
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+            if (lane + 64 * s < K) seen_d[wave * kq + lane + 64 * s] = row.dist[s];
+        wave_lds_sync();
+        int top = 1;
+        while (2 * top <= K) top *= 2;
+        // the searches of a lane (its SL entries in the three other rows and in the row as loaded) advance together:
+        // their reads do not wait for each other
+        int pos[SL][4];
+#pragma unroll
+        for (int s = 0; s < SL; ++s)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) pos[s][w] = 0;
+        const volatile float* arr[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const int other = w + (w >= wave ? 1 : 0);            // 0..3 without this wavefront, then 4 = the row as loaded
+            arr[w] = other < 4 ? seen_d + other * kq : old_d;
+        }
+        for (int b = top; b > 0; b >>= 1) {
+#pragma unroll
+            for (int s = 0; s < SL; ++s) {
+                const float t = row.dist[s];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const int np = pos[s][w] + b;
+                    if (np <= K && arr[w][np - 1] <= t) pos[s][w] = np;
+                }
+            }
+        }
+        float best = INFINITY;
+#pragma unroll
+        for (int s = 0; s < SL; ++s) {
+            const int slot = lane + 64 * s;
+            const float t = row.dist[s];
+            // (arr[0..2]: the other wavefronts, arr[3]: the row as loaded)
+            const int total = slot + 1 + pos[s][0] + pos[s][1] + pos[s][2] - 3 * pos[s][3];
+            const uint64_t okm = ballot64(slot < K && t < INFINITY && total >= K);
+            if (okm != 0 && best == INFINITY) best = read_lane_f(t, first_lane(okm));   // rows are sorted: the first is the smallest
+        }
+        // (read after the rows: once the set no longer records, two wavefronts may hold the same candidate)
+        const bool recording = *reinterpret_cast<volatile int*>(&n_set_s) < kWgTable / 4 * 3;
+        if (recording && lane == 0 && best < INFINITY) atomicMin(&tau_s, __float_as_uint(best));
+    };
+    // the bounds of this wavefront's marks (upper 16 bits of the fp32 number; non-negative floats order like their bits)
+    int lb16[kWgMaxSteps];
+#pragma unroll
+    for (int u = 0; u < kWgMaxSteps; ++u) {
+        const int at = 64 * wave + 256 * u + lane;
+        lb16[u] = at < n_marked ? (int)(marked[at] >> 16) : 0x7fffffff;
+    }
+    auto marks_upto = [&](int from, int upto) {                   // marks with from < bound <= upto
+        int n = 0;
+#pragma unroll
+        for (int u = 0; u < kWgMaxSteps; ++u) {
+            if (64 * wave + 256 * u >= n_marked) break;
+            n += __popcll(ballot64(lb16[u] > from && lb16[u] <= upto));
+        }
+        return n;
+    };
+    int least = 0x7fffffff;                                       // the smallest bound of this wavefront's marks
+#pragma unroll
+    for (int u = 0; u < kWgMaxSteps; ++u) least = min(least, lb16[u]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) least = min(least, __shfl_xor(least, o, 64));
+    int prev = -1;                                                // bounds up to here have been taken
+    bool rows_moved = false;                                      // a batch has run since the last slots were compared
+    for (int r = 0; r < kWgMaxRounds; ++r) {
+        if (rows_moved) {
+            shared_last_slot();
+            rows_moved = false;
+        }
+        const int lim = (int)(*reinterpret_cast<volatile uint32_t*>(&tau_s) >> 16);   // bound <= last slot iff its 16 bits <= lim
+        if (lim <= prev) break;
+        // the smallest limit that takes a batch; everything up to the last slot when that is less (or in the last round)
+        int lo = max(prev + 1, min(least, lim)), hi = lim;
+        if (r + 1 < kWgMaxRounds) {
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (marks_upto(prev, mid) >= 64 - have) hi = mid;
+                else lo = mid + 1;
+            }
+        } else {
+            lo = lim;
+        }
+        const int upto = lo;
         // first the ids of everything this round takes (all reads travel together), then the candidates one step
         // of the walk after the other
-        const float tau_round = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
-        const float lim = fminf(thr, tau_round);
         int c[kWgMaxSteps];
 #pragma unroll
         for (int u = 0; u < kWgMaxSteps; ++u) {
             const int at = 64 * wave + 256 * u + lane;
             c[u] = -1;
-            if (at < n_marked) {
+            if (lb16[u] > prev && lb16[u] <= upto) {              // (false beyond the list)
                 const uint32_t e = marked[at];
-                const float lb = __uint_as_float(e & 0xffff0000u);
-                if (lb > prev && !(lb > lim)) c[u] = old_idx[(size_t)srow[e & 255u] * K + ((e >> 8) & 255u)];
+                c[u] = old_idx[(size_t)srow[e & 255u] * K + ((e >> 8) & 255u)];
             }
         }
 #pragma unroll
@@ -723,9 +827,8 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
             bool fresh = c[u] >= 0 && c[u] < N && c[u] != p;
             if (ballot64(fresh) == 0) continue;
             // the shared last slot may have fallen since the ids were requested
-            const int at = 64 * wave + 256 * u + lane;
             const float tau_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
-            if (fresh && __uint_as_float(marked[at] & 0xffff0000u) > tau_now) fresh = false;
+            if (fresh && __uint_as_float((uint32_t)lb16[u] << 16) > tau_now) fresh = false;
             if (fresh && *reinterpret_cast<volatile int*>(&n_set_s) < kWgTable / 4 * 3) {
                 fresh = set_insert(table, kWgTable - 1, c[u], false);
                 if (fresh) atomicAdd(&n_set_s, 1);
@@ -733,14 +836,22 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
             const uint64_t fm = ballot64(fresh);
             if (fresh) ids[have + mask_prefix(fm)] = c[u];        // have < 64 here: at most 127 entries
             have += __popcll(fm);
-            if (have >= 64) run_batch();
+            if (have >= 64) {
+                run_batch();
+                rows_moved = true;
+            }
         }
-        prev = thr;
+        prev = upto;
+        if (have > 0) {                                           // the next round's limit comes from the rows
+            run_batch();
+            rows_moved = true;
+        }
     }
     if (have > 0) run_batch();
     count_exact(stat, n_exact);
 
     // ---- 3. one row out of four: wavefronts 0 and 1 take the rows of 2 and 3, then 0 takes the row of 1
+    float tau_all = INFINITY;
     auto put_row = [&](int at) {
 #pragma unroll
         for (int s = 0; s < SL; ++s) {
@@ -753,9 +864,15 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         for (int s = 0; s < SL; ++s) {
             const int c = xch[(at * 2 + 0) * (64 * SL) + lane + 64 * s];
             const float d = __int_as_float(xch[(at * 2 + 1) * (64 * SL) + lane + 64 * s]);
-            row.merge(lane + 64 * s < K && c >= 0, c, d);
+            row.merge(lane + 64 * s < K && c >= 0 && d <= tau_all, c, d);
         }
     };
+    // The last slot of the four rows together, once more with all batches done: entries above it (most of what the
+    // rows still share with the row as loaded) need not be offered to the row that takes them.
+    __syncthreads();
+    shared_last_slot();
+    __syncthreads();
+    tau_all = __uint_as_float(tau_s);
     if (wave >= 2) put_row(wave - 2);
     __syncthreads();
     if (wave < 2) take_row(wave);
@@ -771,13 +888,13 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
 int merge_wg_cap(int dpad, int K, int sl)
 {
     const int budget = 78 * 1024 / 4;
-    const int fixed = kWgTable + 2 * ((K + 3) & ~3) + dpad + 4 * kWgTile + 6 * 64 * sl + 4 * 128;
+    const int fixed = kWgTable + 2 * ((K + 3) & ~3) + dpad + 4 * kWgTile + 6 * 64 * sl + 4 * 128 + 5 * ((K + 3) & ~3);
     return std::min(std::min(budget - fixed, K * K), kWgMaxCap);
 }
 
 int merge_wg_ints(int cap, int dpad, int K, int sl)
 {
-    return (kWgTable + 2 * ((K + 3) & ~3) + dpad + cap + 4 * kWgTile + 6 * 64 * sl + 4 * 128 + 3) / 4 * 4;
+    return (kWgTable + 2 * ((K + 3) & ~3) + dpad + cap + 4 * kWgTile + 6 * 64 * sl + 4 * 128 + 5 * ((K + 3) & ~3) + 3) / 4 * 4;
 }
 
 template <int SL>
