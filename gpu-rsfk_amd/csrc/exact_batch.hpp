@@ -40,11 +40,11 @@ __device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int 
 
 // Exact distances of the first n candidates of `list` to the point, then offer them.  CH = dimensions
 // staged per step (32 or 16): a step moves 64 rows x CH floats through the tile.  tau_cap: a bound the caller
-// knows for the row's final last slot (candidates above it need not be finished), else +inf.  DEPTH: the loads of
-// DEPTH steps are in flight while one more is being used (DEPTH register buffers that take turns, so that waiting
-// for one does not wait for the others): 2 or 3 for kernels with few wavefronts per SIMD, whose gathers would
-// otherwise wait for each other.
-template <int SL, int CH = kChunk, int DEPTH = 1>
+// knows for the row's final last slot (candidates above it need not be finished), else +inf.  DEEP: the loads of
+// two steps are in flight while a third is being used (two register buffers that take turns, so that waiting for
+// one does not wait for the other): for kernels with few wavefronts per SIMD, whose gathers would otherwise wait
+// for each other.
+template <int SL, int CH = kChunk, bool DEEP = false>
 __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
                                             const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row,
                                             float tau_cap = INFINITY)
@@ -63,7 +63,7 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
         const int r = i * kRows + sub;
         rp[i] = r < n ? points + (size_t)list[r] * (size_t)D : nullptr;    // nothing is read for the rows beyond n
     }
-    float4 pre[DEPTH][kLoads];
+    float4 pre[DEEP ? 2 : 1][kLoads];
     auto request = [&](float4 (&buf)[kLoads], int d0) {
         if (d0 < D) {
 #pragma unroll
@@ -98,13 +98,16 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
         return ballot64(lane < n && acc <= tau0) != 0;
     };
     bool finished = true;
-#pragma unroll
-    for (int b = 0; b < DEPTH; ++b) request(pre[b], b * CH);
-    for (int d0 = 0; d0 < D && finished; d0 += DEPTH * CH) {
-#pragma unroll
-        for (int b = 0; b < DEPTH; ++b) {
-            if (finished && d0 + b * CH < D && !step(pre[b], d0 + b * CH, DEPTH * CH)) finished = false;
+    request(pre[0], 0);
+    if (DEEP) {
+        request(pre[1], CH);
+        for (int d0 = 0; d0 < D; d0 += 2 * CH) {
+            if (!step(pre[0], d0, 2 * CH)) { finished = false; break; }
+            if (d0 + CH < D && !step(pre[1], d0 + CH, 2 * CH)) { finished = false; break; }
         }
+    } else {
+        for (int d0 = 0; d0 < D; d0 += CH)
+            if (!step(pre[0], d0, CH)) { finished = false; break; }
     }
     wave_lds_sync();
     row.merge(lane < n && finished, my_c, acc);          // unfinished sums are all above the last slot

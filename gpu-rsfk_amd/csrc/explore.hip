@@ -483,7 +483,7 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     auto batch = [&](const int* list, int n) {
         n_exact += n;
         if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
-        else exact_batch<SL, kMergeChunk, 2>(L, list, n, points, D, vec_ok, row);       // two steps of gathers in flight
+        else exact_batch<SL, kMergeChunk, true>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
     };
     if (tbound == nullptr || U <= 64) {
         for (int off = 0; off < U; off += 64) {
@@ -565,8 +565,7 @@ constexpr int kWgTile = 64 * (kWgChunk + 4);
 constexpr int kWgTable = 2048;              // hash set; when three quarters are taken, new ids are no longer recorded
 constexpr int kWgMinCap = 1024;             // the kernel is not used when fewer marks than this would fit
 
-constexpr int kWgMaxRounds = 12;
-constexpr int kWgDepth = 2;                 // steps of gathers in flight (a third one changed nothing)            // the last one takes everything that is left below the last slot
+constexpr int kWgMaxRounds = 12;            // the last one takes everything that is left below the last slot
 constexpr int kWgMaxCap = 6656;             // marks per point: 26 steps of the walk of a wavefront
 constexpr int kWgMaxSteps = kWgMaxCap / 256;
 
@@ -707,7 +706,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         const int n_now = min(64, have);
         n_exact += n_now;
         const float cap_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
-        exact_batch<SL, kWgChunk, kWgDepth>(L, ids, n_now, points, D, vec_ok, row, cap_now);
+        exact_batch<SL, kWgChunk, true>(L, ids, n_now, points, D, vec_ok, row, cap_now);
         if (lane == 0) atomicMin(&tau_s, __float_as_uint(row.tau));   // non-negative floats order like their bits
         have -= n_now;
         const int left = lane < have ? ids[64 + lane] : 0;        // the candidates beyond the batch move to the front
