@@ -21,14 +21,16 @@
 //   3. all candidates of a member are then offered to its row (knn_list.hpp), held
 //      in registers, and the row is stored if it changed.  When far more candidates
 //      are below the row's last slot than the row has slots, a histogram of their
-//      distances first removes those that cannot stay.  The K-NN rows of the next
-//      two members are requested before the chains of these two start.
+//      distances first removes those that cannot stay, and into a row that is new
+//      the rest is written by rank (counted, not inserted).  The K-NN rows of the
+//      next two members are requested before the chains of these two start.
 //
 // No distance matrix, no flags, no barrier after the staging; a row is owned by
 // one wavefront (no locks).
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
 #include "forest.hpp"
+#include "bucket_small_body.hpp"
 #include <algorithm>
 
 namespace rsfk {
@@ -53,7 +55,7 @@ __global__ __launch_bounds__(kRowsThreads) void k_bucket_knn_rows(const float* _
     extern __shared__ __align__(16) float lds_r[];
     float* rows = lds_r;                                          // 64 NT rows of `pitch` floats
     int* lids = reinterpret_cast<int*>(lds_r + 64 * NT * pitch);
-    int* hist = lids + 64 * NT + 64 * (threadIdx.x >> 6);         // this wavefront's histogram
+    int* hist = lids + 64 * NT + 192 * (threadIdx.x >> 6);        // this wavefront's histogram, then 64 distances and 64 ids
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
@@ -148,6 +150,49 @@ __global__ __launch_bounds__(kRowsThreads) void k_bucket_knn_rows(const float* _
                 for (int t = 0; t < NT; ++t) ok[t] = ok[t] && bin[t] <= cross;
             }
         }
+        if (DENSE && n_ok > 0 && small_bucket::fresh_row(ri, rd, lids[m], K)) {
+            // A new row (nothing in it but, possibly, the point itself): the candidates that are left are not inserted
+            // one after the other -- their places in the row are their ranks among themselves.  They are gathered in
+            // lanes 0.. (through LDS), ranked by counting, and stored where they belong.
+            const bool has_self = read_lane_i(ri, 0) >= 0;
+            int n_left = has_self ? 1 : 0;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) n_left += __popcll(ballot64(ok[t] && row.enters(cid[t], acc[t])));
+            if (n_left <= 64) {
+                float* cd = reinterpret_cast<float*>(hist + 64);
+                int* ci = hist + 128;
+                wave_lds_sync();
+                int at = 0;
+                if (has_self) {
+                    if (lane == 0) { cd[0] = rd; ci[0] = ri; }
+                    at = 1;
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const bool in = ok[t] && row.enters(cid[t], acc[t]);
+                    const uint64_t mk = ballot64(in);
+                    if (in) {
+                        const int p = at + mask_prefix(mk);
+                        cd[p] = acc[t];
+                        ci[p] = cid[t];
+                    }
+                    at += __popcll(mk);
+                }
+                wave_lds_sync();
+                const float d = lane < n_left ? cd[lane] : INFINITY;
+                const int c = lane < n_left ? ci[lane] : -1;
+                float place[1] = {d};
+                if (small_bucket::place_by_rank<1>(place, n_left)) {          // (not with equal distances: those take the usual way)
+                    const int slot = __float_as_int(place[0]);
+                    if (slot >= 0 && slot < K) {
+                        const size_t to = (size_t)lids[m] * (size_t)K + slot;
+                        knn_idx[to] = c;
+                        knn_dist[to] = d;
+                    }
+                    return;
+                }
+            }
+        }
         // tile after tile: the last slot a tile leaves behind already turns away candidates of the next
 #pragma unroll
         for (int t = 0; t < NT; ++t)
@@ -220,7 +265,7 @@ int launch_rows_cfg(const float* points, int D, int K, const int* ids, const int
                     int stride, int min_size, int max_size, int* knn_idx, float* knn_dist, int pitch, bool rows_sorted,
                     hipStream_t stream)
 {
-    const size_t lds = (size_t)64 * NT * pitch * sizeof(float) + (size_t)64 * (NT + kRowsWaves) * sizeof(int);
+    const size_t lds = (size_t)64 * NT * pitch * sizeof(float) + (size_t)64 * (NT + 3 * kRowsWaves) * sizeof(int);
     auto kern = k_bucket_knn_rows<NT, DENSE>;
     RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(kern, dim3((unsigned)n_buckets), dim3(kRowsThreads), lds, stream, points, D, K, ids, starts, sizes, stride,
@@ -243,7 +288,7 @@ int bucket_rows_cap(int D, int K)
 {
     if (K > 64) return 0;
     const int per_point = rows_pitch(D) * (int)sizeof(float) + (int)sizeof(int);
-    const int tiles = std::min(4, (kRowsLdsBytes - 64 * kRowsWaves * (int)sizeof(int)) / (64 * per_point));
+    const int tiles = std::min(4, (kRowsLdsBytes - 3 * 64 * kRowsWaves * (int)sizeof(int)) / (64 * per_point));
     return 64 * tiles;
 }
 
