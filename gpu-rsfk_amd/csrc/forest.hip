@@ -228,8 +228,11 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
     // The permutation of the last tree (points grouped by bucket) is kept for the exploration: points of a bucket are
     // close to each other and share neighbours, so working on them one after the other on the same die finds the rows
     // of those neighbours in its L2.
+    // (RSFK_EXPLORE_ORDER=0: the points in their own order)
     DevBuf order;
-    if (n_trees > 0 && nnef > 0 && ws_alloc(&order.p, sizeof(int) * (size_t)N)) return 1;
+    const char* order_env = std::getenv("RSFK_EXPLORE_ORDER");
+    const bool in_bucket_order = !(order_env && order_env[0] == '0');
+    if (n_trees > 0 && nnef > 0 && in_bucket_order && ws_alloc(&order.p, sizeof(int) * (size_t)N)) return 1;
     // The uncentred bfloat16 copy screens the side tests when the 8-bit copy does not, and the general exploration
     // kernel; with the 8-bit screen and the join nobody needs it (the few points the merge kernels may hand back to
     // the general kernel are then worked on without a screen).
