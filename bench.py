@@ -275,7 +275,7 @@ def bucket_sources_hash():
     h = hashlib.sha256()
     src = os.path.join(ROOT, "gpu-rsfk_amd", "csrc")
     for fn in sorted(os.listdir(src)):
-        if fn.startswith("bucket_knn") or fn in ("knn_list.hpp", "mfma_split.hpp", "wave64.hpp"):
+        if fn.startswith("bucket_knn") or fn in ("bucket_small_body.hpp", "knn_list.hpp", "mfma_split.hpp", "wave64.hpp"):
             h.update(open(os.path.join(src, fn), "rb").read())
     return h.hexdigest()[:16]
 
@@ -477,7 +477,7 @@ def main():
         roofline["note"] = ("traffic: HBM bytes per tree of the bucket K-NN kernels from the tracked rocprofv3 summary of this "
                             "command, made with the same kernel sources (profiles/%s: FETCH_SIZE x %.2f + WRITE_SIZE, all "
                             "bucket kernels of a build / trees)" % (PROFILE_FILES[cfg_name], FETCH_SCALE))
-    elif cfg_name:
+    elif cfg_name in PROFILE_FILES:
         roofline["note"] = ("traffic: null -- the tracked rocprofv3 summary (profiles/%s) was made with other sources of the "
                             "bucket kernels than this run's" % PROFILE_FILES[cfg_name])
     # what the device delivers when scattered rows of 4 D bytes are only read: every row of the matrix once, in a random
