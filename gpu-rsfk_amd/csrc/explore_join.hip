@@ -52,6 +52,15 @@ struct ExploreWorkspace {
     uint32_t* pass = nullptr;  // N*K*MW, indexed by entry number
     float2* norm_tau = nullptr; // N: norm of the bfloat16 row and last slot of the K-NN row of a point, side by side
     uint16_t* bounds = nullptr; // N*K*32*MW lower bounds of the marked pairs (bfloat16, rounded down), or null
+    // the builder for large graphs (staged_rev_*): two scatters through LDS instead of one straight to memory
+    bool staged = false;
+    int fshift = 0, cshift = 0; // fine bins of 2^fshift points (their rows are assembled in LDS), coarse bins of 2^cshift
+    int n_fine = 0, n_coarse = 0;
+    int n_sub = 0;              // sub-parts of the coarse bins at the second level (an upper bound)
+    int2* bin_eq2 = nullptr;    // N*K: the records grouped by fine bin
+    int* fine_size = nullptr;   // n_coarse << (cshift - fshift)
+    int* fine_start = nullptr;  // the same + 1
+    int* sub_off = nullptr;     // n_sub x fine bins per coarse bin
     int* todo = nullptr;       // two lists of N+1 ints: points left over by a launch; entry N = their number
     int* host_count = nullptr; // pinned
 };
@@ -221,6 +230,212 @@ __global__ __launch_bounds__(kRowsBlock) void k_bin_rows(const int2* __restrict_
         const int2 eq = bin_eq[i];
         const int at = atomicAdd(&cnt[eq.y], 1);
         rev[s0 + at] = eq.x;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// The same reversed graph for large inputs.  k_bin_scatter sends every record straight to one of several thousand
+// bins and k_bin_rows every entry straight to its row: stores of 8 and 4 bytes whose cache lines leave the L2 long
+// before their neighbours arrive (10 M x 32: 9.4 GB and 8.6 GB written for 2.56 GB and 1.28 GB of payload).  Here
+// every store to memory is a run: (1) the records go to a few hundred coarse bins, a tile of 4096 at a time sorted by
+// bin in LDS first, so a bin receives a run of records per tile; (2) inside a coarse bin the same again to its fine
+// bins; (3) a fine bin is small enough for all of its rows to be assembled in LDS and written whole.  Counting comes
+// before every scatter as in the one-level builder (no atomics on device memory per entry).  A record is
+// (entry number, neighbour).
+constexpr int kStTile = 4096;               // records sorted in LDS at a time
+constexpr int kStSub = 32768;               // records of a sub-part of a coarse bin
+constexpr int kStMaxBins = 1024;            // bins a scatter step distinguishes (LDS counters)
+constexpr int kStRowsCap = 24576;           // entries of a fine bin whose rows are assembled in LDS
+
+// counts of a part of the graph per coarse bin (k_bin_count with another shift; kept apart for the record format)
+// -> reuses k_bin_count / k_bin_scan with shift = cshift.
+
+// Sorts up to kStTile records (rec[i], bin[i] for the thread's 16 records) by bin in LDS and writes them to
+// out[cursor[bin] + rank inside (tile, bin)]; cursor (LDS, n_bins ints) moves on by the tile's counts.
+// LDS: cnt[n_bins] | first[n_bins] | stage[kStTile] (int2).
+__device__ __forceinline__ void staged_tile_out(const int2 (&rec)[16], const int (&bin)[16], int n_bins, int* cnt, int* first,
+                                                int2* stage, unsigned short* sbin, int* cursor, int* wave_lds,
+                                                int2* __restrict__ out)
+{
+    const int tid = threadIdx.x;
+    for (int b = tid; b < n_bins; b += 256) cnt[b] = 0;
+    __syncthreads();
+    int rank[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) rank[u] = bin[u] >= 0 ? atomicAdd(&cnt[bin[u]], 1) : 0;
+    __syncthreads();
+    // exclusive scan of the counts (n_bins <= 1024: four per thread)
+    {
+        int v[4], sum = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { const int b = 4 * tid + j; v[j] = b < n_bins ? cnt[b] : 0; sum += v[j]; }
+        int tot;
+        int ex = block_excl_scan(sum, &tot, wave_lds);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { const int b = 4 * tid + j; if (b < n_bins) first[b] = ex; ex += v[j]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        if (bin[u] >= 0) {
+            const int at = first[bin[u]] + rank[u];
+            stage[at] = rec[u];
+            sbin[at] = (unsigned short)bin[u];
+        }
+    }
+    __syncthreads();
+    const int n_tile = first[n_bins - 1] + cnt[n_bins - 1];
+    for (int i = tid; i < n_tile; i += 256) {
+        const int b = sbin[i];
+        out[(size_t)cursor[b] + (size_t)(i - first[b])] = stage[i];
+    }
+    __syncthreads();
+    for (int b = tid; b < n_bins; b += 256) cursor[b] += cnt[b];
+    __syncthreads();
+}
+
+constexpr size_t staged_lds_bytes(int n_bins)
+{
+    return (size_t)3 * n_bins * sizeof(int) + 8 + (size_t)kStTile * (sizeof(int2) + sizeof(unsigned short));
+}
+
+// (1) a part of the graph to the coarse bins.  part_off / bin_start as left by k_bin_count / k_bin_scan at shift = cshift.
+__global__ __launch_bounds__(256) void k_staged_scatter1(const int* __restrict__ old_idx, int total, int per_part, int N, int cshift,
+                                                         int n_coarse, const int* __restrict__ bin_start,
+                                                         const int* __restrict__ part_off, int2* __restrict__ out)
+{
+    extern __shared__ __align__(16) int lds_st[];
+    __shared__ int wave_lds[4];
+    int* cursor = lds_st;
+    int* cnt = cursor + n_coarse;
+    int* first = cnt + n_coarse;
+    int2* stage = reinterpret_cast<int2*>(first + n_coarse + (n_coarse & 1));
+    unsigned short* sbin = reinterpret_cast<unsigned short*>(stage + kStTile);
+    for (int b = threadIdx.x; b < n_coarse; b += 256) cursor[b] = bin_start[b] + part_off[(size_t)blockIdx.x * n_coarse + b];
+    __syncthreads();
+    const long long begin = (long long)blockIdx.x * per_part;
+    const int e0 = (int)min((long long)total, begin), e1 = (int)min((long long)total, begin + per_part);
+    for (int t0 = e0; t0 < e1; t0 += kStTile) {
+        int2 rec[16];
+        int bin[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            const int e = t0 + 256 * u + (int)threadIdx.x;
+            const int q = e < e1 ? old_idx[e] : -1;
+            const bool ok = q >= 0 && q < N;
+            rec[u] = make_int2(e, q);
+            bin[u] = ok ? q >> cshift : -1;
+        }
+        staged_tile_out(rec, bin, n_coarse, cnt, first, stage, sbin, cursor, wave_lds, out);
+    }
+}
+
+// Sub-parts of coarse bin cb: records [start + s kStSub, ...) for s = 0, 1, ...; their number in the global list of
+// sub-parts is start / kStSub + cb + s (increasing, no two alike: a coarse bin has at most size / kStSub + 1 of them).
+__device__ __forceinline__ int staged_sub_id(int start, int cb, int s) { return start / kStSub + cb + s; }
+
+// (2a) counts of the sub-parts of the coarse bins per fine bin; grid (x: sub-parts walked in turn, y: coarse bin)
+__global__ __launch_bounds__(256) void k_staged_count2(const int2* __restrict__ rec1, const int* __restrict__ cstart, int cshift,
+                                                       int fshift, int* __restrict__ fine_size, int* __restrict__ sub_off)
+{
+    extern __shared__ int hist2[];
+    const int per = 1 << (cshift - fshift);
+    const int cb = blockIdx.y;
+    const int s0 = cstart[cb], s1 = cstart[cb + 1];
+    const int low = (1 << cshift) - 1;
+    for (int s = blockIdx.x; s0 + (long long)s * kStSub < s1; s += gridDim.x) {
+        for (int b = threadIdx.x; b < per; b += 256) hist2[b] = 0;
+        __syncthreads();
+        const int a = s0 + s * kStSub, z = min(s1, a + kStSub);
+        for (int i = a + (int)threadIdx.x; i < z; i += 256) atomicAdd(&hist2[(rec1[i].y & low) >> fshift], 1);
+        __syncthreads();
+        const size_t row = (size_t)staged_sub_id(s0, cb, s) * per;
+        for (int b = threadIdx.x; b < per; b += 256) {
+            const int c = hist2[b];
+            sub_off[row + b] = c ? atomicAdd(&fine_size[(size_t)cb * per + b], c) : 0;
+        }
+        __syncthreads();
+    }
+}
+
+// (2b) the records of the sub-parts to their fine bins
+__global__ __launch_bounds__(256) void k_staged_scatter2(const int2* __restrict__ rec1, const int* __restrict__ cstart, int cshift,
+                                                         int fshift, const int* __restrict__ fine_start,
+                                                         const int* __restrict__ sub_off, int2* __restrict__ out)
+{
+    extern __shared__ __align__(16) int lds_st[];
+    __shared__ int wave_lds[4];
+    const int per = 1 << (cshift - fshift);
+    int* cursor = lds_st;
+    int* cnt = cursor + per;
+    int* first = cnt + per;
+    int2* stage = reinterpret_cast<int2*>(first + per + (per & 1));
+    unsigned short* sbin = reinterpret_cast<unsigned short*>(stage + kStTile);
+    const int cb = blockIdx.y;
+    const int s0 = cstart[cb], s1 = cstart[cb + 1];
+    const int low = (1 << cshift) - 1;
+    for (int s = blockIdx.x; s0 + (long long)s * kStSub < s1; s += gridDim.x) {
+        const size_t row = (size_t)staged_sub_id(s0, cb, s) * per;
+        for (int b = threadIdx.x; b < per; b += 256) cursor[b] = fine_start[(size_t)cb * per + b] + sub_off[row + b];
+        __syncthreads();
+        const int a = s0 + s * kStSub, z = min(s1, a + kStSub);
+        for (int t0 = a; t0 < z; t0 += kStTile) {
+            int2 rec[16];
+            int bin[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int i = t0 + 256 * u + (int)threadIdx.x;
+                rec[u] = i < z ? rec1[i] : make_int2(-1, -1);
+                bin[u] = i < z ? (rec[u].y & low) >> fshift : -1;
+            }
+            staged_tile_out(rec, bin, per, cnt, first, stage, sbin, cursor, wave_lds, out);
+        }
+        __syncthreads();
+    }
+}
+
+// (3) one workgroup per fine bin: row offsets of its points, and its rows -- assembled in LDS and written whole when the
+// bin has at most kStRowsCap entries, entry by entry otherwise.  LDS: cnt[2^fshift] | stage[kStRowsCap].
+__global__ __launch_bounds__(kRowsBlock) void k_staged_rows(const int2* __restrict__ rec2, const int* __restrict__ fine_start,
+                                                            int fshift, int N, int* __restrict__ offs, int* __restrict__ rev)
+{
+    extern __shared__ int lds_rows[];
+    __shared__ int wave_lds[kRowsBlock / 64];
+    const int R = 1 << fshift;
+    int* cnt = lds_rows;
+    int* stage = cnt + R;
+    const int b = blockIdx.x;
+    const int s0 = fine_start[b], s1 = fine_start[b + 1];
+    const int q0 = b << fshift;
+    const int low = R - 1;
+    for (int i = threadIdx.x; i < R; i += kRowsBlock) cnt[i] = 0;
+    __syncthreads();
+    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) atomicAdd(&cnt[rec2[i].y & low], 1);
+    __syncthreads();
+    int carry = 0;
+    for (int c0 = 0; c0 < R; c0 += kRowsBlock) {
+        const int c = c0 + (int)threadIdx.x;
+        const bool in = c < R;
+        const int v = in ? cnt[c] : 0;
+        int tot;
+        const int ex = block_excl_scan(v, &tot, wave_lds);
+        if (in) {
+            cnt[c] = carry + ex;
+            if (q0 + c < N) offs[q0 + c] = s0 + carry + ex;
+        }
+        carry += tot;
+    }
+    __syncthreads();
+    const bool in_lds = s1 - s0 <= kStRowsCap;
+    for (int i = s0 + (int)threadIdx.x; i < s1; i += kRowsBlock) {
+        const int2 eq = rec2[i];
+        const int at = atomicAdd(&cnt[eq.y & low], 1);
+        if (in_lds) stage[at] = eq.x;
+        else rev[s0 + at] = eq.x;
+    }
+    if (in_lds) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < s1 - s0; i += kRowsBlock) rev[s0 + i] = stage[i];
     }
 }
 
@@ -605,6 +820,42 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     w->div_s = 31 + l;
     w->div_m = (uint32_t)((((uint64_t)1 << w->div_s) + (uint64_t)K - 1) / (uint64_t)K);
     auto dm = [](void* p, size_t n) { return ws_alloc(reinterpret_cast<void**>(p), std::max<size_t>(n, 1) * sizeof(int)) ? hipErrorOutOfMemory : hipSuccess; };
+    // Large graphs (2^26 entries and more; RSFK_REV_STAGED=1|0 says otherwise) take the builder that stages its stores
+    // in LDS: fine bins whose rows fit into LDS with room to spare, about as many fine bins per coarse bin as there
+    // are coarse bins.
+    {
+        const char* e = std::getenv("RSFK_REV_STAGED");
+        bool want = total >= ((size_t)1 << 26);
+        if (e && e[0] == '1') want = true;
+        if (e && e[0] == '0') want = false;
+        if (want) {
+            int fs = 5;
+            while (fs < 12 && ((size_t)3 << (fs + 1)) * (size_t)K <= (size_t)2 * kStRowsCap) ++fs;    // 1.5 K 2^fs <= cap
+            const int n_fine = (int)(((size_t)N + ((size_t)1 << fs) - 1) >> fs);
+            int lp = 4;
+            while (lp < 10 && ((size_t)1 << (2 * (lp + 1))) <= (size_t)n_fine) ++lp;                   // 2^lp about sqrt(n_fine)
+            while (lp < 10 && (((size_t)N - 1) >> (fs + lp)) + 1 > (size_t)kStMaxBins) ++lp;
+            const int n_coarse = (int)((((size_t)N - 1) >> (fs + lp)) + 1);
+            if (n_coarse <= kStMaxBins) {
+                w->staged = true;
+                w->fshift = fs;
+                w->cshift = fs + lp;
+                w->n_coarse = n_coarse;
+                w->n_fine = n_coarse << lp;
+                w->n_sub = (int)(total / kStSub) + n_coarse + 2;
+            }
+        }
+    }
+    if (w->staged &&
+        (dm(&w->bin_eq2, 2 * total) != hipSuccess || dm(&w->fine_size, (size_t)w->n_fine) != hipSuccess ||
+         dm(&w->fine_start, (size_t)w->n_fine + 1) != hipSuccess ||
+         dm(&w->sub_off, (size_t)w->n_sub << (w->cshift - w->fshift)) != hipSuccess ||
+         (size_t)w->n_parts * (size_t)w->n_coarse > (size_t)w->n_parts * (size_t)w->n_bins)) {
+        // (the counters of the parts are those of the one-level builder: never fewer bins there than coarse bins here)
+        explore_ws_free(w);
+        set_last_error("exploration workspace: out of device memory");
+        return 1;
+    }
     if (dm(&w->rev, total) != hipSuccess || dm(&w->bin_eq, 2 * total) != hipSuccess ||
         dm(&w->offs, (size_t)N + 1) != hipSuccess || dm(&w->bin_size, (size_t)w->n_bins) != hipSuccess ||
         dm(&w->bin_start, (size_t)w->n_bins + 1) != hipSuccess ||
@@ -630,7 +881,8 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
 void explore_ws_free(ExploreWorkspace* w)
 {
     if (!w) return;
-    void* bufs[] = {w->rev, w->bin_eq, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->norm_tau, w->todo, w->bounds};
+    void* bufs[] = {w->rev, w->bin_eq, w->offs, w->bin_size, w->bin_start, w->part_off, w->pass, w->norm_tau, w->todo, w->bounds,
+                    w->bin_eq2, w->fine_size, w->fine_start, w->sub_off};
     for (void* b : bufs)
         ws_free(b);
     if (w->host_count) (void)hipHostFree(w->host_count);
@@ -650,6 +902,30 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
     RSFK_CHECK(K >= 1 && K <= 256, "exploration join: K must be in 1..256");
     RSFK_CHECK((size_t)N * (size_t)K < kMaxEntries, "exploration join: N*K must be below 2^31 - 4096");
     const int total = (int)((size_t)N * (size_t)K);
+    if (w->staged) {
+        const int nc = w->n_coarse, per = 1 << (w->cshift - w->fshift);
+        hipLaunchKernelGGL(k_zero, dim3((unsigned)((nc + 255) / 256)), dim3(256), 0, stream, w->bin_size, nc, w->todo + N,
+                           w->todo + 2 * (size_t)N + 1);
+        hipLaunchKernelGGL(k_zero, dim3((unsigned)((w->n_fine + 255) / 256)), dim3(256), 0, stream, w->fine_size, w->n_fine,
+                           w->todo + N, w->todo + 2 * (size_t)N + 1);
+        hipLaunchKernelGGL(k_bin_count, dim3((unsigned)w->n_parts), dim3(256), (size_t)nc * sizeof(int), stream, old_idx, total,
+                           w->per_part, N, w->cshift, nc, w->bin_size, w->part_off);
+        hipLaunchKernelGGL(k_bin_scan, dim3(1), dim3(256), 0, stream, w->bin_size, nc, w->bin_start, w->offs + N);
+        hipLaunchKernelGGL(k_staged_scatter1, dim3((unsigned)w->n_parts), dim3(256), staged_lds_bytes(nc), stream, old_idx, total,
+                           w->per_part, N, w->cshift, nc, w->bin_start, w->part_off, w->bin_eq);
+        // sub-parts of a coarse bin walked by a few workgroups each (four times the mean number of sub-parts per bin)
+        const unsigned walkers = (unsigned)std::max<size_t>(1, std::min<size_t>(64, 4 * ((size_t)total / kStSub / (size_t)nc + 1)));
+        hipLaunchKernelGGL(k_staged_count2, dim3(walkers, (unsigned)nc), dim3(256), (size_t)per * sizeof(int), stream, w->bin_eq,
+                           w->bin_start, w->cshift, w->fshift, w->fine_size, w->sub_off);
+        hipLaunchKernelGGL(k_bin_scan, dim3(1), dim3(256), 0, stream, w->fine_size, w->n_fine, w->fine_start, w->offs + N);
+        hipLaunchKernelGGL(k_staged_scatter2, dim3(walkers, (unsigned)nc), dim3(256), staged_lds_bytes(per), stream, w->bin_eq,
+                           w->bin_start, w->cshift, w->fshift, w->fine_start, w->sub_off, w->bin_eq2);
+        const size_t rows_lds = ((size_t)(1 << w->fshift) + kStRowsCap) * sizeof(int);
+        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_staged_rows), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)rows_lds));
+        hipLaunchKernelGGL(k_staged_rows, dim3((unsigned)w->n_fine), dim3(kRowsBlock), rows_lds, stream, w->bin_eq2, w->fine_start,
+                           w->fshift, N, w->offs, w->rev);
+    } else {
     const int nbins = w->n_bins;
     const size_t bin_lds = (size_t)nbins * sizeof(int);
     hipLaunchKernelGGL(k_zero, dim3((unsigned)((nbins + 255) / 256)), dim3(256), 0, stream, w->bin_size, nbins, w->todo + N,
@@ -661,6 +937,7 @@ int launch_explore_join(ExploreWorkspace* w, const Bf16Copy& bf, int N, int D, i
                        w->shift, nbins, w->bin_start, w->part_off, w->bin_eq);
     hipLaunchKernelGGL(k_bin_rows, dim3((unsigned)nbins), dim3(kRowsBlock), sizeof(int) << w->shift, stream, w->bin_eq,
                        w->bin_start, w->shift, N, w->offs, w->rev);
+    }
     hipLaunchKernelGGL(k_norm_tau, dim3((unsigned)((N + 255) / 256)), dim3(256), 0, stream, bf.norms, knn_dist, N, K, w->norm_tau);
     RSFK_HIP(hipGetLastError());
 

@@ -238,7 +238,7 @@ def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
 # ---------------------------------------------------------------------------
 # exploration
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("join", ["join", "plain"])
+@pytest.mark.parametrize("join", ["join", "plain", "staged"])
 @pytest.mark.parametrize("N,D,K,self_in", [(3000, 32, 16, True), (2000, 100, 32, True), (1500, 5, 8, False),
                                            (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True),
                                            (1300, 6, 200, True), (40, 7, 33, True), (5000, 130, 12, True),
@@ -248,10 +248,13 @@ def test_explore_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, self_in, jo
     """Both ways of enumerating the candidates: the join over the reversed graph (default; with partly empty
     rows and a large K its marks overflow the small set; K above about 45 then takes the merge kernel that puts a
     whole workgroup on a point, and the general kernel finishes what is left; rows of more than 128 dimensions have
-    their candidates taken nearer lower bounds first, several hundred per point at 3000 x 200 with K = 32)
-    and every point for itself (RSFK_EXPLORE_JOIN=0)."""
+    their candidates taken nearer lower bounds first, several hundred per point at 3000 x 200 with K = 32),
+    the same with the reversed graph made by the builder for large graphs (RSFK_REV_STAGED=1: two scatters staged in
+    LDS, rows assembled in LDS), and every point for itself (RSFK_EXPLORE_JOIN=0)."""
     if join == "plain":
         monkeypatch.setenv("RSFK_EXPLORE_JOIN", "0")
+    if join == "staged":
+        monkeypatch.setenv("RSFK_REV_STAGED", "1")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K, self_in=self_in)
     MIN = max(2, K // 2)                 # buckets smaller than K+1 leave some rows partly empty
