@@ -247,8 +247,7 @@ constexpr int kStSub = 32768;               // records of a sub-part of a coarse
 constexpr int kStMaxBins = 1024;            // bins a scatter step distinguishes (LDS counters)
 constexpr int kStRowsCap = 24576;           // entries of a fine bin whose rows are assembled in LDS
 
-// counts of a part of the graph per coarse bin (k_bin_count with another shift; kept apart for the record format)
-// -> reuses k_bin_count / k_bin_scan with shift = cshift.
+// (The counts of the parts of the graph per coarse bin are k_bin_count and k_bin_scan with shift = cshift.)
 
 // Sorts up to kStTile records (rec[i], bin[i] for the thread's 16 records) by bin in LDS and writes them to
 // out[cursor[bin] + rank inside (tile, bin)]; cursor (LDS, n_bins ints) moves on by the tile's counts.
@@ -836,7 +835,8 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
             while (lp < 10 && ((size_t)1 << (2 * (lp + 1))) <= (size_t)n_fine) ++lp;                   // 2^lp about sqrt(n_fine)
             while (lp < 10 && (((size_t)N - 1) >> (fs + lp)) + 1 > (size_t)kStMaxBins) ++lp;
             const int n_coarse = (int)((((size_t)N - 1) >> (fs + lp)) + 1);
-            if (n_coarse <= kStMaxBins) {
+            // (the parts' counters and the bins' sizes and starts are the arrays of the one-level builder)
+            if (n_coarse <= kStMaxBins && n_coarse <= w->n_bins) {
                 w->staged = true;
                 w->fshift = fs;
                 w->cshift = fs + lp;
@@ -849,9 +849,7 @@ int explore_ws_alloc(ExploreWorkspace** out, int N, int K, bool with_bounds)
     if (w->staged &&
         (dm(&w->bin_eq2, 2 * total) != hipSuccess || dm(&w->fine_size, (size_t)w->n_fine) != hipSuccess ||
          dm(&w->fine_start, (size_t)w->n_fine + 1) != hipSuccess ||
-         dm(&w->sub_off, (size_t)w->n_sub << (w->cshift - w->fshift)) != hipSuccess ||
-         (size_t)w->n_parts * (size_t)w->n_coarse > (size_t)w->n_parts * (size_t)w->n_bins)) {
-        // (the counters of the parts are those of the one-level builder: never fewer bins there than coarse bins here)
+         dm(&w->sub_off, (size_t)w->n_sub << (w->cshift - w->fshift)) != hipSuccess)) {
         explore_ws_free(w);
         set_last_error("exploration workspace: out of device memory");
         return 1;
