@@ -376,11 +376,36 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     if (slot >= (todo_in ? n_in : N)) return;             // whole wavefront leaves together
     const int p = todo_in ? todo_in[slot] : (order ? order[slot] : slot);
     const int MW = (K + 31) >> 5;
+    int* base = lds_m + (size_t)wave * (size_t)wave_lds_ints;
+    // Rows of at most 64 neighbours (one slot per lane): everything the point needs from memory before its candidates
+    // are known -- its K-NN row, the snapshot of its neighbours, its mark words, its coordinates -- is requested at once;
+    // none of these addresses depends on another's data.  (Longer rows: one after the other, as they are needed.)
+    constexpr bool kEarly = SL == 1;
+    KnnRow<SL> row;
+    int q_own = -1;
+    uint32_t pw[2] = {0u, 0u};
+    if (kEarly) {
+        const size_t at = (size_t)p * K + (lane < K ? lane : 0);
+        row.idx[0] = knn_idx[at];
+        row.dist[0] = knn_dist[at];
+        q_own = old_idx[at];
+        pw[0] = pass[at * MW];
+        if (MW > 1) pw[1] = pass[at * MW + 1];
+        const float* xp0 = points + (size_t)p * D;
+        float* xr = reinterpret_cast<float*>(base + merge_tile_ints(dpad, direct_max));
+        for (int d = lane; d < dpad; d += 64) xr[d] = d < D ? xp0[d] : 0.0f;
+        if (lane >= K) { row.idx[0] = -2; row.dist[0] = INFINITY; q_own = -1; }
+        if (!(q_own >= 0 && q_own < N)) { pw[0] = 0u; pw[1] = 0u; }          // the join writes nothing for such an entry
+    }
     int bits = 0;
-    for (int k = lane; k < K; k += 64) {
-        const int j = graph_entry(old_idx, N, K, p, k);
-        if (j >= 0)
-            for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
+    if (kEarly) {
+        bits = __popc(pw[0]) + __popc(pw[1]);
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const int j = graph_entry(old_idx, N, K, p, k);
+            if (j >= 0)
+                for (int w = 0; w < MW; ++w) bits += __popc(pass[(size_t)j * MW + w]);
+        }
     }
     const int n_given = wave_sum_i(bits);
     if (n_given == 0) return;
@@ -388,7 +413,6 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
         if (lane == 0) todo_out[atomicAdd(n_out, 1)] = p;
         return;
     }
-    int* base = lds_m + (size_t)wave * (size_t)wave_lds_ints;
     ExploreLds L;
     L.tile = reinterpret_cast<float*>(base);
     const int tile_ints = merge_tile_ints(dpad, direct_max);
@@ -402,11 +426,15 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     const int KP = (K + 31) & ~31;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
-    KnnRow<SL> row;
-    row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
-    for (int k = lane; k < K; k += 64) L.srow[k] = old_idx[(size_t)p * K + k];
-    const float* xp = points + (size_t)p * D;
-    for (int d = lane; d < dpad; d += 64) L.xrow[d] = d < D ? xp[d] : 0.0f;
+    if (kEarly) {
+        row.init_from_regs(K);
+        if (lane < K) L.srow[lane] = q_own;
+    } else {
+        row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
+        for (int k = lane; k < K; k += 64) L.srow[k] = old_idx[(size_t)p * K + k];
+        const float* xp = points + (size_t)p * D;
+        for (int d = lane; d < dpad; d += 64) L.xrow[d] = d < D ? xp[d] : 0.0f;
+    }
 
     int ts = 64;
     while (ts < 2 * (n_given + K + 1)) ts <<= 1;
@@ -427,14 +455,15 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     int n_marked = 0;                                     // wave-uniform
     for (int k0 = 0; k0 < K; k0 += 64) {
         const int k = k0 + lane;
-        const int j = k < K ? graph_entry(old_idx, N, K, p, k) : -1;
+        const int j = kEarly ? (q_own >= 0 && q_own < N ? p * K + k : -1) : (k < K ? graph_entry(old_idx, N, K, p, k) : -1);
         int mine = 0;
-        if (j >= 0)
+        if (kEarly) mine = bits;
+        else if (j >= 0)
             for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
         int at = n_marked + wave_excl_scan_i(mine);
         if (j >= 0) {
             for (int w = 0; w < MW; ++w) {
-                uint32_t m = pass[(size_t)j * MW + w];
+                uint32_t m = kEarly ? pw[w & 1] : pass[(size_t)j * MW + w];
                 while (m) {
                     const int b = __ffs(m) - 1;
                     m &= m - 1;
@@ -445,21 +474,30 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
         n_marked += wave_sum_i(mine);
     }
     wave_lds_sync();
-    for (int i0 = 0; i0 < n_marked; i0 += 64) {
-        const int i = i0 + lane;
-        int c = -1, lb = 0;
-        if (i < n_marked) {
-            const int e = marked[i];
-            c = old_idx[(size_t)L.srow[e & 255] * K + (e >> 8)];
-            // the join's lower bound of the pair: entry p K + k of the graph, column = slot in the neighbour's row
-            if (bounds) lb = bounds[((size_t)p * K + (e & 255)) * (size_t)KP + (e >> 8)];
+    // (the ids of 256 marks are requested together: a point's marks then cost one trip to memory, not one per 64)
+    for (int i0 = 0; i0 < n_marked; i0 += 256) {
+        int c[4], lb[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = i0 + 64 * u + lane;
+            c[u] = -1;
+            lb[u] = 0;
+            if (i < n_marked) {
+                const int e = marked[i];
+                c[u] = old_idx[(size_t)L.srow[e & 255] * K + (e >> 8)];
+                // the join's lower bound of the pair: entry p K + k of the graph, column = slot in the neighbour's row
+                if (bounds) lb[u] = bounds[((size_t)p * K + (e & 255)) * (size_t)KP + (e >> 8)];
+            }
         }
-        if (c >= 0 && c < N) {
-            if (tbound) {
-                const int at = set_insert_at(L.table, mask, c);
-                if (at >= 0) atomicMin(&tbound[at], lb);
-            } else {
-                set_insert(L.table, mask, c, false);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (c[u] >= 0 && c[u] < N) {
+                if (tbound) {
+                    const int at = set_insert_at(L.table, mask, c[u]);
+                    if (at >= 0) atomicMin(&tbound[at], lb[u]);
+                } else {
+                    set_insert(L.table, mask, c[u], false);
+                }
             }
         }
     }
