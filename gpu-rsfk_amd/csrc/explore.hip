@@ -651,17 +651,24 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
     float* seen_d = old_d + kq;                                   // [4][kq]: the rows of the wavefronts as they last showed them
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
+    // thread k takes neighbour k (K <= 256): its entry of the snapshot and its mark words are requested together with
+    // the point's row and coordinates (none of these addresses depends on another's data)
+    const int k = threadIdx.x;
+    const size_t entry = (size_t)p * K + (k < K ? k : 0);
+    const int q_own = old_idx[entry];
+    uint32_t pw[8];                                               // MW <= 8
+#pragma unroll
+    for (int w = 0; w < 8; ++w) pw[w] = w < MW ? pass[entry * MW + w] : 0u;
     KnnRow<SL> row;
     row.load(knn_idx + (size_t)p * K, knn_dist + (size_t)p * K, K);
     const float* xp = points + (size_t)p * D;
     for (int d = threadIdx.x; d < dpad; d += 256) xrow[d] = d < D ? xp[d] : 0.0f;
     for (int i = threadIdx.x; i < kWgTable; i += 256) table[i] = kEmpty;
 
-    // ---- 1. the marked pairs of the point; thread k takes neighbour k (K <= 256)
-    const int k = threadIdx.x;
-    const int j = k < K ? graph_entry(old_idx, N, K, p, k) : -1;
+    // ---- 1. the marked pairs of the point
+    const int j = k < K && q_own >= 0 && q_own < N ? (int)entry : -1;     // (the join writes nothing for other entries)
     if (k < K) {
-        srow[k] = old_idx[(size_t)p * K + k];
+        srow[k] = q_own;
         jrow[k] = j;
     }
 #pragma unroll
@@ -672,8 +679,10 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         }
     }
     int mine = 0;
-    if (j >= 0)
-        for (int w = 0; w < MW; ++w) mine += __popc(pass[(size_t)j * MW + w]);
+    if (j >= 0) {
+#pragma unroll
+        for (int w = 0; w < 8; ++w) mine += __popc(pw[w]);
+    }
     const int in_wave = wave_excl_scan_i(mine);
     if (lane == 63) wave_tot[wave] = in_wave + mine;
     if (threadIdx.x == 0) {
@@ -693,8 +702,9 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         return;
     }
     if (j >= 0) {
-        for (int w = 0; w < MW; ++w) {
-            uint32_t m = pass[(size_t)j * MW + w];
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            uint32_t m = pw[w];
             while (m) {
                 const int b = __ffs(m) - 1;
                 m &= m - 1;
