@@ -137,18 +137,22 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
+    const size_t first = starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride;     // (asked for together with s)
     if (s < 2 || s > kCap) return;
-    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int* bid = ids + first;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
     const int n_chunks = SINGLE ? 1 : (D + kChunk - 1) / kChunk;
     const int fm = wave + 2 * lane;                       // bit u of a member set: member wave + 2 u
     const int* lids = M.lids;
 
+    // (a member's last slot is requested here and put into LDS once the rows have been requested too: the two trips to
+    // memory then overlap; nobody reads the last slots before the bounds)
+    float tau_own = 0.0f;
     if (tid < kCap) {
         const int id = tid < s ? bid[tid] : -1;
         M.lids[tid] = id;
-        M.tau[tid] = id >= 0 ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : 0.0f;
+        if (id >= 0) tau_own = knn_dist[(size_t)id * (size_t)K + (K - 1)];
         M.cand[tid] = 0ull;
     }
     if (tid == kCap) M.n_pairs[0] = 0;
@@ -166,6 +170,7 @@ __device__ __forceinline__ void screen_bucket_body(float* __restrict__ lds, cons
         const float* pa = rows + (32 * wave + (lane & 31)) * kPitch + 8 * (lane >> 5);
         const float* pb = rows + (32 + (lane & 31)) * kPitch + 8 * (lane >> 5);
         ld.request(lids, s, points, D, (n_chunks - 1) * kChunk, vec_ok);
+        if (tid < kCap) M.tau[tid] = tau_own;
         for (int step = 0; step < n_chunks; ++step) {
             const int c = n_chunks - 1 - step;           // the last chunk first
             if (!SINGLE && step > 0) __syncthreads();    // the previous chunk has been consumed

@@ -110,15 +110,19 @@ __device__ __forceinline__ void small_bucket_body(float* __restrict__ lds_f, con
 
     const int bkt = blockIdx.x;
     const int s = sizes[bkt];
+    const size_t first = starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride;     // (asked for together with s)
     if (s < min_size || s > kCap) return;
-    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int* bid = ids + first;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
 
+    // (a member's last slot is requested here and put into LDS once the first rows have been requested too: the two
+    // trips to memory then overlap; nobody reads the last slots before the distances are there)
+    float tau_own = INFINITY;
     if (tid < kCap) {
         const int id = tid < s ? bid[tid] : -1;
         lids[tid] = id;
-        tau[tid] = (rows_sorted && id >= 0) ? knn_dist[(size_t)id * (size_t)K + (K - 1)] : INFINITY;
+        if (rows_sorted && id >= 0) tau_own = knn_dist[(size_t)id * (size_t)K + (K - 1)];
         flag[tid] = 0;
     }
     __syncthreads();
@@ -171,6 +175,7 @@ __device__ __forceinline__ void small_bucket_body(float* __restrict__ lds_f, con
                 }
             }
         }
+        if (d0 == 0 && tid < kCap) tau[tid] = tau_own;
         if (d0 > 0) __syncthreads();                 // the previous chunk has been consumed
 #pragma unroll
         for (int i = 0; i < kMaxLoads; ++i) {
