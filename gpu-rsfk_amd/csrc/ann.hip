@@ -387,7 +387,7 @@ int launch_ann_tree(const float* points, const float* queries, int NQ, int D, in
                     hipStream_t stream)
 {
     if (NQ <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 256, "query-set search: K must be in 1..256");
+    RSFK_CHECK(K >= 1 && K <= kMaxK, "query-set search: K must be in 1..1024");
     RSFK_CHECK(recs != nullptr && rec_cap >= 1, "query-set search: the tree has no index");
     int* q_rec = ws;
     int* q_rank = q_rec + NQ;
@@ -429,7 +429,9 @@ int launch_ann_tree(const float* points, const float* queries, int NQ, int D, in
     }
     if (K <= 64) RSFK_ANN_CASE(1)
     else if (K <= 128) RSFK_ANN_CASE(2)
-    else RSFK_ANN_CASE(4)
+    else if (K <= 256) RSFK_ANN_CASE(4)
+    else if (K <= 512) RSFK_ANN_CASE(8)
+    else RSFK_ANN_CASE(16)
 #undef RSFK_ANN_CASE
     RSFK_HIP(hipGetLastError());
     return 0;

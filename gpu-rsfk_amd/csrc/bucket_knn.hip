@@ -19,7 +19,7 @@
 //
 // k_bucket_knn_small (bucket_knn_small.hip): buckets of at most 64 points,
 //     K <= 64 -- the shape the default parameters produce.
-// k_bucket_knn (this file): any bucket size, any K <= 256, 64x64 tiles of the
+// k_bucket_knn (this file): any bucket size, any K <= 1024, 64x64 tiles of the
 //     pair matrix, rows and columns of a tile updated in turn.
 #include "rsfk_common.hpp"
 #include "knn_list.hpp"
@@ -275,7 +275,9 @@ int launch_general(const float* points, int D, int K, const int* ids, const int*
     } while (0)
     if (K <= 64) RSFK_GENERAL_CASE(1);
     else if (K <= 128) RSFK_GENERAL_CASE(2);
-    else RSFK_GENERAL_CASE(4);
+    else if (K <= 256) RSFK_GENERAL_CASE(4);
+    else if (K <= 512) RSFK_GENERAL_CASE(8);
+    else RSFK_GENERAL_CASE(16);
 #undef RSFK_GENERAL_CASE
     RSFK_HIP(hipGetLastError());
     return 0;
@@ -344,9 +346,9 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
                       hipStream_t stream)
 {
     if (n_buckets <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
+    RSFK_CHECK(K >= 1 && K <= kMaxK, "bucket K-NN: K must be in 1..1024");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
-    if (bucket_gram_from() == 0) {
+    if (bucket_gram_from() == 0 && K <= kMaxKJoin) {
         // RSFK_GRAM_FROM=0: the screened kernel for every call; it needs sorted rows and the size of the largest bucket
         if (launch_sort_rows(knn_idx, knn_dist, N, K, stream)) return 1;
         if (max_bucket < 0 && largest_bucket(sizes, n_buckets, stream, &max_bucket)) return 1;
@@ -392,11 +394,11 @@ int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_s
                            int leaf_cap, int n_small, int n_big, int max_bucket, int* knn_idx, float* knn_dist,
                            hipStream_t stream, int part, bool young_rows, int* launched)
 {
-    RSFK_CHECK(K >= 1 && K <= 256, "bucket K-NN: K must be in 1..256");
+    RSFK_CHECK(K >= 1 && K <= kMaxK, "bucket K-NN: K must be in 1..1024");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
     int none = 0;
     int& used = launched ? *launched : none;              // which kernels this tree's buckets went to (kBucketKernel...)
-    if (gram && rows_sorted) {
+    if (gram && rows_sorted && K <= kMaxKJoin) {
         used |= kBucketKernelGram;
         // pair matrix screened on the matrix cores; buckets of 65..72 points (K <= 64) keep their own kernel
         if (n_small > 0 && part != 2 &&

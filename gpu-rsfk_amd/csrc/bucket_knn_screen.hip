@@ -445,11 +445,13 @@ __global__ __launch_bounds__(256) void k_sort_rows(int* __restrict__ knn_idx, fl
 int launch_sort_rows(int* knn_idx, float* knn_dist, int N, int K, hipStream_t stream)
 {
     if (N <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 256, "sort rows: K must be in 1..256");
+    RSFK_CHECK(K >= 1 && K <= kMaxK, "sort rows: K must be in 1..1024");
     const dim3 grid((unsigned)((N + 3) / 4)), block(256);
     if (K <= 64) hipLaunchKernelGGL(k_sort_rows<1>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
     else if (K <= 128) hipLaunchKernelGGL(k_sort_rows<2>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
-    else hipLaunchKernelGGL(k_sort_rows<4>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    else if (K <= 256) hipLaunchKernelGGL(k_sort_rows<4>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    else if (K <= 512) hipLaunchKernelGGL(k_sort_rows<8>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
+    else hipLaunchKernelGGL(k_sort_rows<16>, grid, block, 0, stream, knn_idx, knn_dist, N, K);
     RSFK_HIP(hipGetLastError());
     return 0;
 }

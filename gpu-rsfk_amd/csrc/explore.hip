@@ -1060,7 +1060,7 @@ bool explore_merge_uses_bounds(int D, int K)
 bool explore_merge_fits(int D, int K)
 {
     const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
-    return 4 * merge_wave_ints(small_table, bf16_valid(D), K) <= 150 * 1024 / 4;
+    return K <= kMaxKJoin && 4 * merge_wave_ints(small_table, bf16_valid(D), K) <= 150 * 1024 / 4;
 }
 
 // ws may be null; with a workspace and a bfloat16 copy for the join (bf_join, may be centred; bf must not be)
@@ -1071,7 +1071,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
                    unsigned long long* stat, const int* order)
 {
     if (N <= 0) return 0;
-    RSFK_CHECK(K >= 1 && K <= 256, "exploration: K must be in 1..256");
+    RSFK_CHECK(K >= 1 && K <= kMaxK, "exploration: K must be in 1..1024");
     RSFK_CHECK(bf == nullptr || bf->mu == nullptr, "exploration: the general kernel needs an uncentred copy");
     const int dpad = bf16_valid(D);
     const int small_table = std::min(4096, std::max(256, next_pow2(16 * K)));
@@ -1099,7 +1099,7 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
     const int wave_ints = (fixed + table + 3) / 4 * 4;
     Bf16Copy b;
     if (bf) b = *bf;
-    const int sl = K <= 64 ? 1 : (K <= 128 ? 2 : 4);
+    const int sl = row_slots(K);
     const int* todo = nullptr;
     int n_todo = 0;
     if (join) {
@@ -1161,6 +1161,8 @@ int launch_explore(const float* points, const Bf16Copy* bf, const Bf16Copy* bf_j
     RSFK_EXPLORE_CASE(1, 4) RSFK_EXPLORE_CASE(1, 2) RSFK_EXPLORE_CASE(1, 1)
     RSFK_EXPLORE_CASE(2, 4) RSFK_EXPLORE_CASE(2, 2) RSFK_EXPLORE_CASE(2, 1)
     RSFK_EXPLORE_CASE(4, 4) RSFK_EXPLORE_CASE(4, 2) RSFK_EXPLORE_CASE(4, 1)
+    RSFK_EXPLORE_CASE(8, 4) RSFK_EXPLORE_CASE(8, 2) RSFK_EXPLORE_CASE(8, 1)
+    RSFK_EXPLORE_CASE(16, 4) RSFK_EXPLORE_CASE(16, 2) RSFK_EXPLORE_CASE(16, 1)
 #undef RSFK_EXPLORE_CASE
     RSFK_CHECK(false, "exploration: no kernel for this configuration");
 }

@@ -783,12 +783,13 @@ __global__ __launch_bounds__(256) void k_explore_join_wg(Bf16Copy bf, int N, int
 
 }  // namespace
 
-// The join is used unless RSFK_EXPLORE_JOIN=0 is set, the graph has about 2^31 or more entries or N is beyond what the
+// The join is used unless RSFK_EXPLORE_JOIN=0 is set, K is above 256, the graph has about 2^31 or more entries or N is beyond what the
 // builder of the reversed graph takes (6144 bins of 2^13 points).
 bool explore_join_enabled(int N, int K)
 {
     const char* env = std::getenv("RSFK_EXPLORE_JOIN");
     if (env && env[0] == '0') return false;
+    if (K > kMaxKJoin) return false;          // (rows of more than 256 neighbours: the general kernel only)
     int shift, n_bins;
     return (size_t)N * (size_t)K < kMaxEntries && rev_bins(N, &shift, &n_bins);
 }

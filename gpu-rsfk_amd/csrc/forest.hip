@@ -214,7 +214,7 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
 {
     RSFK_CHECK(N >= 1 && D >= 1 && K >= 1, "forest: N, D and K must be positive");
     RSFK_CHECK(n_trees >= 0, "forest: n_trees must not be negative");
-    RSFK_CHECK(K <= 256, "forest: K above 256 is not supported");
+    RSFK_CHECK(K <= kMaxK, "forest: K above 1024 is not supported");
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
     if (n_trees == 0 && nnef <= 0) return 0;          // nothing to do: no copies are made, nothing is queued
     const double t_forest0 = now_s();
@@ -392,7 +392,7 @@ int knn_ann_forest_device(int n_trees, int K, int N, int NQ, int D, int MIN, int
 {
     RSFK_CHECK(N >= 1 && D >= 1 && K >= 1 && NQ >= 0, "query-set search: N, D and K must be positive");
     RSFK_CHECK(n_trees >= 0, "query-set search: n_trees must not be negative");
-    RSFK_CHECK(K <= 256, "query-set search: K above 256 is not supported");
+    RSFK_CHECK(K <= kMaxK, "query-set search: K above 1024 is not supported");
     if (log_forest) std::memset(log_forest, 0, sizeof(float) * ((size_t)16 * n_trees + 2));
     const double t0 = now_s();
     if (n_trees > 0 && NQ > 0) {

@@ -125,7 +125,9 @@ int sym_launch_flags(const int* idx, int N, int K, int drop_self, unsigned char*
     const dim3 grid((unsigned)((N + 3) / 4)), block(256);
     if (K <= 64) hipLaunchKernelGGL(k_sym_flags<1>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
     else if (K <= 128) hipLaunchKernelGGL(k_sym_flags<2>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
-    else hipLaunchKernelGGL(k_sym_flags<4>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
+    else if (K <= 256) hipLaunchKernelGGL(k_sym_flags<4>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
+    else if (K <= 512) hipLaunchKernelGGL(k_sym_flags<8>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
+    else hipLaunchKernelGGL(k_sym_flags<16>, grid, block, 0, stream, idx, N, K, drop_self, flag, n_own, extra);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -138,8 +140,12 @@ int sym_launch_fill(const int* idx, const float* dist, int N, int K, const unsig
         hipLaunchKernelGGL(k_sym_fill<1>, grid, block, 0, stream, idx, dist, N, K, flag, n_own, cursor, indptr, cols, vals);
     else if (K <= 128)
         hipLaunchKernelGGL(k_sym_fill<2>, grid, block, 0, stream, idx, dist, N, K, flag, n_own, cursor, indptr, cols, vals);
-    else
+    else if (K <= 256)
         hipLaunchKernelGGL(k_sym_fill<4>, grid, block, 0, stream, idx, dist, N, K, flag, n_own, cursor, indptr, cols, vals);
+    else if (K <= 512)
+        hipLaunchKernelGGL(k_sym_fill<8>, grid, block, 0, stream, idx, dist, N, K, flag, n_own, cursor, indptr, cols, vals);
+    else
+        hipLaunchKernelGGL(k_sym_fill<16>, grid, block, 0, stream, idx, dist, N, K, flag, n_own, cursor, indptr, cols, vals);
     RSFK_HIP(hipGetLastError());
     return 0;
 }
@@ -157,7 +163,7 @@ struct Buf {
 int symmetrize_device(const int* d_idx, const float* d_dist, int N, int K, int drop_self, int* d_indptr, int* d_cols,
                       float* d_vals, long long cap, long long* nnz, hipStream_t stream)
 {
-    RSFK_CHECK(N >= 1 && K >= 1 && K <= 256, "graph export: N must be positive and K in 1..256");
+    RSFK_CHECK(N >= 1 && K >= 1 && K <= kMaxK, "graph export: N must be positive and K in 1..1024");
     RSFK_CHECK((long long)N * K < (1ll << 30), "graph export: N * K of 2^30 and more is not supported");
     RSFK_CHECK(d_idx && d_indptr && nnz, "graph export: null argument");
     RSFK_CHECK((d_cols == nullptr) == (d_vals == nullptr), "graph export: indices and data go together");
@@ -264,7 +270,7 @@ __global__ __launch_bounds__(256) void k_zero_counters(int* __restrict__ v, int 
 int symmetrize_count_noalloc(const int* d_idx, int N, int K, int drop_self, int* d_indptr, long long* nnz, hipStream_t stream)
 {
     RSFK_CHECK(d_idx && d_indptr, "graph export: null argument");
-    RSFK_CHECK(N >= 1 && K >= 1 && K <= 256, "graph export: N must be positive and K in 1..256");
+    RSFK_CHECK(N >= 1 && K >= 1 && K <= kMaxK, "graph export: N must be positive and K in 1..1024");
     RSFK_CHECK(N <= kNaMaxPoints && (long long)N * K <= kNaMaxSlots,
                "graph export without allocation: at most 2^20 points and 2^25 neighbour slots (N * K)");
     unsigned char* base = nullptr;

@@ -124,6 +124,15 @@ struct TreeRec {
 // tree builder keeps them apart from the larger ones.
 constexpr int kBucketSplit = 64;
 
+// A K-NN row is the register state of one wavefront: slot k in lane k % 64, register k / 64 (knn_list.hpp).  The
+// kernels are compiled for 1, 2, 4, 8 and 16 registers per lane, so K may be at most 1024.  (The reference scans a row
+// of any K from global memory: src/kernels/compute_knn_from_buckets.cu:1035-1099.)
+constexpr int kMaxK = 1024;
+inline int row_slots(int K) { return K <= 64 ? 1 : (K <= 128 ? 2 : (K <= 256 ? 4 : (K <= 512 ? 8 : 16))); }
+// Rows of more than this many neighbours take the general kernels only: the specialised ones (reversed-graph join,
+// merge kernels, pair matrix on the matrix cores) keep per-neighbour state of a row in 256 threads or in LDS.
+constexpr int kMaxKJoin = 256;
+
 // bit 31 of a permutation entry marks "right side" during a split; ids use the low 31 bits
 constexpr int kIdMask = 0x7fffffff;
 

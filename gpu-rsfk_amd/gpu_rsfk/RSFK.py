@@ -30,7 +30,7 @@ def random_motion(points, random_motion_force):
         points[:, d] = points[:, d] + random_motion_force * np.random.uniform(-range_uniform, range_uniform, N)
 
 
-MAX_NEIGHBORS = 256      # a K-NN row is held by one wavefront, up to four slots per lane
+MAX_NEIGHBORS = 1024     # a K-NN row is held by one wavefront, up to sixteen slots per lane
 
 
 def _check_sizes(points, K, n_trees=0):

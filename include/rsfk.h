@@ -14,7 +14,7 @@
  * rows unordered, empty slot = (-1, +inf or FLT_MAX).  The library merges into
  * whatever the K-NN arrays hold on entry; it never resets them.
  * All calls use the current HIP device and block until their results are
- * complete.  K is limited to 256.
+ * complete.  K is limited to 1024.
  */
 #ifndef RSFK_H
 #define RSFK_H

@@ -90,6 +90,7 @@ def test_tree_edge_cases(gpu, orc, rng):
     (2000, 32, 16, 17, 34), (3000, 100, 32, 33, 66), (3000, 33, 8, 100, 300), (1500, 7, 90, 91, 182),
     (1200, 1, 4, 5, 10), (2500, 3, 1, 2, 4), (2000, 130, 64, 65, 130), (1500, 20, 65, 66, 140),
     (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
+    (2500, 10, 300, 301, 620), (4200, 6, 700, 701, 1500), (1600, 40, 1024, 400, 900),
 ])
 @pytest.mark.parametrize("kernel", ["direct", "direct_per_bucket", "gram", "screen"])
 def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
@@ -243,7 +244,7 @@ def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
                                            (1200, 9, 90, True), (900, 3, 1, True), (2500, 20, 40, True),
                                            (1300, 6, 200, True), (40, 7, 33, True), (5000, 130, 12, True),
                                            (2200, 24, 64, True), (1600, 300, 100, True), (2600, 48, 20, True),
-                                           (3000, 200, 32, True)])
+                                           (3000, 200, 32, True), (1100, 6, 300, True), (800, 5, 520, False)])
 def test_explore_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, self_in, join):
     """Both ways of enumerating the candidates: the join over the reversed graph (default; with partly empty
     rows and a large K its marks overflow the small set; K above about 45 then takes the merge kernel that puts a
@@ -254,6 +255,8 @@ def test_explore_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, self_in, jo
     if join == "plain":
         monkeypatch.setenv("RSFK_EXPLORE_JOIN", "0")
     if join == "staged":
+        if K > 256:
+            pytest.skip("rows of more than 256 neighbours never take the join")
         monkeypatch.setenv("RSFK_REV_STAGED", "1")
     X = rng.random((N, D), dtype=np.float32)
     oi, od = orc.init_lists(N, K, self_in=self_in)
@@ -305,6 +308,8 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
     (5000, 16, 8, 3, dict(min_tree_children=4, max_tree_children=9)),          # second call with K+1 .. 3(K+1)
     (6000, 24, 40, 3, dict(nn_exploring_factor=2)),
     (4000, 12, 10, 2, dict(point_in_self_neigh=False, nn_exploring_factor=0)),
+    (4000, 10, 300, 2, dict(nn_exploring_factor=1)),                           # eight slots per lane
+    (1400, 8, 520, 2, dict(nn_exploring_factor=1, min_tree_children=200, max_tree_children=500)),   # sixteen
 ])
 @pytest.mark.parametrize("variant", ["default", "bucket_screen"])
 def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, T, kw, variant):
@@ -644,6 +649,8 @@ def test_queries_reach_the_leaf_the_oracle_routes_them_to(gpu, orc, rng, N, NQ, 
     (9000, 500, 50, 100, 3, {}),
     (7000, 2000, 33, 200, 2, dict(min_tree_children=40, max_tree_children=90, ensure_valid_indices=False)),
     (300, 50, 7, 5, 4, {}),
+    (6000, 800, 12, 300, 2, {}),
+    (5000, 300, 9, 700, 2, {}),
 ])
 def test_find_nearest_neighbors_ann_matches_oracle(gpu, orc, rng, N, NQ, D, K, T, kw):
     import gpu_rsfk
@@ -712,7 +719,7 @@ def test_ann_recall_rises_with_the_number_of_trees(gpu, rng):
 # symmetrised graph export
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("N,K,drop_self", [(5000, 16, True), (3000, 100, False), (2000, 200, True), (1, 3, False),
-                                           (700, 1, True)])
+                                           (700, 1, True), (900, 300, True), (700, 1000, False)])
 def test_symmetric_graph_matches_oracle(gpu, orc, rng, N, K, drop_self):
     import gpu_rsfk
     idx = np.stack([rng.permutation(max(N, K + 1))[:K] for _ in range(N)]).astype(np.int32)
@@ -898,4 +905,28 @@ def test_random_shapes_match_oracle(gpu, orc, seed):
     assert_knn_equal(ai, ad, qi, qd)
     ip, cc, vv = gpu_rsfk.symmetric_knn_graph(gi, gd, drop_self=bool(seed & 1))
     op, oc, ov = orc.symmetrize(gi, gd, drop_self=bool(seed & 1))
+    assert np.array_equal(ip, op) and np.array_equal(cc, oc) and np.array_equal(vv, ov)
+
+
+@pytest.mark.parametrize("N,D,K,nnef", [(1500, 3, 400, 1), (2400, 2, 1024, 0)])
+def test_rows_of_many_neighbours_on_tied_data(gpu, orc, N, D, K, nnef):
+    """Rows of more than 256 neighbours (eight and sixteen slots per lane) on grid data, where most distances are tied
+    and points are duplicated: graph (with an exploration pass in the smaller case), query-set search and graph export."""
+    import gpu_rsfk
+    g = np.random.default_rng(K)
+    X = g.integers(0, 6, (N, D)).astype(np.float32)
+    _say("many neighbours, tied data", N, D, K)
+    r = gpu_rsfk.RSFK(random_state=5)
+    gi, gd = r.find_nearest_neighbors(X, K, n_trees=2, min_tree_children=K // 2, max_tree_children=K + 50,
+                                      nn_exploring_factor=nnef, ensure_valid_indices=False)
+    oi, od = orc.forest(X, K, 2, K // 2, K + 50, 5000, 5, nnef)
+    assert_knn_equal(gi, gd, oi, od)
+    assert rows_have_no_duplicates(gi)
+    Q = X[::5] + np.float32(0.25)
+    ai, ad = r.find_nearest_neighbors_ann(X, Q, K, n_trees=2, min_tree_children=K // 2, max_tree_children=K + 50,
+                                          ensure_valid_indices=False)
+    qi, qd = orc.ann_forest(X, Q, K, 2, K // 2, K + 50, 5000, 5)
+    assert_knn_equal(ai, ad, qi, qd)
+    ip, cc, vv = gpu_rsfk.symmetric_knn_graph(gi, gd, drop_self=True)
+    op, oc, ov = orc.symmetrize(gi, gd, drop_self=True)
     assert np.array_equal(ip, op) and np.array_equal(cc, oc) and np.array_equal(vv, ov)

@@ -153,12 +153,12 @@ def test_golden_vectors_still_come_out_of_the_oracle(orc):
 
 
 def test_sizes_the_library_would_refuse_raise_in_python(capi):
-    """K above 256, no rows, negative n_trees: an exception before the call, not exit(1) inside the library."""
+    """K above 1024, no rows, negative n_trees: an exception before the call, not exit(1) inside the library."""
     import gpu_rsfk
     r = gpu_rsfk.RSFK(random_state=0)
     X = np.zeros((10, 3), np.float32)
     with pytest.raises(ValueError):
-        r.find_nearest_neighbors(X, 300)
+        r.find_nearest_neighbors(X, 1025)
     with pytest.raises(ValueError):
         r.find_nearest_neighbors(X, 0)
     with pytest.raises(ValueError):
