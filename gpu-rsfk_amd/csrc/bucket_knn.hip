@@ -38,7 +38,7 @@ constexpr int kStripBuckets = 4096;  // launches over at most this many buckets 
 // ---------------------------------------------------------------------------
 // general kernel
 // ---------------------------------------------------------------------------
-struct BucketKnnLds {
+struct alignas(16) BucketKnnLds {
     float a[kTile * kDCP];
     float b[kTile * kDCP];
     float dist[kTile * kDistPitch];
@@ -250,14 +250,224 @@ __global__ __launch_bounds__(256) void k_bucket_knn(const float* __restrict__ po
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// every pair once: the distances of a launch's buckets go through memory
+// ---------------------------------------------------------------------------
+// The chains of one tile: NRB x NCB blocks of 16 x 16 pairs (a thread has one pair of each block), DIAG: a tile on the
+// diagonal, only the blocks on and above the diagonal.  Rows of the two tiles come through LDS 32 dimensions at a time,
+// the next 32 on their way while these are used.
+template <int NRB, int NCB, bool DIAG>
+__device__ __forceinline__ void pair_tile_chains(BucketKnnLds& L, const float* __restrict__ points, int D, int rows, int cols,
+                                                 bool vec_ok, float (&acc)[4][4])
+{
+    const int tid = threadIdx.x;
+    const int ty = tid >> 4, tx = tid & 15;
+    StagedRows sa, sb;
+    sa.request(L.ida, rows, points, D, 0, vec_ok);
+    if (!DIAG) sb.request(L.idb, cols, points, D, 0, vec_ok);
+    const float* B = DIAG ? L.a : L.b;
+    for (int d0 = 0; d0 < D; d0 += kDC) {
+        sa.commit(L.a);
+        if (!DIAG) sb.commit(L.b);
+        __syncthreads();
+        if (d0 + kDC < D) {
+            sa.request(L.ida, rows, points, D, d0 + kDC, vec_ok);
+            if (!DIAG) sb.request(L.idb, cols, points, D, d0 + kDC, vec_ok);
+        }
+#pragma unroll 2
+        for (int dd = 0; dd < kDC; dd += 4) {
+            float4 av[NRB], bv[NCB];
+#pragma unroll
+            for (int r = 0; r < NRB; ++r) av[r] = *reinterpret_cast<const float4*>(&L.a[(ty + 16 * r) * kDCP + dd]);
+#pragma unroll
+            for (int c = 0; c < NCB; ++c) bv[c] = *reinterpret_cast<const float4*>(&B[(tx + 16 * c) * kDCP + dd]);
+#pragma unroll
+            for (int r = 0; r < NRB; ++r) {
+#pragma unroll
+                for (int c = 0; c < NCB; ++c) {
+                    if (DIAG && c < r) continue;
+                    float df;
+                    df = av[r].x - bv[c].x; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                    df = av[r].y - bv[c].y; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                    df = av[r].z - bv[c].z; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                    df = av[r].w - bv[c].w; acc[r][c] = __builtin_fmaf(df, df, acc[r][c]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// k_bucket_pairs: workgroup (bucket, I, J >= I) evaluates the 64 x 64 tile (I, J) of the bucket's pair matrix -- the
+// chains of k_bucket_knn, one pair per accumulator -- and stores it, and its mirror image (J, I), into the bucket's
+// matrix of `pitch` x `pitch` floats (pitch = 64 x the largest number of tiles of a bucket of the launch).  No row is
+// touched: every tile of every bucket is a workgroup of its own, whatever the number of buckets, and no pair is
+// evaluated from both ends.  k_bucket_merge_pairs (below) then gives every member its row of that matrix.
+// tri = max_tiles (max_tiles + 1) / 2 workgroups per bucket; those beyond a bucket's own tiles leave at once.
+__global__ __launch_bounds__(256) void k_bucket_pairs(const float* __restrict__ points, int D, const int* __restrict__ ids,
+                                                       const int* __restrict__ starts, const int* __restrict__ sizes, int stride,
+                                                       int skip_upto, int max_tiles, int tri, int pitch,
+                                                       float* __restrict__ pair_dist)
+{
+    __shared__ BucketKnnLds L;
+    const int bkt = blockIdx.x / tri;
+    const int s = sizes[bkt];
+    if (s < 2 || s <= skip_upto) return;
+    // tile (I, J) of place t in the order (0,0) (0,1) .. (0,T-1) (1,1) ..
+    int t = (int)blockIdx.x - bkt * tri, I = 0;
+    while (t >= max_tiles - I) { t -= max_tiles - I; ++I; }
+    const int J = I + t;
+    if (J * kTile >= s) return;
+    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int tid = threadIdx.x;
+    const int ty = tid >> 4, tx = tid & 15;
+    const bool vec_ok = (D & 3) == 0 && ((reinterpret_cast<uintptr_t>(points) & 15) == 0);
+    const int rows = min(kTile, s - I * kTile), cols = min(kTile, s - J * kTile);
+    const bool diag = I == J;
+    if (tid < kTile) L.ida[tid] = tid < rows ? bid[I * kTile + tid] : -1;
+    else if (tid < 2 * kTile) L.idb[tid - kTile] = tid - kTile < cols ? bid[J * kTile + tid - kTile] : -1;
+    const int nrb = (rows + 15) >> 4, ncb = (cols + 15) >> 4;
+    float acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = 0.0f;
+    __syncthreads();
+    // (off the diagonal tile I is full: J > I; on it rows == cols)
+    if (diag) {
+        switch (nrb) {
+        case 1: pair_tile_chains<1, 1, true>(L, points, D, rows, cols, vec_ok, acc); break;
+        case 2: pair_tile_chains<2, 2, true>(L, points, D, rows, cols, vec_ok, acc); break;
+        case 3: pair_tile_chains<3, 3, true>(L, points, D, rows, cols, vec_ok, acc); break;
+        default: pair_tile_chains<4, 4, true>(L, points, D, rows, cols, vec_ok, acc); break;
+        }
+    } else {
+        switch (ncb) {
+        case 1: pair_tile_chains<4, 1, false>(L, points, D, rows, cols, vec_ok, acc); break;
+        case 2: pair_tile_chains<4, 2, false>(L, points, D, rows, cols, vec_ok, acc); break;
+        case 3: pair_tile_chains<4, 3, false>(L, points, D, rows, cols, vec_ok, acc); break;
+        default: pair_tile_chains<4, 4, false>(L, points, D, rows, cols, vec_ok, acc); break;
+        }
+    }
+    // the tile -> LDS (the blocks below the diagonal of a diagonal tile are the mirror image of those above)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (r >= nrb || c >= ncb || (diag && c < r)) continue;
+            const int i = ty + 16 * r, j = tx + 16 * c;
+            L.dist[i * kDistPitch + j] = acc[r][c];
+            if (diag && c > r) L.dist[j * kDistPitch + i] = acc[r][c];
+        }
+    __syncthreads();
+    // ... -> the bucket's matrix: rows of tile I (a wavefront stores 64 consecutive floats of a row), then, off the
+    // diagonal, the rows of tile J (the columns of the tile in LDS: pitch 65, no bank conflicts)
+    float* M = pair_dist + (size_t)bkt * (size_t)pitch * (size_t)pitch;
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int i = wave; i < rows; i += 4)
+        if (lane < cols) M[(size_t)(I * kTile + i) * pitch + J * kTile + lane] = L.dist[i * kDistPitch + lane];
+    if (!diag)
+        for (int j = wave; j < cols; j += 4)
+            if (lane < rows) M[(size_t)(J * kTile + j) * pitch + I * kTile + lane] = L.dist[lane * kDistPitch + j];
+}
+
+// One wavefront per member of a bucket: the member's row of the bucket's pair matrix (k_bucket_pairs), 64 distances
+// at a time; the K-NN row is read when the first distance at or below its last slot turns up (rows_sorted; else at
+// once), takes the candidates of every such batch, and is written back if it changed.
+template <int SL>
+__global__ __launch_bounds__(256) void k_bucket_merge_pairs(int K, const int* __restrict__ ids, const int* __restrict__ starts,
+                                                             const int* __restrict__ sizes, int stride, int skip_upto,
+                                                             int pitch, const float* __restrict__ pair_dist,
+                                                             int* __restrict__ knn_idx, float* __restrict__ knn_dist,
+                                                             int rows_sorted)
+{
+    const int per = pitch >> 2;                            // workgroups per bucket: four members each
+    const int bkt = blockIdx.x / per;
+    const int lane = threadIdx.x & 63;
+    const int m = (((int)blockIdx.x - bkt * per) << 2) + (threadIdx.x >> 6);
+    const int s = sizes[bkt];
+    if (s < 2 || s <= skip_upto || m >= s) return;         // (a whole wavefront leaves)
+    const int* bid = ids + (starts ? (size_t)starts[bkt] : (size_t)bkt * (size_t)stride);
+    const int p = bid[m];
+    const size_t at = (size_t)p * (size_t)K;
+    const float* drow = pair_dist + ((size_t)bkt * (size_t)pitch + (size_t)m) * (size_t)pitch;
+    const float tau0 = rows_sorted ? knn_dist[at + (K - 1)] : INFINITY;
+    KnnRow<SL> row;
+    bool loaded = false;
+    for (int j0 = 0; j0 < s; j0 += 64) {
+        const int j = j0 + lane;
+        const bool in = j < s && j != m;
+        const float d = in ? drow[j] : INFINITY;
+        const int c = in ? bid[j] : -1;
+        const bool ok = in && d <= tau0;
+        if (ballot64(ok) == 0) continue;
+        if (!loaded) {
+            row.load(knn_idx + at, knn_dist + at, K);         // rows that arrive unsorted are rebuilt here
+            loaded = true;
+        }
+        row.merge(ok, c, d);
+    }
+    if (loaded && row.changed) row.store(knn_idx + at, knn_dist + at);
+}
+
 namespace {
 
+// Is the form that evaluates every pair once wanted?  RSFK_BUCKET_PAIRS=0 / 1 overrides the choice (the results are
+// the same).
+bool pairs_form_wanted()
+{
+    const char* env = std::getenv("RSFK_BUCKET_PAIRS");
+    return !(env && env[0] == '0');
+}
+
+// The buckets of a launch through k_bucket_pairs + k_bucket_merge_pairs, as many at a time as the working memory holds.
+int launch_pairs_form(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
+                      int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted,
+                      int max_tiles, const PairScratch& ps)
+{
+    const int pitch = max_tiles * kTile, tri = max_tiles * (max_tiles + 1) / 2;
+    const size_t per_bucket = (size_t)pitch * (size_t)pitch;
+    // (grids stay below 2^31 workgroups)
+    const size_t most = std::min(ps.floats / per_bucket, (size_t)0x7fffffff / (size_t)std::max(tri, pitch / 4));
+    const int rs = rows_sorted ? 1 : 0;
+    for (int b0 = 0; b0 < n_buckets; b0 += (int)most) {
+        const int nb = (int)std::min<size_t>(most, (size_t)(n_buckets - b0));
+        const int* ids_c = starts ? ids : ids + (size_t)b0 * (size_t)stride;
+        const int* starts_c = starts ? starts + b0 : nullptr;
+        hipLaunchKernelGGL(k_bucket_pairs, dim3((unsigned)nb * (unsigned)tri), dim3(256), 0, stream, points, D, ids_c, starts_c,
+                           sizes + b0, stride, skip_upto, max_tiles, tri, pitch, ps.p);
+        const dim3 grid((unsigned)nb * (unsigned)(pitch / 4)), block(256);
+#define RSFK_PAIRS_CASE(SLV)                                                                                                \
+        hipLaunchKernelGGL(k_bucket_merge_pairs<SLV>, grid, block, 0, stream, K, ids_c, starts_c, sizes + b0, stride, skip_upto, \
+                           pitch, ps.p, knn_idx, knn_dist, rs)
+        if (K <= 64) RSFK_PAIRS_CASE(1);
+        else if (K <= 128) RSFK_PAIRS_CASE(2);
+        else if (K <= 256) RSFK_PAIRS_CASE(4);
+        else if (K <= 512) RSFK_PAIRS_CASE(8);
+        else RSFK_PAIRS_CASE(16);
+#undef RSFK_PAIRS_CASE
+    }
+    RSFK_HIP(hipGetLastError());
+    return 0;
+}
+
+// pairs: working memory for the form that evaluates every pair once (null, or too small for one bucket of the
+// launch: the forms that need none)
 int launch_general(const float* points, int D, int K, const int* ids, const int* starts, const int* sizes, int n_buckets,
                    int stride, int skip_upto, int* knn_idx, float* knn_dist, hipStream_t stream, bool rows_sorted = false,
-                   int max_bucket = -1, int* launched = nullptr)
+                   int max_bucket = -1, int* launched = nullptr, const PairScratch* pairs = nullptr)
 {
     if (n_buckets <= 0) return 0;
     const int rs = rows_sorted ? 1 : 0;
+    if (pairs && pairs->p && max_bucket > 0 && pairs_form_wanted()) {
+        const int mt = (max_bucket + kTile - 1) / kTile;
+        if ((size_t)mt * kTile * (size_t)mt * kTile <= pairs->floats) {
+            if (launched) *launched |= kBucketKernelPairs;
+            return launch_pairs_form(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream,
+                                     rows_sorted, mt, *pairs);
+        }
+    }
     // few buckets (and their largest size known): a workgroup per 64 members instead of one per bucket
     const int max_tiles = max_bucket > 0 ? (max_bucket + kTile - 1) / kTile : 0;
     const char* env = std::getenv("RSFK_BUCKET_STRIP");        // 0 / 1 overrides the choice (the results are the same)
@@ -339,6 +549,23 @@ int bucket_gram_from()
     return 0x7fffffff;
 }
 
+size_t pair_scratch_max()
+{
+    const char* e = std::getenv("RSFK_BUCKET_PAIRS_MB");
+    const long long mb = e && *e ? std::atoll(e) : 512;
+    return (size_t)std::max(1ll, std::min(mb, 16384ll)) << 18;          // floats
+}
+
+size_t bucket_pairs_scratch_floats(int D, int K, int n_buckets, int max_bucket)
+{
+    if (n_buckets <= 0 || max_bucket < 2 || !pairs_form_wanted()) return 0;
+    // (buckets the specialised kernels take never reach the general one)
+    if (K <= 64 && max_bucket <= std::max(medium_bucket_cap(), resident_rows_cap(D, K))) return 0;
+    const size_t pitch = (size_t)((max_bucket + kTile - 1) / kTile) * kTile;
+    if (pitch * pitch > pair_scratch_max()) return 0;
+    return std::min(pair_scratch_max(), (size_t)n_buckets * pitch * pitch);
+}
+
 // Host launcher for an arbitrary list of buckets.  All pointers are device pointers.  max_bucket: size of
 // the largest bucket if known, otherwise -1.
 int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, const int* starts,
@@ -378,8 +605,26 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
             skip_upto = rows_cap;
         }
     }
-    return launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream, false,
-                          max_bucket);
+    // the rest: every pair once, with working memory for the pair matrices, when there is room for it
+    PairScratch ps;
+    if (pairs_form_wanted()) {
+        if (max_bucket < 0 && largest_bucket(sizes, n_buckets, stream, &max_bucket)) return 1;
+        const size_t want = bucket_pairs_scratch_floats(D, K, n_buckets, max_bucket);
+        void* mem = nullptr;
+        if (want > 0 && ws_try_alloc(&mem, want * sizeof(float)) == 0) {
+            ps.p = static_cast<float*>(mem);
+            ps.floats = want;
+        }
+    }
+    const int rc = launch_general(points, D, K, ids, starts, sizes, n_buckets, stride, skip_upto, knn_idx, knn_dist, stream, false,
+                                  max_bucket, nullptr, &ps);
+    if (ps.p) {
+        // (the block goes back to the pool only when nothing uses it any more)
+        const hipError_t e = hipStreamSynchronize(stream);
+        ws_free(ps.p);
+        if (rc == 0 && e != hipSuccess) { set_last_error(std::string("bucket K-NN: ") + hipGetErrorString(e)); return 1; }
+    }
+    return rc;
 }
 
 // Host launcher for the leaf table of one tree: n_small buckets of at most kBucketSplit points at the front of
@@ -388,11 +633,12 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
 // kernel that chooses between the direct and the screened form from the pairs of the tree before (prev_stats, null for
 // the first tree) and leaves its own numbers in stats.  part: 0 = all buckets, 1 = only the small ones, 2 = only the larger ones (the two
 // kinds touch different rows, so the two parts of one tree may run side by side).  young_rows: the rows may be new or
-// far from done (first trees of a build).
+// far from done (first trees of a build).  pairs: working memory for the buckets that reach the general kernel (null:
+// its forms that need none); launches that may run side by side need one each.
 int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_stats, unsigned long long* stats,
                            bool rows_sorted, bool gram, int D, int K, const int* ids, const int* starts, const int* sizes,
                            int leaf_cap, int n_small, int n_big, int max_bucket, int* knn_idx, float* knn_dist,
-                           hipStream_t stream, int part, bool young_rows, int* launched)
+                           hipStream_t stream, int part, bool young_rows, int* launched, const PairScratch* pairs)
 {
     RSFK_CHECK(K >= 1 && K <= kMaxK, "bucket K-NN: K must be in 1..1024");
     RSFK_CHECK(D >= 1, "bucket K-NN: D must be positive");
@@ -427,7 +673,7 @@ int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_s
             used |= kBucketKernelSmall;
             if (launch_bucket_knn_small(points, D, K, ids, starts, sizes, n_small, 0, rows_sorted, knn_idx, knn_dist, stream)) return 1;
         } else if (launch_general(points, D, K, ids, starts, sizes, n_small, 0, 0, knn_idx, knn_dist, stream, rows_sorted,
-                                  kBucketSplit, &used)) {
+                                  kBucketSplit, &used, pairs)) {
             return 1;
         }
     }
@@ -453,7 +699,7 @@ int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_s
         }
     }
     return launch_general(points, D, K, ids, starts + off, sizes + off, n_big, 0, skip_upto, knn_idx, knn_dist, stream,
-                          rows_sorted, max_bucket, &used);
+                          rows_sorted, max_bucket, &used, pairs);
 }
 
 }  // namespace rsfk

@@ -153,7 +153,8 @@ int build_report_json(char* buf, int cap)
         {kBucketKernelSmall, "k_bucket_knn_small<64>"}, {kBucketKernelScreen, "k_bucket_knn_screen"},
         {kBucketKernelMedium, "k_bucket_knn_small<72>"}, {kBucketKernelRows, "k_bucket_knn_rows"},
         {kBucketKernelTiled, "k_bucket_knn<per bucket>"}, {kBucketKernelStrip, "k_bucket_knn<per 64 members>"},
-        {kBucketKernelGram, "k_bucket_knn_gram"}, {kBucketKernelAuto, "k_bucket_knn_auto"}};
+        {kBucketKernelGram, "k_bucket_knn_gram"}, {kBucketKernelAuto, "k_bucket_knn_auto"},
+        {kBucketKernelPairs, "k_bucket_pairs + k_bucket_merge_pairs"}};
     std::string s = "{";
     auto num = [&](const char* key, double v, bool last = false) {
         char t[96];
@@ -267,6 +268,23 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
         constexpr int kYoungTrees = 2;          // trees of a build whose bucket step still finds rows that are far from done
         SideStream sync;
         if (std::getenv("RSFK_KNN_ONE_STREAM") == nullptr && sync.open()) return 1;
+        // working memory of the bucket kernels that pass the distances of a bucket's pairs through memory (only
+        // buckets the specialised kernels do not take): one block per stream, grown when a tree asks for more
+        DevBuf pair_buf[2];
+        PairScratch pair_mem[2];
+        auto pair_room = [&](int which, size_t want) -> int {
+            if (want <= pair_mem[which].floats) return 0;
+            RSFK_HIP(hipStreamSynchronize(stream));
+            if (sync.side) RSFK_HIP(hipStreamSynchronize(sync.side));
+            if (pair_buf[which].p) { ws_free(pair_buf[which].p); pair_buf[which].p = nullptr; }
+            pair_mem[which] = PairScratch();
+            want = std::min(pair_scratch_max(), want + want / 4);
+            if (ws_try_alloc(&pair_buf[which].p, want * sizeof(float)) == 0) {
+                pair_mem[which].p = static_cast<float*>(pair_buf[which].p);
+                pair_mem[which].floats = want;
+            }
+            return 0;
+        };
         int rc = 0;
         for (int t0 = 0; t0 < n_trees && rc == 0; t0 += B) {
             const int nb = std::min(B, n_trees - t0);
@@ -289,15 +307,22 @@ int knn_forest_device(int n_trees, int K, int N, int D, int MIN, int MAX, int MA
                 if (split) (void)hipStreamWaitEvent(sync.side, ev[j].e, 0);      // everything before this tree
                 const bool gram = t0 + j >= gram_from;
                 const int t = t0 + j;
+                {
+                    const size_t want_small = K > 64 ? bucket_pairs_scratch_floats(D, K, n_small, kBucketSplit) : 0;
+                    const size_t want_big = bucket_pairs_scratch_floats(D, K, n_big, stats[5 * j + 2]);
+                    if (pair_room(0, split ? want_small : std::max(want_small, want_big))) return 1;
+                    if (split && pair_room(1, want_big)) return 1;
+                }
                 rc = launch_bucket_knn_tree(d_points, t > 0 ? d_pairs + (size_t)8 * (t - 1) : nullptr, d_pairs + (size_t)8 * t, true,
                                             gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                             tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big, stats[5 * j + 2],
-                                            d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees, &rep.kernels[(size_t)(t0 + j)]);
+                                            d_idx, d_dist, stream, split ? 1 : 0, t0 + j < kYoungTrees, &rep.kernels[(size_t)(t0 + j)],
+                                            &pair_mem[0]);
                 if (!rc && split) {
                     rc = launch_bucket_knn_tree(d_points, nullptr, nullptr, true, gram, D, K, tree_ws_perm(ws.w, j), tree_ws_leaf_start(ws.w, j),
                                                 tree_ws_leaf_size(ws.w, j), tree_ws_leaf_cap(ws.w), n_small, n_big,
                                                 stats[5 * j + 2], d_idx, d_dist, sync.side, 2, t0 + j < kYoungTrees,
-                                                &rep.kernels[(size_t)(t0 + j)]);
+                                                &rep.kernels[(size_t)(t0 + j)], &pair_mem[1]);
                     (void)hipEventRecord(sync.big, sync.side);
                 }
                 big_pending = split;

@@ -48,11 +48,24 @@ enum : int {
     kBucketKernelTiled = 16,     // k_bucket_knn<SL, false>: 64 x 64 tiles, a workgroup per bucket
     kBucketKernelStrip = 32,     // k_bucket_knn<SL, true>: 64 x 64 tiles, a workgroup per 64 members of a bucket
     kBucketKernelGram = 64,      // k_bucket_knn_gram: any bucket size, pair matrix bounded on the matrix cores
+    kBucketKernelPairs = 256,    // k_bucket_pairs + k_bucket_merge_pairs: 64 x 64 tiles, every pair once, distances through memory
 };
+// Working memory of k_bucket_pairs / k_bucket_merge_pairs: the pair matrices of as many buckets as fit are in it at a
+// time.  One per stream of launches; p == null: the forms of the general kernel that need none are taken.
+struct PairScratch {
+    float* p = nullptr;
+    size_t floats = 0;
+};
+// Floats of working memory the buckets of a launch would like (0: none of them reaches the general kernel, or the
+// form is switched off); at most pair_scratch_max() (512 MB; RSFK_BUCKET_PAIRS_MB overrides), the launch then goes in
+// several parts.
+size_t pair_scratch_max();
+size_t bucket_pairs_scratch_floats(int D, int K, int n_buckets, int max_bucket);
 int launch_bucket_knn_tree(const float* points, const unsigned long long* prev_stats, unsigned long long* stats,
                            bool rows_sorted, bool gram, int D, int K, const int* ids, const int* starts, const int* sizes,
                            int leaf_cap, int n_small, int n_big, int max_bucket, int* knn_idx, float* knn_dist,
-                           hipStream_t stream, int part = 0, bool young_rows = true, int* launched = nullptr);
+                           hipStream_t stream, int part = 0, bool young_rows = true, int* launched = nullptr,
+                           const PairScratch* pairs = nullptr);
 
 // What the last K-NN-graph build of this process did, as a line of JSON (rsfk_last_build_report): which bucket
 // kernels every tree went to, the counts the algorithmic bytes of the tree build and of the exploration are made of,

@@ -92,19 +92,26 @@ def test_tree_edge_cases(gpu, orc, rng):
     (1800, 12, 200, 201, 420), (4000, 256, 32, 33, 66), (1500, 784, 90, 91, 182), (2000, 30, 32, 400, 1024),
     (2500, 10, 300, 301, 620), (4200, 6, 700, 701, 1500), (1600, 40, 1024, 400, 900),
 ])
-@pytest.mark.parametrize("kernel", ["direct", "direct_per_bucket", "gram", "screen"])
+@pytest.mark.parametrize("kernel", ["direct", "direct_per_bucket", "direct_per_64", "pairs_in_parts", "gram", "screen"])
 def test_bucket_knn_matches_oracle(gpu, orc, rng, monkeypatch, N, D, K, MIN, MAX, kernel):
-    """kernel: "direct" = fp32 chains for every pair; "gram" = the kernel that bounds the pair matrix on the matrix
-    cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0); "screen" = the same
-    idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=always; other buckets, and K > 64,
-    take the direct kernels); "direct_per_bucket" = the tiled direct kernel with a workgroup per bucket, as launches
-    over many buckets run it (RSFK_BUCKET_STRIP=0; with the few buckets of a test it otherwise takes a workgroup per 64
-    members), and without the kernel that keeps a bucket's points in LDS (RSFK_BUCKET_ROWS=0)."""
-    if kernel == "direct_per_bucket":
+    """kernel: "direct" = fp32 chains for every pair, the buckets the specialised kernels leave through the pair of
+    kernels that evaluates every pair once and hands the distances on through memory; "pairs_in_parts" = the same with
+    1 MB of that memory, so that a launch goes in many parts (RSFK_BUCKET_PAIRS_MB=1), and without the kernel that keeps
+    a bucket's points in LDS (RSFK_BUCKET_ROWS=0); "direct_per_bucket" / "direct_per_64" = the tiled kernels that need
+    no working memory (RSFK_BUCKET_PAIRS=0), a workgroup per bucket or per 64 members of a bucket
+    (RSFK_BUCKET_STRIP=0 / 1), also without the kernel for resident buckets; "gram" = the kernel that bounds the pair
+    matrix on the matrix cores first and runs the chains only for the pairs that may enter a row (RSFK_GRAM_FROM=0);
+    "screen" = the same idea in the two-wavefront kernel for buckets of up to 64 points (RSFK_BUCKET_SCREEN=always;
+    other buckets, and K > 64, take the direct kernels)."""
+    if kernel in ("direct_per_bucket", "direct_per_64", "pairs_in_parts"):
         if MAX <= 72 and K <= 64:
-            pytest.skip("no bucket of this shape reaches the tiled kernel")
-        monkeypatch.setenv("RSFK_BUCKET_STRIP", "0")
+            pytest.skip("no bucket of this shape reaches the tiled kernels")
         monkeypatch.setenv("RSFK_BUCKET_ROWS", "0")
+        if kernel == "pairs_in_parts":
+            monkeypatch.setenv("RSFK_BUCKET_PAIRS_MB", "1")
+        else:
+            monkeypatch.setenv("RSFK_BUCKET_PAIRS", "0")
+            monkeypatch.setenv("RSFK_BUCKET_STRIP", "0" if kernel == "direct_per_bucket" else "1")
     if kernel == "gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "0")
     if kernel == "screen":
@@ -339,9 +346,13 @@ def test_find_nearest_neighbors_matches_oracle(gpu, orc, rng, monkeypatch, N, D,
     ("c4", 9000, 90, 4, dict(nn_exploring_factor=1)),
     ("c5", 70000, 32, 5, dict(min_tree_children=64, max_tree_children=256)),
 ], ids=["config3_gmm64_d256_k32", "config4_sparse_d784_k90_explore", "config5_normal_d32_buckets64_256"])
-@pytest.mark.parametrize("kernel", ["direct", "gram", "screen"])
+@pytest.mark.parametrize("kernel", ["direct", "gram", "screen", "tiled"])
 def test_baseline_config_workloads_match_oracle(gpu, orc, monkeypatch, config, N, K, T, kw, kernel):
     import gpu_rsfk
+    if kernel == "tiled":
+        if config != "c4":
+            pytest.skip("no bucket of this configuration reaches the general kernel")
+        monkeypatch.setenv("RSFK_BUCKET_PAIRS", "0")       # the forms of the general kernel that need no working memory
     if kernel == "gram":
         monkeypatch.setenv("RSFK_GRAM_FROM", "1")          # every tree but the first through the screened bucket kernel
     if kernel == "screen":
