@@ -295,7 +295,7 @@ def profiled_traffic(config, steps_profiled=2):
     launches, kib = {}, {}
     for line in text.splitlines():
         cells = [c.strip() for c in line.strip().strip("|").split("|")]
-        if len(cells) == 7 and cells[0].startswith("k_bucket_knn"):
+        if len(cells) == 7 and cells[0].startswith("k_bucket_"):
             try:
                 if "." in cells[2]:                       # trace table: launches, total ms, ...
                     launches[cells[0]] = int(cells[1])
