@@ -43,8 +43,9 @@ __device__ __forceinline__ float4 load_piece(const float* __restrict__ row, int 
 // knows for the row's final last slot (candidates above it need not be finished), else +inf.  DEEP: the loads of
 // two steps are in flight while a third is being used (two register buffers that take turns, so that waiting for
 // one does not wait for the other): for kernels with few wavefronts per SIMD, whose gathers would otherwise wait
-// for each other.
-template <int SL, int CH = kChunk, bool DEEP = false>
+// for each other.  GROUP: 16-byte pieces of a row whose reads from the tile are requested together (0: one at a time, the
+// form that needs the fewest registers).
+template <int SL, int CH = kChunk, bool DEEP = false, int GROUP = 0>
 __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list, int n,
                                             const float* __restrict__ points, int D, bool vec_ok, KnnRow<SL>& row,
                                             float tau_cap = INFINITY)
@@ -85,14 +86,32 @@ __device__ __forceinline__ void exact_batch(const ExploreLds& L, const int* list
         const int pieces = min(kPieces, (D - d0 + 3) >> 2);
         const float* mine = &L.tile[lane * kP];
         const float* xs = &L.xrow[d0];
-        for (int q = 0; q < pieces; ++q) {
-            const float4 a = *reinterpret_cast<const float4*>(mine + 4 * q);
-            const float4 x = *reinterpret_cast<const float4*>(xs + 4 * q);
+        auto chain4 = [&](const float4& a, const float4& x) {
             float df;
             df = a.x - x.x; acc = __builtin_fmaf(df, df, acc);
             df = a.y - x.y; acc = __builtin_fmaf(df, df, acc);
             df = a.z - x.z; acc = __builtin_fmaf(df, df, acc);
             df = a.w - x.w; acc = __builtin_fmaf(df, df, acc);
+        };
+        if (GROUP > 0 && pieces == kPieces) {
+            // a whole step: the reads of the tile and of the point for 4 GROUP dimensions are requested together, so
+            // that the chain waits for LDS once per group and not once per four dimensions (8 GROUP registers)
+            constexpr int kGroup = GROUP > 0 ? GROUP : 1;
+            static_assert(kPieces % kGroup == 0, "a step is a whole number of groups");
+#pragma unroll
+            for (int q0 = 0; q0 < kPieces; q0 += kGroup) {
+                float4 a[kGroup], x[kGroup];
+#pragma unroll
+                for (int q = 0; q < kGroup; ++q) {
+                    a[q] = *reinterpret_cast<const float4*>(mine + 4 * (q0 + q));
+                    x[q] = *reinterpret_cast<const float4*>(xs + 4 * (q0 + q));
+                }
+#pragma unroll
+                for (int q = 0; q < kGroup; ++q) chain4(a[q], x[q]);
+            }
+        } else {
+            for (int q = 0; q < pieces; ++q)
+                chain4(*reinterpret_cast<const float4*>(mine + 4 * q), *reinterpret_cast<const float4*>(xs + 4 * q));
         }
         // partial sums only grow: once all of them are above the row maximum nothing can enter
         return ballot64(lane < n && acc <= tau0) != 0;

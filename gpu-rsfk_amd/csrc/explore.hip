@@ -343,6 +343,10 @@ __device__ __forceinline__ int graph_entry(const int* __restrict__ old_idx, int 
 }
 
 constexpr int kMergeChunk = 16;
+// 16-byte pieces of a candidate's row a lane requests from the tile together (exact_batch): 16 dimensions per wait for
+// LDS.  (Measured: 1M x 256 pass 26.2 -> 24.8 ms, 70k x 784 pass 26.2 -> 25.0 ms; eight pieces cost the workgroup
+// kernel its second wavefront per SIMD: 39 ms.)
+constexpr int kChainGroup = 4;
 constexpr int kMergeTile = 64 * (kMergeChunk + 4);
 // Rows of at most this many (padded) dimensions are read by the lane that runs their chain, 32 dimensions at a time,
 // without the transposing tile in LDS (exact_direct): the LDS of a wavefront shrinks by the tile.
@@ -358,7 +362,9 @@ int merge_direct_max()
 }
 
 
-template <int SL, int WAVES>
+// TILE: the candidates' rows go through the transposing tile (rows longer than direct_max dimensions); the two forms
+// are kernels of their own, so that the shorter one does not carry the registers of the other.
+template <int SL, int WAVES, bool TILE>
 __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __restrict__ points, int N, int D, int K,
                                                                const int* __restrict__ old_idx, int* __restrict__ knn_idx,
                                                                float* __restrict__ knn_dist, int table_size,
@@ -520,8 +526,8 @@ __global__ __launch_bounds__(64 * WAVES) void k_explore_merge(const float* __res
     int n_exact = 0;                                      // exact distances of this point (wave-uniform)
     auto batch = [&](const int* list, int n) {
         n_exact += n;
-        if (tile_ints == 0) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
-        else exact_batch<SL, kMergeChunk, true>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
+        if (!TILE) exact_direct<SL>(L, list, n, points, D, vec_ok, row);
+        else exact_batch<SL, kMergeChunk, true, kChainGroup>(L, list, n, points, D, vec_ok, row);    // two steps of gathers in flight
     };
     if (tbound == nullptr || U <= 64) {
         for (int off = 0; off < U; off += 64) {
@@ -754,7 +760,7 @@ __global__ __launch_bounds__(256) void k_explore_merge_wg(const float* __restric
         const int n_now = min(64, have);
         n_exact += n_now;
         const float cap_now = __uint_as_float(*reinterpret_cast<volatile uint32_t*>(&tau_s));
-        exact_batch<SL, kWgChunk, true>(L, ids, n_now, points, D, vec_ok, row, cap_now);
+        exact_batch<SL, kWgChunk, true, kChainGroup>(L, ids, n_now, points, D, vec_ok, row, cap_now);
         if (lane == 0) atomicMin(&tau_s, __float_as_uint(row.tau));   // non-negative floats order like their bits
         have -= n_now;
         const int left = lane < have ? ids[64 + lane] : 0;        // the candidates beyond the batch move to the front
@@ -972,13 +978,21 @@ int launch_merge(const float* points, int N, int D, int K, const int* old_idx, i
                  int* todo_out, int* n_out, unsigned long long* stat, const int* order, hipStream_t stream)
 {
     const size_t lds = (size_t)WAVES * (size_t)wave_ints * sizeof(int);
-    RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES>),
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     const int n_work = todo_in ? n_in : N;
     dim3 grid(grid_for_dies(((size_t)n_work + WAVES - 1) / WAVES)), block(64 * WAVES);
-    hipLaunchKernelGGL((k_explore_merge<SL, WAVES>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
-                       knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out, stat,
-                       order);
+    if (merge_tile_ints(dpad, merge_direct_max()) == 0) {
+        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES, false>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL((k_explore_merge<SL, WAVES, false>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
+                           knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out,
+                           stat, order);
+    } else {
+        RSFK_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(k_explore_merge<SL, WAVES, true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL((k_explore_merge<SL, WAVES, true>), grid, block, lds, stream, points, N, D, K, old_idx, knn_idx,
+                           knn_dist, table, wave_ints, dpad, merge_direct_max(), pass, bounds, todo_in, n_in, todo_out, n_out,
+                           stat, order);
+    }
     RSFK_HIP(hipGetLastError());
     return 0;
 }
