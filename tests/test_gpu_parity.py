@@ -243,6 +243,32 @@ def test_bucket_knn_padded_matrix_ragged_and_empty(gpu, orc, rng):
                        starts=np.array([0], np.int32))
 
 
+@pytest.mark.parametrize("memory_mb", [None, "1"])
+def test_bucket_knn_padded_matrix_of_large_buckets(gpu, orc, rng, monkeypatch, memory_mb):
+    """Buckets handed over as rows of a padded matrix (no table of starts) that reach the pair of kernels which passes
+    a bucket's distances through working memory: all at once, and in parts of a few buckets (1 MB of that memory)."""
+    if memory_mb:
+        monkeypatch.setenv("RSFK_BUCKET_PAIRS_MB", memory_mb)
+    N, D, K = 2600, 12, 70
+    X = rng.random((N, D), dtype=np.float32)
+    perm, ls, lz, _ = orc.build_tree(X, 71, 150, 5000, 8)
+    mc = int(lz.max())
+    nb = len(lz) + 1
+    padded = np.full((nb, mc), -1, np.int32)
+    sizes = np.zeros(nb, np.int32)                      # the bucket in the middle of the matrix is empty
+    for b, (s, z) in enumerate(zip(ls, lz)):
+        row = b if b < nb // 2 else b + 1
+        padded[row, :z] = perm[s:s + z]
+        sizes[row] = z
+    oi, od = orc.init_lists(N, K)
+    gi, gd = orc.init_lists(N, K)
+    for _ in range(2):                                  # the second call finds rows that are full
+        orc.bucket_knn(X, K, padded.ravel(), sizes, oi, od, starts=None, stride=mc)
+        _say("bucket_knn padded, large buckets", memory_mb)
+        gpu.bucket_knn(X, K, padded.ravel(), sizes, gi, gd, starts=None, stride=mc)
+        assert_knn_equal(gi, gd, oi, od)
+
+
 # ---------------------------------------------------------------------------
 # exploration
 # ---------------------------------------------------------------------------
