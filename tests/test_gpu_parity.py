@@ -609,6 +609,42 @@ def test_screens_never_change_a_result(gpu, orc, rng, monkeypatch, kind, variant
     assert rows_have_no_duplicates(gi)
 
 
+@pytest.mark.parametrize("K,mn,mx,env,expected", [
+    (16, 17, 34, {}, ["k_bucket_knn_auto"]),
+    (16, 17, 34, {"RSFK_BUCKET_SCREEN": "never"}, ["k_bucket_knn_auto"]),
+    (16, 17, 34, {"RSFK_BUCKET_SCREEN": "always"}, ["k_bucket_knn_auto"]),
+    (16, 40, 100, {}, ["k_bucket_knn_auto", "k_bucket_knn_small<72>", "k_bucket_knn_rows"]),
+    (90, 91, 182, {}, ["k_bucket_pairs + k_bucket_merge_pairs"]),
+    (90, 91, 182, {"RSFK_BUCKET_PAIRS": "0"}, ["k_bucket_knn<per 64 members>"]),
+    (90, 91, 182, {"RSFK_BUCKET_PAIRS": "0", "RSFK_BUCKET_STRIP": "0"}, ["k_bucket_knn<per bucket>"]),
+    (90, 91, 182, {"RSFK_GRAM_FROM": "1"}, ["k_bucket_pairs + k_bucket_merge_pairs", "k_bucket_knn_gram"]),
+])
+def test_report_of_a_build_names_what_ran(gpu, rng, monkeypatch, K, mn, mx, env, expected):
+    """rsfk_last_build_report: the kernels every tree's buckets went to, the counts the algorithmic bytes are made of
+    and the seconds of the three steps, for the build that has just run."""
+    import gpu_rsfk
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    N, D, T = 6000, 20, 3
+    X = rng.random((N, D), dtype=np.float32)
+    r = gpu_rsfk.RSFK(random_state=4)
+    _say("report of a build", K, mn, mx, env)
+    r.find_nearest_neighbors(X, K, n_trees=T, min_tree_children=mn, max_tree_children=mx, nn_exploring_factor=1)
+    rep = gpu.last_build_report()
+    assert (rep["N"], rep["D"], rep["K"], rep["n_trees"]) == (N, D, K, T)
+    runs = rep["bucket_kernels"]
+    assert runs[0][0] == 0 and runs[-1][1] == T - 1
+    assert all(runs[i][1] + 1 == runs[i + 1][0] for i in range(len(runs) - 1))
+    named = set(name for _, _, names in runs for name in names)
+    assert named == set(expected), named
+    assert len(rep["bucket_pair_share"]) == T and len(rep["bucket_screened"]) == T
+    if "RSFK_BUCKET_SCREEN" in env:                     # the form of the kernel the trees took
+        assert rep["bucket_screened"] == [1 if env["RSFK_BUCKET_SCREEN"] == "always" else 0] * T
+    assert rep["tree_points_tested"] >= N * T and 0 <= rep["tree_points_undecided"] <= rep["tree_points_tested"]
+    assert rep["explore_passes"] == 1 and rep["explore_exact_distances"] > 0
+    assert rep["tree_seconds"] > 0 and rep["bucket_seconds"] > 0 and rep["explore_seconds"] > 0
+
+
 def test_workspace_is_reused_and_can_be_released(gpu, rng):
     """Device buffers are kept between calls; releasing them changes nothing but the next call's allocations."""
     import gpu_rsfk
