@@ -18,7 +18,7 @@ int tree_ws_leaf_cap(const TreeBatchWorkspace* w);
 const int* tree_ws_perm(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_start(const TreeBatchWorkspace* w, int t);
 const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t);
-int tree_small_threshold(int D);
+int tree_small_threshold(int D, int N, int B);
 const float* tree_ws_phase_seconds(const TreeBatchWorkspace* w);
 const unsigned long long* tree_ws_counts(const TreeBatchWorkspace* w);
 int tree_screen_row_bytes(int D, bool q8);

@@ -1059,11 +1059,14 @@ const int* tree_ws_leaf_size(const TreeBatchWorkspace* w, int t) { return w->lea
 
 // Nodes of at most this many points are finished by one workgroup (k_tail): 1024, or 2048 for short rows, where a
 // wide level costs more per byte of row it reads (the permutation entries it moves weigh more) -- measured on 10M x 32
-// points 4.46 against 4.81 ms per tree, on 1M x 100 points 0.548 against 0.520.  RSFK_TREE_SMALL overrides (tests).
-int tree_small_threshold(int D)
+// points 4.46 against 4.81 ms per tree, on 1M x 100 points 0.548 against 0.520 -- and for batches so small (N x B below
+// 2^21 points) that the subtrees do not fill the device anyway: a wide level then costs its launches and little else
+// (70,000 x 784, 10 trees: 0.964 against 0.996 ms per tree).  RSFK_TREE_SMALL overrides (tests).
+int tree_small_threshold(int D, int N, int B)
 {
     const char* e = std::getenv("RSFK_TREE_SMALL");
-    const int v = e && *e ? std::atoi(e) : (D <= 48 ? 2048 : 1024);
+    const bool few = (size_t)N * (size_t)std::max(B, 1) < ((size_t)1 << 21);
+    const int v = e && *e ? std::atoi(e) : (D <= 48 || few ? 2048 : 1024);
     return std::min(2048, std::max(64, v));
 }
 constexpr int kWideChunk = 1024;         // points per workgroup in the wide passes (k_side keeps a chunk's undecided points in LDS)
@@ -1097,7 +1100,7 @@ int tree_ws_alloc(TreeBatchWorkspace** out, int N, int D, int MIN, int B)
     TreeBatchWorkspace* w = new TreeBatchWorkspace();
     *out = w;
     w->B = B; w->N = N; w->D = D;
-    const int small = tree_small_threshold(D);
+    const int small = tree_small_threshold(D, N, B);
     w->leaf_cap = N / std::max(MIN, 1) + 2;
     w->node_cap = B * (N / small + 2);
     w->tail_cap = B * w->leaf_cap;
@@ -1157,7 +1160,7 @@ int build_tree_batch(TreeBatchWorkspace* w, const float* points, const uint16_t*
     RSFK_CHECK(N >= 1 && D >= 1, "tree batch: N and D must be positive");
     TreeParams P;
     P.N = N; P.D = D; P.MIN = MIN; P.MAX = MAX; P.MAX_DEPTH = MAX_DEPTH;
-    P.small = tree_small_threshold(D);
+    P.small = tree_small_threshold(D, N, w->B);
     P.chunk = kWideChunk;
     // bfloat16 rounding 2^-8 (1 + 2^-7), plus the summation errors of the screen (D/8 terms per lane and a 3-step
     // tree) and of the exact test (D/32 terms per lane and a 5-step tree), 1 % on top
