@@ -341,6 +341,7 @@ def test_find_nearest_neighbors_small_plumbing_config(gpu, orc):
     (5000, 16, 8, 3, dict(min_tree_children=4, max_tree_children=9)),          # second call with K+1 .. 3(K+1)
     (6000, 24, 40, 3, dict(nn_exploring_factor=2)),
     (4000, 12, 10, 2, dict(point_in_self_neigh=False, nn_exploring_factor=0)),
+    (9000, 12, 64, 6, dict(nn_exploring_factor=2)),     # rows of 64: the small set of the merge is tried on a sample first
     (4000, 10, 300, 2, dict(nn_exploring_factor=1)),                           # eight slots per lane
     (1400, 8, 520, 2, dict(nn_exploring_factor=1, min_tree_children=200, max_tree_children=500)),   # sixteen
 ])
