@@ -601,12 +601,32 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
     const int k = c - first;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
+    const size_t toff = (size_t)nd.tree * (size_t)P.N;
+    const int* src = (nd.buf ? perm1 : perm0) + toff;
+    int* dst = (nd.buf ? perm0 : perm1) + toff;
+    const int pos0 = nd.start + k * P.chunk;
+    const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
+    // rounds of four entries per thread (entry u of a thread at r0 + u kBlock + tid: loads and stores stay coalesced,
+    // four loads in flight, one exchange of the wavefronts' counts per round); the entries of the first round (the
+    // only one with chunks of 1024) are requested before the counts of the node's chunks are added up, so that the
+    // two trips to memory go side by side
+    constexpr int kPer = 4;
+    int v[kPer];
+    auto request = [&](int r0) {
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const int pos = r0 + u * kBlock + tid;
+            v[u] = pos < pos1 ? src[pos] : -1;            // (beyond the chunk: counts as a right one, is not stored)
+        }
+    };
+    request(pos0);
+
     // lefts in the chunks before this one, and in the whole node
     int before = 0, all = 0;
     for (int j = tid; j < nch; j += kBlock) {
-        const int v = chunk_left[first + j];
-        all += v;
-        if (j < k) before += v;
+        const int x = chunk_left[first + j];
+        all += x;
+        if (j < k) before += x;
     }
     before = wave_sum_i(before);
     all = wave_sum_i(all);
@@ -616,24 +636,11 @@ __global__ __launch_bounds__(kBlock) void k_scatter(TreeParams P, int* __restric
 #pragma unroll
     for (int w = 0; w < kBlock / 64; ++w) { before += red[0][w]; all += red[1][w]; }
 
-    const size_t toff = (size_t)nd.tree * (size_t)P.N;
-    const int* src = (nd.buf ? perm1 : perm0) + toff;
-    int* dst = (nd.buf ? perm0 : perm1) + toff;
-    const int pos0 = nd.start + k * P.chunk;
-    const int pos1 = min(nd.start + nd.count, pos0 + P.chunk);
     int lbase = before;                                   // lefts of the node before the current round
-    // rounds of four entries per thread (entry u of a thread at r0 + u kBlock + tid: loads and stores stay coalesced,
-    // four loads in flight, one exchange of the wavefronts' counts per round)
-    constexpr int kPer = 4;
     __shared__ int wcnt4[kPer][kBlock / 64];
     for (int r0 = pos0; r0 < pos1; r0 += kPer * kBlock) {
-        int v[kPer];
+        if (r0 > pos0) request(r0);
         uint64_t m[kPer];
-#pragma unroll
-        for (int u = 0; u < kPer; ++u) {
-            const int pos = r0 + u * kBlock + tid;
-            v[u] = pos < pos1 ? src[pos] : -1;            // (beyond the chunk: counts as a right one, is not stored)
-        }
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
             m[u] = ballot64(v[u] >= 0);
