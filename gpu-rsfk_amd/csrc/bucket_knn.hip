@@ -609,6 +609,7 @@ int launch_bucket_knn(const float* points, int N, int D, int K, const int* ids, 
     PairScratch ps;
     if (pairs_form_wanted()) {
         if (max_bucket < 0 && largest_bucket(sizes, n_buckets, stream, &max_bucket)) return 1;
+        if (max_bucket <= skip_upto) return 0;            // (the kernels above have taken every bucket)
         const size_t want = bucket_pairs_scratch_floats(D, K, n_buckets, max_bucket);
         void* mem = nullptr;
         if (want > 0 && ws_try_alloc(&mem, want * sizeof(float)) == 0) {
